@@ -1,0 +1,15 @@
+"""entropack_amd: the lossy decode-and-matmul path of EntroPack, built for AMD Instinct MI355X (gfx950).
+
+Drop-in names: `compress`, `decompress`, `CompressedTensor`, `EntroPackLossyConfig`, `CompressedLinear`,
+`CompressedINT8Linear`. Decoding runs on the `hip` backend only.
+"""
+from .compression import CompressedTensor, CompressionFallbackWarning, compress, decompress
+from .registry import DispatchError
+from .schemes import CompressionConfig, EntroPackLossyConfig, LatticeRANSConfig, RawConfig
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "CompressedTensor", "CompressionConfig", "CompressionFallbackWarning", "DispatchError", "EntroPackLossyConfig",
+    "LatticeRANSConfig", "RawConfig", "__version__", "compress", "decompress",
+]

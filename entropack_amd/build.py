@@ -1,0 +1,45 @@
+"""Builds the native libraries of this package in-tree with hipcc (gfx950 only).
+
+    python -m entropack_amd.build          # compile everything
+"""
+import os
+import subprocess
+import sys
+
+PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PACKAGE_DIR, "csrc")
+INCLUDE = os.path.join(os.path.dirname(PACKAGE_DIR), "include")
+HIP_LIBRARY = os.path.join(PACKAGE_DIR, "libentropack_hip.so")
+HIP_SOURCES = ("ep_plan.hip", "ep_decode.hip")
+
+HIPCC_FLAGS = (
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    # Packed FP32 VALU forms are kept out of every kernel of this library.
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+)
+
+
+def hipcc() -> str:
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def build_hip(verbose: bool = False, extra_flags=()) -> str:
+    sources = [os.path.join(CSRC, name) for name in HIP_SOURCES]
+    command = [hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, "-I", CSRC, "-o", HIP_LIBRARY, *sources]
+    if verbose:
+        print(" ".join(command), flush=True)
+    done = subprocess.run(command, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({done.returncode}):\n{done.stdout}\n{done.stderr}")
+    if verbose and done.stderr.strip():
+        print(done.stderr, file=sys.stderr)
+    return HIP_LIBRARY
+
+
+def build_all(verbose: bool = False) -> None:
+    build_hip(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)

@@ -1,0 +1,54 @@
+// Shared declarations of libentropack_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "entropack_hip.h"
+
+namespace ep {
+
+constexpr int kStreams = 17;          // 1 coset stream + 8 fields x 2 cosets
+constexpr int kFieldStreams = 16;
+constexpr int kFields = 8;
+constexpr int kStatesPerTile = 32;    // interleaved rANS lanes per tile, fixed by the bitstream
+constexpr uint32_t kStateMin = 1u << 15;
+constexpr int kMetaWidth = 4;         // (n_symbols, sym_min, freq_offset, alphabet)
+
+// Plan buffer: a 256-byte header of u32 words, then the tables.
+constexpr uint32_t kPlanMagic = 0x45504C54u;
+constexpr int kHdrMagic = 0, kHdrKind = 1, kHdrProbBits = 2, kHdrCosetFreq0 = 3, kHdrSymMin = 4, kHdrAlphabet = 21;
+constexpr int kHeaderWords = 64;
+constexpr size_t kHeaderBytes = kHeaderWords * 4;
+
+// LDS_BYTE entry: freq[0:12) | (slot - cdf)[12:23) | (value + 128)[24:32)
+// LDS_WIDE entry: freq[0:11) | (slot - cdf)[11:22) | symbol[22:32)
+// GLOBAL64 entry: symbol[0:16) | freq[16:32) | (slot - cdf)[32:64)
+
+// Payload ring kept in LDS per tile by the LDS-table kernels: 2 chunks of 64 words.
+constexpr int kRingWords = 128;
+constexpr int kRingBytes = kRingWords * 2;
+constexpr int kChunkWords = 64;
+
+void set_runtime_error(hipError_t e);
+
+#define EP_HIP_TRY(expr)                         \
+  do {                                           \
+    hipError_t ep_try_status_ = (expr);          \
+    if (ep_try_status_ != hipSuccess) {          \
+      ::ep::set_runtime_error(ep_try_status_);   \
+      return EP_HIP_ERUNTIME;                    \
+    }                                            \
+  } while (0)
+
+inline int tile_vectors_of(int tile_elements) {
+  const int v = tile_elements / 9;
+  return v > 32 ? v : 32;
+}
+
+// LDS bytes the LDS-table decode kernel needs for `waves` wavefronts each carrying `ilp` tile pairs.
+inline int lds_decode_bytes(int prob_bits, int waves, int ilp) {
+  return (kFieldStreams << prob_bits) * 4 + waves * ilp * 2 * kRingBytes + 256;
+}
+
+}  // namespace ep

@@ -1,0 +1,190 @@
+// Library bookkeeping, device query, and the decode plan: choosing a table representation on the host and
+// building the slot tables on the device.
+#include <string.h>
+
+#include "ep_common.hpp"
+
+namespace ep {
+
+static thread_local int g_last_runtime_error = 0;
+
+void set_runtime_error(hipError_t e) { g_last_runtime_error = static_cast<int>(e); }
+
+// One block per stream. Threads split the alphabet into contiguous chunks, scan the chunk sums, then each
+// thread writes the slot entries of its own symbols, so slot ranges are disjoint and no atomics are needed.
+__global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __restrict__ meta,
+                                                           const uint16_t* __restrict__ freq_tables, int kind,
+                                                           int prob_bits, uint32_t* __restrict__ plan) {
+  __shared__ uint32_t chunk_sum[256];
+  const int stream = blockIdx.x;
+  const int tid = threadIdx.x;
+  const uint32_t size = 1u << prob_bits;
+  const int sym_min = meta[stream * kMetaWidth + 1];
+  const int freq_off = meta[stream * kMetaWidth + 2];
+  const int alphabet = meta[stream * kMetaWidth + 3];
+
+  if (tid == 0) {
+    plan[kHdrSymMin + stream] = static_cast<uint32_t>(sym_min);
+    plan[kHdrAlphabet + stream] = static_cast<uint32_t>(alphabet);
+    if (stream == 0) {
+      plan[kHdrMagic] = kPlanMagic;
+      plan[kHdrKind] = static_cast<uint32_t>(kind);
+      plan[kHdrProbBits] = static_cast<uint32_t>(prob_bits);
+      // Symbol-0 frequency of the coset stream; an empty coset stream cannot occur in a valid container.
+      plan[kHdrCosetFreq0] = alphabet > 0 ? freq_tables[freq_off] : size;
+    }
+  }
+  if (kind != EP_TABLE_GLOBAL64 && stream == 0) return;   // the coset stream is decoded in closed form
+  if (alphabet <= 0) return;
+
+  const uint16_t* freq = freq_tables + freq_off;
+  const int per = (alphabet + 255) / 256;
+  const int first = tid * per;
+  const int last = first + per < alphabet ? first + per : alphabet;
+  uint32_t local = 0;
+  for (int s = first; s < last; ++s) local += freq[s];
+  chunk_sum[tid] = local;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t running = 0;
+    for (int i = 0; i < 256; ++i) {
+      const uint32_t v = chunk_sum[i];
+      chunk_sum[i] = running;
+      running += v;
+    }
+  }
+  __syncthreads();
+  uint32_t running = chunk_sum[tid];
+  uint8_t* tables = reinterpret_cast<uint8_t*>(plan) + kHeaderBytes;
+  for (int s = first; s < last; ++s) {
+    const uint32_t f = freq[s];
+    for (uint32_t d = 0; d < f && running + d < size; ++d) {
+      const uint32_t slot = running + d;
+      if (kind == EP_TABLE_GLOBAL64) {
+        uint64_t* lut = reinterpret_cast<uint64_t*>(tables) + (static_cast<size_t>(stream) << prob_bits);
+        lut[slot] = (static_cast<uint64_t>(d) << 32) | (static_cast<uint64_t>(f) << 16) | static_cast<uint64_t>(s);
+      } else {
+        uint32_t* lut = reinterpret_cast<uint32_t*>(tables) + (static_cast<size_t>(stream - 1) << prob_bits);
+        if (kind == EP_TABLE_LDS_BYTE) {
+          lut[slot] = f | (d << 12) | (static_cast<uint32_t>(s + sym_min + 128) << 24);
+        } else {
+          lut[slot] = f | (d << 11) | (static_cast<uint32_t>(s) << 22);
+        }
+      }
+    }
+    running += f;
+  }
+}
+
+}  // namespace ep
+
+extern "C" {
+
+int ep_hip_abi_version(void) { return EP_HIP_ABI_VERSION; }
+
+const char* ep_hip_error_string(int status) {
+  switch (status) {
+    case EP_HIP_OK: return "ok";
+    case EP_HIP_EINVAL: return "invalid argument";
+    case EP_HIP_EUNSUPPORTED: return "unsupported by this build";
+    case EP_HIP_ERUNTIME: return "HIP runtime call failed";
+    case EP_HIP_ENODEVICE: return "no gfx950 device";
+    default: return "unknown status";
+  }
+}
+
+int ep_hip_last_runtime_error(void) { return ep::g_last_runtime_error; }
+
+int ep_hip_device_query(int device, ep_hip_device_info* info) {
+  if (info == nullptr) return EP_HIP_EINVAL;
+  memset(info, 0, sizeof(*info));
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return EP_HIP_ENODEVICE;
+  if (device < 0) EP_HIP_TRY(hipGetDevice(&device));
+  if (device >= count) return EP_HIP_EINVAL;
+  hipDeviceProp_t prop;
+  EP_HIP_TRY(hipGetDeviceProperties(&prop, device));
+  info->device = device;
+  info->compute_units = prop.multiProcessorCount;
+  info->wavefront_size = prop.warpSize;
+  int lds = 0;
+  if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess) lds = 65536;
+  info->lds_bytes_per_block = lds;
+  strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+  info->is_gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+  return info->is_gfx950 ? EP_HIP_OK : EP_HIP_ENODEVICE;
+}
+
+int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_freq, int prob_bits, int lds_limit_bytes,
+                         int force_kind, ep_hip_plan_desc* desc) {
+  if (meta == nullptr || desc == nullptr || (freq == nullptr && n_freq != 0)) return EP_HIP_EINVAL;
+  if (prob_bits < 9 || prob_bits > 15) return EP_HIP_EINVAL;
+  memset(desc, 0, sizeof(*desc));
+  const int64_t size = int64_t{1} << prob_bits;
+  int64_t cursor = 0;
+  int max_alphabet = 0;
+  bool byte_ok = true, wide_ok = true;
+  for (int s = 0; s < ep::kStreams; ++s) {
+    const int64_t sym_min = meta[s * 4 + 1], off = meta[s * 4 + 2], alphabet = meta[s * 4 + 3];
+    if (meta[s * 4 + 0] < 0 || alphabet < 0 || off != cursor || off + alphabet > static_cast<int64_t>(n_freq)) return EP_HIP_EINVAL;
+    if (alphabet > size) return EP_HIP_EINVAL;
+    if (alphabet > 0) {
+      int64_t sum = 0, top = 0;
+      for (int64_t i = 0; i < alphabet; ++i) {
+        sum += freq[off + i];
+        top = freq[off + i] > top ? freq[off + i] : top;
+      }
+      if (sum != size) return EP_HIP_EINVAL;
+      if (s == 0) {
+        if (alphabet > 2 || sym_min != 0) return EP_HIP_EINVAL;   // the coset stream codes 0/1
+      } else {
+        if (sym_min < -128 || sym_min + alphabet - 1 > 127) byte_ok = false;
+        if (alphabet > 1024 || top > 2047) wide_ok = false;
+      }
+    }
+    if (alphabet > max_alphabet) max_alphabet = static_cast<int>(alphabet);
+    cursor += alphabet;
+  }
+  if (cursor != static_cast<int64_t>(n_freq)) return EP_HIP_EINVAL;
+  if (meta[0 * 4 + 3] == 0) return EP_HIP_EINVAL;
+
+  const bool lds_fits = prob_bits <= 11 && ep::lds_decode_bytes(prob_bits, 1, 1) <= lds_limit_bytes;
+  int kind = EP_TABLE_GLOBAL64;
+  if (lds_fits && byte_ok) kind = EP_TABLE_LDS_BYTE;
+  else if (lds_fits && wide_ok) kind = EP_TABLE_LDS_WIDE;
+  if (force_kind >= 0) {
+    const bool allowed = force_kind == EP_TABLE_GLOBAL64 || (force_kind == EP_TABLE_LDS_BYTE && lds_fits && byte_ok) ||
+                         (force_kind == EP_TABLE_LDS_WIDE && lds_fits && wide_ok);
+    if (!allowed) return EP_HIP_EUNSUPPORTED;
+    kind = force_kind;
+  }
+  desc->table_kind = kind;
+  desc->prob_bits = prob_bits;
+  desc->max_alphabet = max_alphabet;
+  desc->alphabet_sum = static_cast<int>(cursor);
+  if (kind == EP_TABLE_GLOBAL64) {
+    desc->table_bytes = ep::kHeaderBytes + (static_cast<size_t>(ep::kStreams) << prob_bits) * 8;
+    desc->lds_bytes = 0;
+  } else {
+    desc->table_bytes = ep::kHeaderBytes + (static_cast<size_t>(ep::kFieldStreams) << prob_bits) * 4;
+    desc->lds_bytes = (ep::kFieldStreams << prob_bits) * 4;
+  }
+  return EP_HIP_OK;
+}
+
+int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_tables_dev, const ep_hip_plan_desc* desc,
+                      void* tables_dev, void* stream) {
+  if (stream_meta_dev == nullptr || desc == nullptr || tables_dev == nullptr) return EP_HIP_EINVAL;
+  if (freq_tables_dev == nullptr && desc->alphabet_sum != 0) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(tables_dev) % 256 != 0) return EP_HIP_EINVAL;
+  if (desc->prob_bits < 9 || desc->prob_bits > 15 || desc->table_kind < 0 || desc->table_kind > EP_TABLE_LDS_WIDE) return EP_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // Slots of empty streams are never read, but keep the buffer deterministic.
+  EP_HIP_TRY(hipMemsetAsync(tables_dev, 0, desc->table_bytes, s));
+  hipLaunchKernelGGL(ep::build_tables_kernel, dim3(ep::kStreams), dim3(256), 0, s, stream_meta_dev, freq_tables_dev,
+                     desc->table_kind, desc->prob_bits, static_cast<uint32_t*>(tables_dev));
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,120 @@
+/* entropack_hip.h -- C ABI of libentropack_hip.so: the MI355X (gfx950) lane of the lattice_rans decode path.
+ *
+ * Every pointer named *_dev is a device pointer (e.g. torch `tensor.data_ptr()`), every *_host pointer is host
+ * memory. No entry point allocates or frees device memory and none synchronises the stream unless it says so;
+ * work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the default stream). All functions return
+ * 0 (EP_HIP_OK) or one of the EP_HIP_E* codes below; ep_hip_error_string() names them.
+ *
+ * The reference has no C ABI: its CUDA lane hands raw pointers and numpy scalars to CuPy-compiled kernels. Each
+ * entry point below cites the reference interface it stands in for (paths relative to the reference root).
+ */
+#ifndef ENTROPACK_HIP_H
+#define ENTROPACK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EP_HIP_ABI_VERSION 1
+
+enum ep_hip_status {
+  EP_HIP_OK = 0,
+  EP_HIP_EINVAL = 1,        /* a size, alignment or enum argument is out of range */
+  EP_HIP_EUNSUPPORTED = 2,  /* valid request this build has no kernel for */
+  EP_HIP_ERUNTIME = 3,      /* a HIP runtime call failed; ep_hip_last_runtime_error() has the hipError_t */
+  EP_HIP_ENODEVICE = 4      /* no gfx950 device visible */
+};
+
+/* Output container kinds. 0..12 keep the numbering of the reference's store kinds
+ * (entropack/schemes/lattice_rans/cuda.py:65-68, lattice_rans.cu:525-539); bf16 is its own kind here instead of
+ * a separate kernel family. */
+enum ep_hip_store_kind {
+  EP_STORE_F32 = 0, EP_STORE_F16 = 1, EP_STORE_F8E4M3FN = 2, EP_STORE_F8E5M2 = 3,
+  EP_STORE_I8 = 4, EP_STORE_I16 = 5, EP_STORE_I32 = 6, EP_STORE_I64 = 7,
+  EP_STORE_U8 = 8, EP_STORE_U16 = 9, EP_STORE_U32 = 10, EP_STORE_U64 = 11,
+  EP_STORE_BOOL = 12, EP_STORE_BF16 = 13
+};
+
+/* How a plan holds the slot -> (symbol, frequency, slot - cdf) map. The reference chooses among "shared",
+ * "packed" and "wide" tables (entropack/schemes/lattice_rans/cuda.py:600-610,697-741); all decode to identical
+ * output, and so do these. */
+enum ep_hip_table_kind {
+  EP_TABLE_GLOBAL64 = 0,    /* u64 per slot in HBM/L2, any prob_bits 9..15, any alphabet */
+  EP_TABLE_LDS_BYTE = 1,    /* u32 per slot, LDS-resident; prob_bits <= 11, every field value in [-128, 127] */
+  EP_TABLE_LDS_WIDE = 2     /* u32 per slot, LDS-resident; prob_bits <= 11, alphabets <= 1024, frequencies < 2048 */
+};
+
+/* Device-side error flag values written (first one wins) to *error_dev by the decode kernels; same meaning as the
+ * reference's set_error codes (lattice_rans.cu:51-53,777,799). */
+enum ep_hip_decode_error {
+  EP_DECODE_OK = 0,
+  EP_DECODE_OVERREAD = 2,      /* renormalisation would read below the tile's first payload word */
+  EP_DECODE_NOT_CONSUMED = 3,  /* tile ended with unread words or a lane state != 2^15 */
+  EP_DECODE_BAD_OFFSETS = 4    /* offsets[t] > offsets[t+1] or offsets[t+1] > payload_words */
+};
+
+typedef struct ep_hip_device_info {
+  int device;                 /* HIP device ordinal */
+  int compute_units;
+  int lds_bytes_per_block;    /* largest LDS allocation one workgroup may make */
+  int wavefront_size;
+  int is_gfx950;              /* 1 when gcnArchName starts with "gfx950" */
+  char arch[64];
+} ep_hip_device_info;
+
+typedef struct ep_hip_plan_desc {
+  int table_kind;             /* enum ep_hip_table_kind chosen for this container */
+  int prob_bits;
+  size_t table_bytes;         /* size of the device buffer ep_hip_plan_build fills (256-byte aligned start needed) */
+  int lds_bytes;              /* dynamic LDS the decode kernel will request (0 for GLOBAL64) */
+  int max_alphabet;
+  int alphabet_sum;
+} ep_hip_plan_desc;
+
+/* Library / device ------------------------------------------------------------------------------------------ */
+
+int ep_hip_abi_version(void);
+const char* ep_hip_error_string(int status);
+int ep_hip_last_runtime_error(void);   /* hipError_t of the last failed runtime call on this thread, 0 if none */
+
+/* Stands in for the reference's probe() + caps() (entropack/backends/cuda/__init__.py:4-12,
+ * entropack/backends/cuda/device.py:66-81). `device` < 0 = current device. */
+int ep_hip_device_query(int device, ep_hip_device_info* info);
+
+/* Plan ------------------------------------------------------------------------------------------------------ */
+
+/* Chooses the table representation from host copies of the container's stream_meta (int32[17][4] =
+ * n_symbols, sym_min, freq_offset, alphabet) and freq_tables (u16[n_freq]), and validates them (offsets
+ * contiguous, every stream's frequencies sum to 2^prob_bits). Pure host code, no GPU needed.
+ * Reference: _decode_plan's representation choice, entropack/schemes/lattice_rans/cuda.py:697-732.
+ * `force_kind` < 0 lets the library choose; otherwise it must be a kind the container qualifies for. */
+int ep_hip_plan_describe(const int32_t* stream_meta_host, const uint16_t* freq_tables_host, size_t n_freq,
+                         int prob_bits, int lds_limit_bytes, int force_kind, ep_hip_plan_desc* desc);
+
+/* Builds the decode tables on the device, from the container's own device buffers, into `tables_dev`
+ * (desc->table_bytes bytes, caller-allocated, 256-byte aligned). Asynchronous on `stream`.
+ * Reference: _shared_tables / _packed_tables / _wide_tables (host numpy + upload),
+ * entropack/schemes/lattice_rans/cuda.py:647-679. */
+int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_tables_dev, const ep_hip_plan_desc* desc,
+                      void* tables_dev, void* stream);
+
+/* Decode ---------------------------------------------------------------------------------------------------- */
+
+/* Entropy-decodes every tile and reconstructs straight into `out_dev` ([rows][cols_padded] of `store_kind`,
+ * row-major, 16-byte aligned): rANS symbol steps, shared renormalisation, field minima, E8 point, row scale and
+ * container cast, in one kernel. payload_dev must be 4-byte aligned. `error_dev` (int32, caller-zeroed) receives
+ * an ep_hip_decode_error; it is never read back here.
+ * Reference: decode() + _decode_launch() and the e8_decode_vector_* kernels they launch,
+ * entropack/schemes/lattice_rans/cuda.py:744-805, lattice_rans.cu:732-1141. */
+int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, const uint32_t* offsets_dev,
+                          const uint32_t* states_dev, const float* scales_dev, const void* tables_dev,
+                          const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows,
+                          int64_t cols_padded, int tile_elements, int32_t* error_dev, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ENTROPACK_HIP_H */
