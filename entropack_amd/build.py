@@ -11,6 +11,9 @@ CSRC = os.path.join(PACKAGE_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PACKAGE_DIR), "include")
 HIP_LIBRARY = os.path.join(PACKAGE_DIR, "libentropack_hip.so")
 HIP_SOURCES = ("ep_plan.hip", "ep_decode.hip")
+HOST_LIBRARY = os.path.join(PACKAGE_DIR, "libentropack_host.so")
+HOST_SOURCES = ("host_codec.c",)
+HOST_FLAGS = ("-O2", "-std=c11", "-fPIC", "-shared", "-fopenmp", "-ffp-contract=off", "-Wall", "-Wextra")
 
 HIPCC_FLAGS = (
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
@@ -37,7 +40,20 @@ def build_hip(verbose: bool = False, extra_flags=()) -> str:
     return HIP_LIBRARY
 
 
+def build_host(verbose: bool = False) -> str:
+    """The CPU encoder kernels (plain C)."""
+    sources = [os.path.join(CSRC, name) for name in HOST_SOURCES]
+    command = [os.environ.get("CC", "gcc"), *HOST_FLAGS, "-o", HOST_LIBRARY, *sources, "-lm"]
+    if verbose:
+        print(" ".join(command), flush=True)
+    done = subprocess.run(command, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError(f"gcc failed ({done.returncode}):\n{done.stdout}\n{done.stderr}")
+    return HOST_LIBRARY
+
+
 def build_all(verbose: bool = False) -> None:
+    build_host(verbose)
     build_hip(verbose)
 
 

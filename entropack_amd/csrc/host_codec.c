@@ -1,0 +1,229 @@
+/* libentropack_host.so: CPU encoder kernels of the lattice_rans scheme (plain C + OpenMP, no GPU).
+ *
+ * The MI355X path only decodes. Containers still have to come from somewhere, so the package carries its own
+ * CPU restatement of the reference encoder; the heavy loops live here and the orchestration (scale search,
+ * Hamilton normalisation, row-scale refit) in schemes/lattice_rans/eager.py. Algorithms followed, in the
+ * reference tree:
+ *   hc_quantize      entropack/schemes/lattice_rans/eager.py:18-51  (nearest E8 point, point -> coset + fields)
+ *   hc_levels        entropack/schemes/lattice_rans/eager.py:54-58  (fields -> point)
+ *   hc_rans_encode   entropack/schemes/lattice_rans/rans.py:133-186 (tiled 32-way interleaved rANS encode)
+ * Built with -ffp-contract=off: every float operation below is a single IEEE operation, as in the reference.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define HC_STATES 32
+#define HC_STATE_MIN (1u << 15)
+#define HC_STREAMS 17
+
+static void nearest_dn(const float* y, float* out) {
+  float r[8];
+  float total = 0.0f;
+  for (int j = 0; j < 8; ++j) {
+    out[j] = rintf(y[j]);            /* round half to even */
+    r[j] = y[j] - out[j];
+    total += out[j];                 /* small integers: exact in any order */
+  }
+  int at = 0;
+  float best = -1.0f;
+  for (int j = 0; j < 8; ++j) {
+    const float a = fabsf(r[j]);
+    if (a > best) { best = a; at = j; }   /* first maximum wins */
+  }
+  if (fmodf(total, 2.0f) != 0.0f) out[at] += (r[at] < 0.0f) ? -1.0f : 1.0f;   /* a zero residual steps up */
+}
+
+/* Sum of squared differences in float64, paired as (0+4)+(2+6) and (1+5)+(3+7): the order the reference's
+ * per-row float64 reduction uses, which decides exact ties between the two cosets. */
+static double distance2(const float* y, const float* p) {
+  double s[8];
+  for (int j = 0; j < 8; ++j) {
+    const double d = (double)y[j] - (double)p[j];
+    s[j] = d * d;
+  }
+  return ((s[0] + s[4]) + (s[2] + s[6])) + ((s[1] + s[5]) + (s[3] + s[7]));
+}
+
+/* Quantises rows `row_index[0..n_sel)` (or rows 0..n_sel when row_index is NULL) of x[rows][cols]:
+ * y = (x / rms[row]) / scale, nearest E8 point, split into coset bit and the 8 fields (z0..z6, m).
+ * coset: int8[n_sel * cols / 8]; fields: int32[n_sel * cols / 8][8]. */
+void hc_quantize(const float* x, const float* rms, int64_t cols, float scale, const int64_t* row_index, int64_t n_sel,
+                 int8_t* coset, int32_t* fields, int threads) {
+  const int64_t vpr = cols / 8;
+#pragma omp parallel for schedule(static) num_threads(threads > 0 ? threads : 1)
+  for (int64_t i = 0; i < n_sel; ++i) {
+    const int64_t row = row_index ? row_index[i] : i;
+    const float* src = x + row * cols;
+    const float norm = rms[row];
+    for (int64_t v = 0; v < vpr; ++v) {
+      float y[8], shifted[8], c0[8], c1[8];
+      for (int j = 0; j < 8; ++j) {
+        y[j] = (src[v * 8 + j] / norm) / scale;
+        shifted[j] = y[j] - 0.5f;
+      }
+      nearest_dn(y, c0);
+      nearest_dn(shifted, c1);
+      for (int j = 0; j < 8; ++j) c1[j] += 0.5f;
+      const int c = !(distance2(y, c0) <= distance2(y, c1));
+      const float* p = c ? c1 : c0;
+      int32_t z[8];
+      int32_t sum = 0;
+      for (int j = 0; j < 8; ++j) z[j] = (int32_t)rintf(p[j] - (c ? 0.5f : 0.0f));
+      for (int j = 0; j < 7; ++j) sum += z[j];
+      const int32_t parity = sum & 1;
+      const int32_t top = z[7] - parity;          /* even by construction of E8; floor-divide anyway */
+      z[7] = (top >= 0) ? top / 2 : -((-top + 1) / 2);
+      const int64_t at = i * vpr + v;
+      coset[at] = (int8_t)c;
+      memcpy(fields + at * 8, z, sizeof(z));
+    }
+  }
+}
+
+/* Lattice point of each vector as float32[V][8]: z0..z6, 2 m + parity, plus c / 2. */
+void hc_levels(const int8_t* coset, const int32_t* fields, int64_t vectors, float* levels, int threads) {
+#pragma omp parallel for schedule(static) num_threads(threads > 0 ? threads : 1)
+  for (int64_t v = 0; v < vectors; ++v) {
+    const int32_t* z = fields + v * 8;
+    int32_t sum = 0;
+    for (int j = 0; j < 7; ++j) sum += z[j];
+    const float half = coset[v] ? 0.5f : 0.0f;
+    for (int j = 0; j < 7; ++j) levels[v * 8 + j] = (float)z[j] + half;
+    levels[v * 8 + 7] = (float)(2 * z[7] + (sum & 1)) + half;
+  }
+}
+
+/* Per stream (0 = coset, 1 + 2f + c = field f of coset-c vectors): symbol count, minimum and maximum.
+ * stats: int64[17][3] = (n, min, max); min/max are 0 for empty streams. */
+void hc_stream_stats(const int8_t* coset, const int32_t* fields, int64_t vectors, int64_t* stats) {
+  int64_t n[HC_STREAMS] = {0}, lo[HC_STREAMS], hi[HC_STREAMS];
+  for (int s = 0; s < HC_STREAMS; ++s) { lo[s] = INT64_MAX; hi[s] = INT64_MIN; }
+  for (int64_t v = 0; v < vectors; ++v) {
+    const int c = coset[v];
+    n[0]++;
+    if (c < lo[0]) lo[0] = c;
+    if (c > hi[0]) hi[0] = c;
+    for (int f = 0; f < 8; ++f) {
+      const int s = 1 + 2 * f + c;
+      const int64_t z = fields[v * 8 + f];
+      n[s]++;
+      if (z < lo[s]) lo[s] = z;
+      if (z > hi[s]) hi[s] = z;
+    }
+  }
+  for (int s = 0; s < HC_STREAMS; ++s) {
+    stats[3 * s] = n[s];
+    stats[3 * s + 1] = n[s] ? lo[s] : 0;
+    stats[3 * s + 2] = n[s] ? hi[s] : 0;
+  }
+}
+
+/* Histogram of every stream. counts is the concatenation of the 17 histograms; stream s starts at
+ * count_offset[s] and bins (value - sym_min[s]). */
+void hc_stream_counts(const int8_t* coset, const int32_t* fields, int64_t vectors, const int64_t* sym_min,
+                      const int64_t* count_offset, int64_t* counts) {
+  for (int64_t v = 0; v < vectors; ++v) {
+    const int c = coset[v];
+    counts[count_offset[0] + c - sym_min[0]]++;
+    for (int f = 0; f < 8; ++f) {
+      const int s = 1 + 2 * f + c;
+      counts[count_offset[s] + fields[v * 8 + f] - sym_min[s]]++;
+    }
+  }
+}
+
+typedef struct {
+  uint16_t* words;
+  size_t size, capacity;
+} word_list;
+
+static int push_word(word_list* list, uint16_t w) {
+  if (list->size == list->capacity) {
+    const size_t grown = list->capacity ? list->capacity * 2 : 4096;
+    uint16_t* moved = (uint16_t*)realloc(list->words, grown * sizeof(uint16_t));
+    if (!moved) return -1;
+    list->words = moved;
+    list->capacity = grown;
+  }
+  list->words[list->size++] = w;
+  return 0;
+}
+
+static inline int put(uint32_t* state, uint32_t freq, uint32_t cdf, int prob_bits, word_list* out) {
+  uint32_t x = *state;
+  if (x >= (freq << (31 - prob_bits))) {          /* rans.py:168-170 */
+    if (push_word(out, (uint16_t)(x & 0xFFFFu))) return -1;
+    x >>= 16;
+  }
+  *state = (x / freq) * (1u << prob_bits) + (x % freq) + cdf;
+  return 0;
+}
+
+/* Tiled 32-way interleaved rANS encode of all vectors. freq / cdf: per stream, indexed by (value - sym_min[s]),
+ * concatenated with stream s starting at table_offset[s]. states: u32[tiles][32]; offsets: u32[tiles + 1];
+ * *payload receives a malloc'd array of offsets[tiles] words (free it with hc_free). Returns 0, or -1 when out of
+ * memory, or -2 when the payload would not fit 32-bit offsets. */
+int hc_rans_encode(const int8_t* coset, const int32_t* fields, int64_t vectors, const int64_t* sym_min,
+                   const int64_t* table_offset, const uint32_t* freq, const uint32_t* cdf, int prob_bits,
+                   int tile_vectors, uint32_t* states, uint32_t* offsets, uint16_t** payload, int threads) {
+  int64_t tiles = (vectors + tile_vectors - 1) / tile_vectors;
+  if (tiles < 1) tiles = 1;
+  word_list* lists = (word_list*)calloc((size_t)tiles, sizeof(word_list));
+  if (!lists) return -1;
+  int failed = 0;
+#pragma omp parallel for schedule(dynamic, 8) num_threads(threads > 0 ? threads : 1)
+  for (int64_t tile = 0; tile < tiles; ++tile) {
+    const int64_t begin = tile * tile_vectors;
+    const int64_t end = begin + tile_vectors < vectors ? begin + tile_vectors : vectors;
+    uint32_t x[HC_STATES];
+    for (int l = 0; l < HC_STATES; ++l) x[l] = HC_STATE_MIN;
+    word_list* out = &lists[tile];
+    int bad = 0;
+    for (int64_t base = begin; base < end && !bad; base += HC_STATES) {
+      const int lanes = (int)(end - base < HC_STATES ? end - base : HC_STATES);
+      for (int f = 7; f >= 0 && !bad; --f) {                     /* fields last to first, then the coset */
+        for (int l = 0; l < lanes; ++l) {
+          const int64_t v = base + l;
+          const int s = 1 + 2 * f + coset[v];
+          const int64_t at = table_offset[s] + fields[v * 8 + f] - sym_min[s];
+          if (put(&x[l], freq[at], cdf[at], prob_bits, out)) { bad = 1; break; }
+        }
+      }
+      for (int l = 0; l < lanes && !bad; ++l) {
+        const int64_t at = table_offset[0] + coset[base + l] - sym_min[0];
+        if (put(&x[l], freq[at], cdf[at], prob_bits, out)) bad = 1;
+      }
+    }
+    memcpy(states + tile * HC_STATES, x, sizeof(x));
+    if (bad) {
+#pragma omp atomic write
+      failed = 1;
+    }
+  }
+  uint64_t total = 0;
+  offsets[0] = 0;
+  for (int64_t tile = 0; tile < tiles; ++tile) {
+    total += lists[tile].size;
+    if (total > 0xFFFFFFFFull) failed = 2;
+    offsets[tile + 1] = (uint32_t)total;
+  }
+  uint16_t* joined = NULL;
+  if (!failed) {
+    joined = (uint16_t*)malloc((total ? total : 1) * sizeof(uint16_t));
+    if (!joined) failed = 1;
+  }
+  if (!failed) {
+#pragma omp parallel for schedule(static) num_threads(threads > 0 ? threads : 1)
+    for (int64_t tile = 0; tile < tiles; ++tile) {
+      if (lists[tile].size) memcpy(joined + offsets[tile], lists[tile].words, lists[tile].size * sizeof(uint16_t));
+    }
+  }
+  for (int64_t tile = 0; tile < tiles; ++tile) free(lists[tile].words);
+  free(lists);
+  *payload = joined;
+  return failed == 0 ? 0 : (failed == 2 ? -2 : -1);
+}
+
+void hc_free(void* p) { free(p); }

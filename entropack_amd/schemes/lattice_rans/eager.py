@@ -1,8 +1,334 @@
-"""`eager` (CPU) lane of lattice_rans. Placeholder until the encoder lands."""
+"""`eager` (CPU) lane of lattice_rans: the encoder.
+
+The accelerated path of this package is decode-only; this lane produces the containers it decodes. It restates the
+reference's CPU encoder (entropack/schemes/lattice_rans/eager.py:91-341 and rans.py:12-95,133-258) so that the same
+input and config give the same container, bit for bit: row RMS normalisation, a bisection of the lattice scale
+against an analytic size model on a seeded row subsample, nearest-E8 quantisation, least-squares refit of the row
+scales, Hamilton-normalised frequency tables and the tiled 32-way interleaved rANS encode. The per-vector and
+per-symbol loops run in libentropack_host.so (csrc/host_codec.c).
+
+Not restated: the optional per-row rate-distortion pass (`row_rdo_iterations > 0` raises).
+
+`decode` is deliberately absent: containers are decoded by the `hip` lane. Asking this lane to decode raises.
+"""
+import ctypes
+import math
+import os
+
+import numpy as np
+import torch
+
+from .format import (
+    LATTICE_DIM, META_ALPHABET, META_FREQ_OFFSET, META_N_SYMBOLS, META_SYM_MIN, META_WIDTH, NUM_FIELDS, NUM_STATES,
+    NUM_STREAMS, LatticeBuffers, log, make_layout, resolve_prob_bits, vector_tile_elements,
+)
+
+MIN_RMS = 1.0e-12
+ALPHABET_COARSEN_MARGIN = 1.05
+SUBSAMPLE_SEED_MULTIPLIER = 1000003
+#: Constants of the analytic size model; they are part of what the scale search converges to.
+MODEL_LAYOUT_BYTES = 64
+MODEL_STREAM_META_BYTES = 408
+MODEL_SLACK_BYTES = 384
+
+_PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+HOST_LIBRARY_PATH = os.path.join(_PACKAGE_DIR, "libentropack_host.so")
+_host = None
 
 
-def encode(**kwargs):
-    raise NotImplementedError("CPU encoder not built yet")
+def host_library() -> ctypes.CDLL:
+    global _host
+    if _host is None:
+        if not os.path.exists(HOST_LIBRARY_PATH):
+            raise ImportError(f"{HOST_LIBRARY_PATH} is missing: build it with `python -m entropack_amd.build`")
+        lib = ctypes.CDLL(HOST_LIBRARY_PATH)
+        p, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        lib.hc_quantize.argtypes = [p, p, i64, ctypes.c_float, p, i64, p, p, i32]
+        lib.hc_quantize.restype = None
+        lib.hc_levels.argtypes = [p, p, i64, p, i32]
+        lib.hc_levels.restype = None
+        lib.hc_stream_stats.argtypes = [p, p, i64, p]
+        lib.hc_stream_stats.restype = None
+        lib.hc_stream_counts.argtypes = [p, p, i64, p, p, p]
+        lib.hc_stream_counts.restype = None
+        lib.hc_rans_encode.argtypes = [p, p, i64, p, p, p, p, i32, i32, p, p, ctypes.POINTER(ctypes.c_void_p), i32]
+        lib.hc_rans_encode.restype = i32
+        lib.hc_free.argtypes = [p]
+        lib.hc_free.restype = None
+        _host = lib
+    return _host
+
+
+def _threads() -> int:
+    return max(1, min(torch.get_num_threads(), os.cpu_count() or 1))
+
+
+def _address(array: np.ndarray) -> int:
+    return array.ctypes.data
+
+
+# ---- quantisation ----------------------------------------------------------------------------------------------
+
+class Quantized:
+    """Coset bit and the eight integer fields (z0..z6, m) of every vector, as the C kernels hold them."""
+
+    def __init__(self, coset: np.ndarray, fields: np.ndarray):
+        self.coset, self.fields = coset, fields          # int8[V], int32[V, 8]
+
+    @property
+    def vectors(self) -> int:
+        return int(self.coset.size)
+
+    def stats(self) -> np.ndarray:
+        """int64[17, 3]: n, min, max of each stream."""
+        out = np.zeros((NUM_STREAMS, 3), dtype=np.int64)
+        host_library().hc_stream_stats(_address(self.coset), _address(self.fields), self.vectors, _address(out))
+        out[0, 1] = 0                    # the coset stream always counts from symbol 0
+        return out
+
+    def histograms(self, stats: np.ndarray):
+        """Per stream: counts over value - min (empty array for an empty stream)."""
+        alphabets = np.where(stats[:, 0] > 0, stats[:, 2] - stats[:, 1] + 1, 0)
+        starts = np.concatenate([[0], np.cumsum(alphabets)]).astype(np.int64)
+        counts = np.zeros(int(starts[-1]), dtype=np.int64)
+        minima = np.ascontiguousarray(stats[:, 1])
+        host_library().hc_stream_counts(_address(self.coset), _address(self.fields), self.vectors, _address(minima),
+                                        _address(starts), _address(counts))
+        return [counts[starts[s]:starts[s + 1]] for s in range(NUM_STREAMS)]
+
+    def levels(self) -> torch.Tensor:
+        out = np.empty((self.vectors, LATTICE_DIM), dtype=np.float32)
+        host_library().hc_levels(_address(self.coset), _address(self.fields), self.vectors, _address(out), _threads())
+        return torch.from_numpy(out)
+
+
+def quantize(x: np.ndarray, rms: np.ndarray, scale: float, rows_selected: np.ndarray | None = None) -> Quantized:
+    rows, cols = x.shape
+    picked = rows if rows_selected is None else int(rows_selected.size)
+    vectors = picked * (cols // LATTICE_DIM)
+    coset = np.empty(vectors, dtype=np.int8)
+    fields = np.empty((vectors, NUM_FIELDS), dtype=np.int32)
+    host_library().hc_quantize(
+        _address(x), _address(rms), cols, ctypes.c_float(scale), None if rows_selected is None else _address(rows_selected),
+        picked, _address(coset), _address(fields), _threads())
+    return Quantized(coset, fields)
+
+
+# ---- frequency tables and the size model -------------------------------------------------------------------------
+
+def normalize_counts(counts: np.ndarray, table_size: int) -> np.ndarray:
+    """Largest-remainder (Hamilton) allocation of `table_size` slots, every present symbol getting at least one.
+
+    A surplus is handed out by descending residual, a deficit taken back by ascending residual from symbols still
+    above 1; ties go to the smaller symbol (stable sorts), and a symbol can be visited again in a later pass.
+    """
+    counts = np.asarray(counts, dtype=np.int64)
+    if counts.size == 0 or int(counts.sum()) == 0:
+        raise ValueError("cannot build an rANS table from an empty symbol stream")
+    if counts.size > table_size:
+        raise ValueError(
+            f"E8 coordinate alphabet {counts.size} exceeds rANS table_size {table_size}; "
+            "raise prob_bits or coarsen the lattice scale")
+    seen = np.flatnonzero(counts)
+    ideal = counts.astype(np.float64) * (table_size / int(counts.sum()))
+    freq = np.floor(ideal).astype(np.int64)
+    freq[seen] = np.maximum(freq[seen], 1)
+    gap = table_size - int(freq.sum())
+    if gap > 0:
+        order = seen[np.argsort(-(ideal - freq)[seen], kind="stable")]
+        while gap > 0:
+            chosen = order[:gap]
+            freq[chosen] += 1
+            gap -= chosen.size
+    elif gap < 0:
+        rest = ideal - freq
+        pool = seen[freq[seen] > 1]
+        if pool.size == 0:
+            raise ValueError("unable to normalize rANS frequencies")
+        order = pool[np.argsort(rest[pool], kind="stable")]
+        while gap < 0:
+            alive = order[freq[order] > 1]
+            if alive.size == 0:
+                raise ValueError("unable to normalize rANS frequencies")
+            chosen = alive[:-gap]
+            freq[chosen] -= 1
+            gap += chosen.size
+    return freq.astype(np.uint16)
+
+
+def modelled_bytes(histograms, sizes, rows: int, prob_bits: int, tile_elements: int) -> float:
+    """Analytic container size for a set of stream histograms (reference rans.py:224-258 + eager.py:102-107)."""
+    table_size = 1 << prob_bits
+    bits = 0.0
+    table_bytes = 0
+    overflow_bits = 0.0
+    for n, hist in zip(sizes, histograms):
+        if n and hist.size <= table_size:
+            freq = normalize_counts(hist, table_size)
+            live = hist > 0
+            bits += float(np.sum(hist[live].astype(np.float64) * (prob_bits - np.log2(freq[live].astype(np.float64)))))
+            table_bytes += freq.size * 2
+        else:
+            overflow_bits += n * prob_bits
+    tile_vectors = vector_tile_elements(tile_elements)
+    tiles = max(1, (sizes[0] + tile_vectors - 1) // tile_vectors)
+    payload_words = int(np.ceil(max(0.0, bits - tiles * NUM_STATES * 16) / 16.0))
+    coded = payload_words * 2 + tiles * NUM_STATES * 4 + (tiles + 1) * 4 + table_bytes
+    return coded + overflow_bits / 8 + rows * 4 + MODEL_LAYOUT_BYTES + MODEL_STREAM_META_BYTES + MODEL_SLACK_BYTES
+
+
+def _model_of(q: Quantized, rows: int, prob_bits: int, tile_elements: int) -> float:
+    stats = q.stats()
+    return modelled_bytes(q.histograms(stats), [int(n) for n in stats[:, 0]], rows, prob_bits, tile_elements)
+
+
+def _largest_alphabet(q: Quantized) -> int:
+    stats = q.stats()
+    spans = np.where(stats[:, 0] > 0, stats[:, 2] - stats[:, 1] + 1, 0)
+    return int(spans.max())
+
+
+def bisect_scale(x, rms, rows, cols, target_bpp, prob_bits, tile_elements, iterations, max_vectors) -> float:
+    """Geometric bisection of the lattice scale on [0.001, 8] against the size model, on a seeded row subsample."""
+    per_row = cols // LATTICE_DIM
+    sample_rows = max(1, min(rows, max_vectors // per_row))
+    picked = None
+    if sample_rows < rows:
+        generator = torch.Generator().manual_seed(rows * SUBSAMPLE_SEED_MULTIPLIER + cols)
+        picked = np.ascontiguousarray(torch.randperm(rows, generator=generator)[:sample_rows].numpy(), dtype=np.int64)
+    elements = sample_rows * cols
+    low, high = 0.001, 8.0
+    for _ in range(iterations):
+        middle = math.sqrt(low * high)
+        size = _model_of(quantize(x, rms, middle, picked), sample_rows, prob_bits, tile_elements)
+        if 8 * size / elements > target_bpp:
+            low = middle
+        else:
+            high = middle
+    return math.sqrt(low * high)
+
+
+def refit_row_scales(x_t: torch.Tensor, rms_t: torch.Tensor, q: Quantized, scale: float) -> torch.Tensor:
+    """Least-squares scale of each row against the points chosen for it (float32 row sums, as torch computes them)."""
+    rows, cols = x_t.shape
+    levels = q.levels().reshape(rows, cols)
+    numerator = (x_t * levels).sum(1)
+    denominator = levels.square().sum(1)
+    return torch.where(denominator > 0, (numerator / denominator).clamp_min(MIN_RMS), scale * rms_t.squeeze(1))
+
+
+def resolve_scale(x_t, rms_t, target_bpp, prob_bits, tile_elements, iterations, max_vectors):
+    """Scale search plus the alphabet guard: grow an automatic prob_bits (to 15 at most) while an alphabet overflows
+    the table, after that coarsen the scale by the overflow. Returns (quantised vectors, row scales, prob_bits)."""
+    rows, cols = x_t.shape
+    x = x_t.numpy()
+    rms = np.ascontiguousarray(rms_t.squeeze(1).numpy())
+    prob_bits, automatic = resolve_prob_bits(prob_bits, target_bpp)
+    if float(x_t.abs().amax()) == 0.0:
+        q = quantize(x, rms, 1.0)
+        return q, refit_row_scales(x_t, rms_t, q, 1.0), prob_bits
+    clamped = False
+    while True:
+        table_size = 1 << prob_bits
+        scale = bisect_scale(x, rms, rows, cols, target_bpp, prob_bits, tile_elements, iterations, max_vectors)
+        grow = False
+        while True:
+            q = quantize(x, rms, scale)
+            widest = _largest_alphabet(q)
+            if widest <= table_size:
+                break
+            if automatic and prob_bits < 15:
+                prob_bits += 1
+                grow = True
+                break
+            clamped = True
+            scale *= widest / table_size * ALPHABET_COARSEN_MARGIN
+        if grow:
+            continue
+        if clamped:
+            log.debug("lattice_rans coarsened the lattice scale to %.6g so a coordinate alphabet of %d fits the "
+                      "%d-entry rANS table; actual_bpp for this tensor will fall below target_bpp", scale, widest, table_size)
+        return q, refit_row_scales(x_t, rms_t, q, scale), prob_bits
+
+
+# ---- stream encode ---------------------------------------------------------------------------------------------
+
+def encode_streams(q: Quantized, prob_bits: int, tile_elements: int):
+    """Frequency tables + tiled rANS encode. Returns payload, states, offsets, stream_meta, freq_tables (numpy)."""
+    table_size = 1 << prob_bits
+    stats = q.stats()
+    histograms = q.histograms(stats)
+    meta = np.zeros((NUM_STREAMS, META_WIDTH), dtype=np.int64)
+    freq_parts, cdf_parts = [], []
+    cursor = 0
+    for stream, hist in enumerate(histograms):
+        n = int(stats[stream, 0])
+        meta[stream, META_N_SYMBOLS] = n
+        meta[stream, META_SYM_MIN] = int(stats[stream, 1]) if n else 0
+        meta[stream, META_FREQ_OFFSET] = cursor
+        meta[stream, META_ALPHABET] = hist.size if n else 0
+        if n:
+            freq = normalize_counts(hist, table_size).astype(np.int64)
+            freq_parts.append(freq)
+            cdf_parts.append(np.concatenate([[0], np.cumsum(freq)[:-1]]))
+            cursor += hist.size
+    freq_all = np.concatenate(freq_parts) if freq_parts else np.zeros(0, dtype=np.int64)
+    cdf_all = np.concatenate(cdf_parts) if cdf_parts else np.zeros(0, dtype=np.int64)
+
+    tile_vectors = vector_tile_elements(tile_elements)
+    tiles = max(1, (q.vectors + tile_vectors - 1) // tile_vectors)
+    states = np.empty((tiles, NUM_STATES), dtype=np.uint32)
+    offsets = np.zeros(tiles + 1, dtype=np.uint32)
+    minima = np.ascontiguousarray(meta[:, META_SYM_MIN])
+    starts = np.ascontiguousarray(meta[:, META_FREQ_OFFSET])
+    freq32 = np.ascontiguousarray(freq_all.astype(np.uint32))
+    cdf32 = np.ascontiguousarray(cdf_all.astype(np.uint32))
+    handle = ctypes.c_void_p()
+    status = host_library().hc_rans_encode(
+        _address(q.coset), _address(q.fields), q.vectors, _address(minima), _address(starts), _address(freq32),
+        _address(cdf32), prob_bits, tile_vectors, _address(states), _address(offsets), ctypes.byref(handle), _threads())
+    if status != 0:
+        raise MemoryError("rANS encode ran out of memory" if status == -1 else "payload exceeds 2**32 words")
+    try:
+        words = int(offsets[-1])
+        payload = np.ctypeslib.as_array(ctypes.cast(handle, ctypes.POINTER(ctypes.c_uint16)), shape=(max(words, 1),))[:words].copy()
+    finally:
+        host_library().hc_free(handle)
+    return payload, states, offsets, meta, freq_all.astype(np.uint16)
+
+
+def _as_torch(array: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
+    """numpy unsigned arrays -> torch tensors of the matching unsigned dtype (via a same-width signed view)."""
+    signed = {torch.uint16: np.int16, torch.uint32: np.int32}.get(dtype)
+    if signed is None:
+        return torch.from_numpy(np.ascontiguousarray(array))
+    return torch.from_numpy(np.ascontiguousarray(array).view(signed)).view(dtype)
+
+
+def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0, row_rdo_candidates=5,
+           scale_search_iterations=12, scale_search_max_vectors=262144) -> LatticeBuffers:
+    if int(row_rdo_iterations) > 0:
+        raise NotImplementedError("per-row rate-distortion refinement is not part of this build; use row_rdo_iterations=0")
+    if weight.shape[1] % LATTICE_DIM:
+        raise ValueError(
+            f"lattice_rans quantizes whole E8 vectors, so the column count must be a multiple of {LATTICE_DIM}; got cols={weight.shape[1]}")
+    device = weight.device
+    x_t = weight.detach().to("cpu").float().contiguous()
+    rows, cols = x_t.shape
+    rms_t = x_t.square().mean(dim=1, keepdim=True).sqrt().clamp_min(MIN_RMS)
+    if not bool(torch.isfinite(rms_t).all()):
+        raise ValueError(
+            f"lattice_rans normalizes rows in fp32, and the row RMS of this {weight.dtype} tensor overflowed; rescale the source")
+    q, scales, prob_bits = resolve_scale(
+        x_t, rms_t, float(target_bpp), None if prob_bits in (None, 0) else int(prob_bits), int(tile_elements),
+        int(scale_search_iterations), int(scale_search_max_vectors))
+    payload, states, offsets, meta, freq_tables = encode_streams(q, prob_bits, int(tile_elements))
+    return LatticeBuffers(
+        payload=_as_torch(payload, torch.uint16).to(device), offsets=_as_torch(offsets, torch.uint32).to(device),
+        states=_as_torch(states, torch.uint32).to(device), stream_meta=torch.from_numpy(meta.astype(np.int32)).to(device),
+        freq_tables=_as_torch(freq_tables, torch.uint16).to(device), scales=scales.contiguous().to(device),
+        layout=make_layout(cols, prob_bits, int(tile_elements)).to(device),
+    )
 
 
 def decode(buffers, *, shape, dtype, threads_per_block=None, l2_prefetch=True):
