@@ -131,7 +131,8 @@ def main():
     for _ in range(max(args.warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
-    hip_lane.check_errors(lattice)
+    if not os.environ.get("EP_HIP_DEBUG"):
+        hip_lane.check_errors(lattice)
 
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     torch.cuda.synchronize()

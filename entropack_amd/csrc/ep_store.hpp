@@ -1,0 +1,158 @@
+// Decode kernel arguments and the container casts / vector stores shared by the decode kernels.
+#pragma once
+
+#include "ep_common.hpp"
+
+namespace ep {
+
+struct DecodeArgs {
+  const uint16_t* payload;
+  uint64_t payload_words;
+  const uint32_t* offsets;
+  const uint32_t* states;
+  const float* scales;
+  const uint32_t* plan;     // header + tables
+  void* out;
+  int store_kind;
+  int vecs_per_row;
+  uint32_t row_magic;       // row = umulhi(v << row_pre, row_magic) >> row_shift
+  int row_shift;
+  int row_pre;
+  int64_t num_vectors;
+  int tile_vectors;
+  int num_tiles;
+  int* error;
+};
+
+__device__ __forceinline__ void flag_error(int* error, int code) { atomicCAS(error, 0, code); }
+
+// ---- container casts (format.py:153-168 / lattice_rans.cu:560-653 of the reference) -----------------------
+
+__device__ __forceinline__ uint32_t bf16_bits_rne(float v) {
+  const uint32_t bits = __float_as_uint(v);
+  return (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;      // finite input
+}
+
+__device__ __forceinline__ float clamp_bf16(float v) {
+  return __builtin_fminf(__builtin_fmaxf(v, -3.3895313892515355e38f), 3.3895313892515355e38f);
+}
+
+__device__ __forceinline__ uint32_t f16_bits(float v) {
+  const _Float16 h = static_cast<_Float16>(__builtin_fminf(__builtin_fmaxf(v, -65504.0f), 65504.0f));
+  return __builtin_bit_cast(unsigned short, h);
+}
+
+// Round-to-nearest-even float -> OCP fp8 after saturating to the largest finite value.
+template <int MBITS, int BIAS>
+__device__ __forceinline__ uint32_t fp8_bits(float v, float limit) {
+  const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+  float a = __builtin_fminf(__builtin_fabsf(v), limit);
+  const float min_normal = __uint_as_float(static_cast<uint32_t>(127 + 1 - BIAS) << 23);
+  if (!(a >= min_normal)) {
+    const float quantum = __uint_as_float(static_cast<uint32_t>(127 + 1 - BIAS - MBITS) << 23);
+    return sign | static_cast<uint32_t>(__builtin_rintf(a / quantum));
+  }
+  const uint32_t bits = __float_as_uint(a);
+  const int exponent = static_cast<int>(bits >> 23) - 127 + BIAS;
+  constexpr int kShift = 23 - MBITS;
+  const uint32_t mant = bits & 0x7FFFFFu;
+  uint32_t r = mant >> kShift;
+  const uint32_t rest = mant & ((1u << kShift) - 1u);
+  constexpr uint32_t kHalf = 1u << (kShift - 1);
+  r += (rest > kHalf) || (rest == kHalf && (r & 1u));
+  return sign | ((static_cast<uint32_t>(exponent) << MBITS) + r);
+}
+
+template <typename T>
+__device__ __forceinline__ T snap_integer(float v, float low, float high_exclusive) {
+  const float high = __uint_as_float(__float_as_uint(high_exclusive) - 1u);   // nextafter(high_exclusive, 0)
+  return static_cast<T>(__builtin_fminf(__builtin_fmaxf(__builtin_rintf(v), low), high));
+}
+
+// Writes the eight values of vector `vector` in any container kind.
+__device__ __forceinline__ void store_vector(void* out, int kind, int64_t vector, const float (&w)[8]) {
+  switch (kind) {
+    case EP_STORE_BF16: {
+      uint32_t p[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p[i] = bf16_bits_rne(clamp_bf16(w[2 * i])) | (bf16_bits_rne(clamp_bf16(w[2 * i + 1])) << 16);
+      reinterpret_cast<uint4*>(out)[vector] = make_uint4(p[0], p[1], p[2], p[3]);
+      break;
+    }
+    case EP_STORE_F16: {
+      uint32_t p[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p[i] = f16_bits(w[2 * i]) | (f16_bits(w[2 * i + 1]) << 16);
+      reinterpret_cast<uint4*>(out)[vector] = make_uint4(p[0], p[1], p[2], p[3]);
+      break;
+    }
+    case EP_STORE_F32: {
+      float4* dst = reinterpret_cast<float4*>(out) + vector * 2;
+      dst[0] = make_float4(w[0], w[1], w[2], w[3]);
+      dst[1] = make_float4(w[4], w[5], w[6], w[7]);
+      break;
+    }
+    case EP_STORE_F8E4M3FN:
+    case EP_STORE_F8E5M2:
+    case EP_STORE_I8:
+    case EP_STORE_U8:
+    case EP_STORE_BOOL: {
+      uint32_t b[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (kind == EP_STORE_F8E4M3FN) b[i] = fp8_bits<3, 7>(w[i], 448.0f);
+        else if (kind == EP_STORE_F8E5M2) b[i] = fp8_bits<2, 15>(w[i], 57344.0f);
+        else if (kind == EP_STORE_I8) b[i] = static_cast<uint8_t>(snap_integer<int8_t>(w[i], -128.0f, 128.0f));
+        else if (kind == EP_STORE_U8) b[i] = snap_integer<uint8_t>(w[i], 0.0f, 256.0f);
+        else b[i] = __builtin_rintf(w[i]) != 0.0f;
+      }
+      reinterpret_cast<uint2*>(out)[vector] =
+          make_uint2(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24), b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
+      break;
+    }
+    case EP_STORE_I16:
+    case EP_STORE_U16: {
+      uint32_t b[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        b[i] = kind == EP_STORE_I16 ? static_cast<uint16_t>(snap_integer<int16_t>(w[i], -32768.0f, 32768.0f))
+                                    : snap_integer<uint16_t>(w[i], 0.0f, 65536.0f);
+      }
+      reinterpret_cast<uint4*>(out)[vector] =
+          make_uint4(b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16));
+      break;
+    }
+    case EP_STORE_I32:
+    case EP_STORE_U32: {
+      uint32_t b[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        b[i] = kind == EP_STORE_I32 ? static_cast<uint32_t>(snap_integer<int32_t>(w[i], -2147483648.0f, 2147483648.0f))
+                                    : snap_integer<uint32_t>(w[i], 0.0f, 4294967296.0f);
+      }
+      uint4* dst = reinterpret_cast<uint4*>(out) + vector * 2;
+      dst[0] = make_uint4(b[0], b[1], b[2], b[3]);
+      dst[1] = make_uint4(b[4], b[5], b[6], b[7]);
+      break;
+    }
+    default: {   // EP_STORE_I64 / EP_STORE_U64
+      uint64_t* dst = reinterpret_cast<uint64_t*>(out) + vector * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        dst[i] = kind == EP_STORE_I64
+                     ? static_cast<uint64_t>(snap_integer<int64_t>(w[i], -9223372036854775808.0f, 9223372036854775808.0f))
+                     : snap_integer<uint64_t>(w[i], 0.0f, 18446744073709551616.0f);
+      }
+      break;
+    }
+  }
+}
+
+__device__ __forceinline__ uint32_t row_of(const DecodeArgs& a, uint32_t vector) {
+  return __umulhi(vector << a.row_pre, a.row_magic) >> a.row_shift;
+}
+
+// Launches the LDS-table decode kernel (ep_decode_lds.hip) for an EP_TABLE_LDS_* plan.
+int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int num_pairs, hipStream_t stream);
+
+}  // namespace ep
