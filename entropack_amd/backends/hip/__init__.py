@@ -60,7 +60,8 @@ _SIGNATURES = {
     "ep_hip_last_runtime_error": (ctypes.c_int, []),
     "ep_hip_device_query": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(DeviceInfo)]),
     "ep_hip_plan_describe": (ctypes.c_int, [
-        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(PlanDesc)]),
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.POINTER(PlanDesc)]),
     "ep_hip_plan_build": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(PlanDesc), ctypes.c_void_p, ctypes.c_void_p]),
     "ep_hip_decode_lattice": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

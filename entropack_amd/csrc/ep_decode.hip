@@ -165,8 +165,5 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   if (desc->table_kind != EP_TABLE_LDS_BYTE && desc->table_kind != EP_TABLE_LDS_WIDE) return EP_HIP_EINVAL;
   if (desc->prob_bits > 11) return EP_HIP_EINVAL;
 
-  if (tv * 9 + 64 >= 65536) {
-    return EP_HIP_EUNSUPPORTED;   // the LDS kernel keeps tile-relative payload positions in 16 bits
-  }
   return launch_lds_decode(args, *desc, pairs, s);
 }

@@ -332,7 +332,7 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
         const int64_t left = a.num_vectors - v0;
         s.vector0 = static_cast<uint32_t>(v0);
         s.count = static_cast<int>(left < a.tile_vectors ? left : a.tile_vectors);
-        if (word_begin > word_end || word_end > a.payload_words || word_end - word_begin > 65000u) {
+        if (word_begin > word_end || word_end > a.payload_words) {
           flag_error(a.error, EP_DECODE_BAD_OFFSETS);
           s.count = 0;
           word_begin = word_end = 0;

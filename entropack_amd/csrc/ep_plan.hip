@@ -115,10 +115,10 @@ int ep_hip_device_query(int device, ep_hip_device_info* info) {
   return info->is_gfx950 ? EP_HIP_OK : EP_HIP_ENODEVICE;
 }
 
-int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_freq, int prob_bits, int lds_limit_bytes,
-                         int force_kind, ep_hip_plan_desc* desc) {
+int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_freq, int prob_bits, int tile_elements,
+                         int lds_limit_bytes, int force_kind, ep_hip_plan_desc* desc) {
   if (meta == nullptr || desc == nullptr || (freq == nullptr && n_freq != 0)) return EP_HIP_EINVAL;
-  if (prob_bits < 9 || prob_bits > 15) return EP_HIP_EINVAL;
+  if (prob_bits < 9 || prob_bits > 15 || tile_elements <= 0) return EP_HIP_EINVAL;
   memset(desc, 0, sizeof(*desc));
   const int64_t size = int64_t{1} << prob_bits;
   int64_t cursor = 0;

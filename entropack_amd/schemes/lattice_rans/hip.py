@@ -53,7 +53,7 @@ def _plan_for(buffers: LatticeBuffers, info: dict) -> DecodePlan:
     caps = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device())
     status = lib.ep_hip_plan_describe(
         meta_host.ctypes.data, freq_host.ctypes.data if freq_host.size else None, freq_host.size, info["prob_bits"],
-        caps.lds_bytes_per_block, -1 if FORCE_TABLE_KIND is None else FORCE_TABLE_KIND, ctypes.byref(desc))
+        info["tile_elements"], caps.lds_bytes_per_block, -1 if FORCE_TABLE_KIND is None else FORCE_TABLE_KIND, ctypes.byref(desc))
     if status == _hip.EINVAL:
         raise ValueError("lattice_rans stream_meta / freq_tables are inconsistent (ranges, sums or coset stream)")
     _hip.check("ep_hip_plan_describe", status)

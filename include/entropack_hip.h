@@ -88,11 +88,13 @@ int ep_hip_device_query(int device, ep_hip_device_info* info);
 
 /* Chooses the table representation from host copies of the container's stream_meta (int32[17][4] =
  * n_symbols, sym_min, freq_offset, alphabet) and freq_tables (u16[n_freq]), and validates them (offsets
- * contiguous, every stream's frequencies sum to 2^prob_bits). Pure host code, no GPU needed.
+ * contiguous, every stream's frequencies sum to 2^prob_bits). Pure host code, no GPU needed. `tile_elements` is
+ * the container's layout[2] (must be positive).
  * Reference: _decode_plan's representation choice, entropack/schemes/lattice_rans/cuda.py:697-732.
  * `force_kind` < 0 lets the library choose; otherwise it must be a kind the container qualifies for. */
 int ep_hip_plan_describe(const int32_t* stream_meta_host, const uint16_t* freq_tables_host, size_t n_freq,
-                         int prob_bits, int lds_limit_bytes, int force_kind, ep_hip_plan_desc* desc);
+                         int prob_bits, int tile_elements, int lds_limit_bytes, int force_kind,
+                         ep_hip_plan_desc* desc);
 
 /* Builds the decode tables on the device, from the container's own device buffers, into `tables_dev`
  * (desc->table_bytes bytes, caller-allocated, 256-byte aligned). Asynchronous on `stream`.

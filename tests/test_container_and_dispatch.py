@@ -1,0 +1,218 @@
+"""Host logic that needs no GPU: container blob layout, configs, registry dispatch, the C-ABI surface, plan choice."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import entropack_amd as ep
+from entropack_amd import registry
+from entropack_amd.backends import hip as hip_backend
+from entropack_amd.compression.compressed_tensor import pack_quant_state, parse_quant_state
+from entropack_amd.schemes.config import validate_config
+from entropack_amd.schemes.lattice_rans import format as fmt
+from conftest import ROOT, Golden
+
+
+def _blob(golden):
+    return torch.from_numpy(golden.quant_state.copy())
+
+
+def test_blob_parses_to_the_reference_buffers(golden):
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    assert tuple(container.shape) == golden.shape
+    assert str(container.encoded_dtype) == "torch." + golden.dtype
+    assert container.compress_method == "lattice_rans" and not container.lossless
+    assert container.actual_bpp == pytest.approx(golden.actual_bpp, abs=0)
+    assert list(container.buffers) == list(fmt.PACKED_KEYS)
+    for key, expect in golden.buffers.items():
+        got = container.buffers[key]
+        assert got.dtype == fmt.BUFFER_DTYPES[key]
+        assert got.data_ptr() % 16 == 0 or got.numel() == 0            # every component starts 16-byte aligned
+        raw = got.contiguous().view(torch.uint8).numpy().reshape(-1) if got.numel() else np.zeros(0, np.uint8)
+        assert np.array_equal(raw, np.ascontiguousarray(expect).view(np.uint8).reshape(-1))
+    fmt.validate_packed(dict(container.buffers), golden.shape, container.encoded_dtype)
+
+
+def test_repacking_reproduces_the_reference_blob_byte_for_byte(golden):
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    again = pack_quant_state(container.header, container.buffers, container.shape, container.encoded_dtype)
+    assert torch.equal(again, container.entropack_quant_state)
+    header, start = parse_quant_state(again)
+    assert start % 16 == 0 and header["buffer_names"] == list(fmt.PACKED_KEYS)
+
+
+def test_state_dict_round_trip_and_sharing():
+    golden = Golden("c1_256x256_bf16_3p5")
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    state = container.state_dict()
+    assert list(state) == ["entropack_quant_state"] and state["entropack_quant_state"].dtype == torch.uint8
+    clone = ep.CompressedTensor.from_state_dict(state)
+    assert clone.entropack_quant_state.data_ptr() == container.entropack_quant_state.data_ptr()   # shares storage
+    assert ep.CompressedTensor.from_state_dict(container.state_dict("w"), "w").shape == container.shape
+    with pytest.raises(ValueError):
+        ep.CompressedTensor.from_state_dict({}, None)
+    as_f16 = container.to(torch.float16)
+    assert as_f16.dtype == torch.float16 and as_f16.encoded_dtype == torch.bfloat16
+    assert as_f16.entropack_quant_state.data_ptr() == container.entropack_quant_state.data_ptr()
+    independent = container.clone()
+    assert independent.entropack_quant_state.data_ptr() != container.entropack_quant_state.data_ptr()
+    with pytest.raises(RuntimeError):
+        container.requires_grad_(True)
+
+
+def test_torch_save_load_weights_only(tmp_path):
+    golden = Golden("ragged_66x200_bf16_4p0")
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    path = tmp_path / "ckpt.pt"
+    torch.save(container.state_dict(), path)
+    loaded = torch.load(path, weights_only=True)
+    back = ep.CompressedTensor.from_state_dict(loaded)
+    assert torch.equal(back.entropack_quant_state, container.entropack_quant_state)
+
+
+def test_malformed_blobs_are_rejected():
+    golden = Golden("low_64x512_bf16_2p0")
+    blob = _blob(golden)
+    with pytest.raises(TypeError):
+        ep.CompressedTensor.unpack(blob.to(torch.int8))
+    with pytest.raises(ValueError, match="too short"):
+        ep.CompressedTensor.unpack(blob[:4])
+    with pytest.raises(ValueError, match="truncated"):
+        ep.CompressedTensor.unpack(blob[:100])
+    with pytest.raises(ValueError):
+        ep.CompressedTensor.unpack(blob[:-16])                                  # last buffer cut short
+    with pytest.raises(ValueError, match="trailing"):
+        ep.CompressedTensor.unpack(torch.cat([blob, torch.zeros(16, dtype=torch.uint8)]))
+    header, _ = parse_quant_state(blob)
+    container = ep.CompressedTensor.unpack(blob)
+    fewer = {k: v for k, v in container.buffers.items() if k != "scales"}
+    with pytest.raises(ValueError, match="must be"):
+        ep.CompressedTensor({"compress_method": "lattice_rans"}, fewer, container.shape, torch.bfloat16)
+    with pytest.raises(KeyError):
+        ep.CompressedTensor({"compress_method": "nope"}, dict(container.buffers), container.shape, torch.bfloat16)
+    garbled = blob.clone()
+    garbled[8:12] = 0xFF
+    with pytest.raises(ValueError, match="invalid"):
+        ep.CompressedTensor.unpack(garbled)
+
+
+def test_validate_packed_catches_structural_damage():
+    golden = Golden("c1_256x256_bf16_3p5")
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    good = dict(container.buffers)
+    fmt.validate_packed(good, golden.shape, torch.bfloat16)
+    bad = dict(good, offsets=good["offsets"].clone())
+    bad["offsets"].view(torch.int32)[2] = 1
+    with pytest.raises(ValueError, match="monotone"):
+        fmt.validate_packed(bad, golden.shape, torch.bfloat16)
+    bad = dict(good, freq_tables=good["freq_tables"].clone())
+    bad["freq_tables"].view(torch.int16)[3] += 1
+    with pytest.raises(ValueError, match="sum"):
+        fmt.validate_packed(bad, golden.shape, torch.bfloat16)
+    bad = dict(good, scales=good["scales"].clone())
+    bad["scales"][5] = -1.0
+    with pytest.raises(ValueError, match="positive"):
+        fmt.validate_packed(bad, golden.shape, torch.bfloat16)
+    with pytest.raises(ValueError, match="columns"):
+        fmt.validate_packed(good, (256, 300), torch.bfloat16)
+
+
+def test_config_validation():
+    validate_config(ep.EntroPackLossyConfig())
+    validate_config(ep.EntroPackLossyConfig(target_bpp=2, prob_bits=0, tile_elements=None))
+    for bad in (dict(target_bpp=0.0), dict(target_bpp=12.0), dict(prob_bits=8), dict(tile_elements=0), dict(row_rdo_iterations=9)):
+        with pytest.raises(ValueError):
+            validate_config(ep.EntroPackLossyConfig(**bad))
+    for bad in (dict(target_bpp="4"), dict(target_bpp=True), dict(prob_bits=11.0), dict(l2_prefetch=1), dict(row_rdo_iterations=None)):
+        with pytest.raises(TypeError):
+            validate_config(ep.EntroPackLossyConfig(**bad))
+    assert registry.name_for_config(ep.EntroPackLossyConfig()) == "lattice_rans"
+    assert registry.name_for_config(ep.RawConfig()) == "raw"
+    scheme = registry.get_scheme("lattice_rans")
+    with pytest.raises(TypeError, match="Unknown"):
+        scheme.make_config({"bogus": 1})
+    assert fmt.recommended_tile_elements(2.0) == 32768 and fmt.recommended_tile_elements(4.0) == 16384
+    assert fmt.recommended_tile_elements(7.0) == 8192 and fmt.recommended_tile_elements(7.5) == 4096
+    assert fmt.resolve_prob_bits(None, 7.0) == (11, True) and fmt.resolve_prob_bits(0, 7.1) == (12, True)
+    assert fmt.resolve_prob_bits(13, 2.0) == (13, False)
+    assert fmt.vector_tile_elements(16384) == 1820 and fmt.vector_tile_elements(100) == 32
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")
+def test_without_a_gpu_every_decode_request_fails_loudly():
+    golden = Golden("zeros_16x64_bf16_4p0")
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    reason = registry.reason("hip")
+    assert reason is not None and "cuda" in reason.lower()
+    with pytest.raises(ep.DispatchError) as caught:
+        ep.decompress(container, ep.EntroPackLossyConfig(execution_backend="hip"))
+    assert "hip" in caught.value.reasons and caught.value.scheme == "lattice_rans"
+    with pytest.raises(ep.DispatchError) as caught:
+        ep.decompress(container, ep.EntroPackLossyConfig(execution_backend="cuda"))
+    assert caught.value.reasons == {"cuda": "not registered"}
+    with pytest.raises(RuntimeError, match="no CPU decoder"):                  # auto -> eager lane -> refuses to decode
+        ep.decompress(container, ep.EntroPackLossyConfig())
+    assert registry.select(registry.get_scheme("lattice_rans"), None, None) == "eager"
+
+
+def test_c_abi_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "entropack_hip.h")).read()
+    declared = sorted(set(re.findall(r"\b(ep_hip_[a-z0-9_]+)\s*\(", header)))
+    assert declared, "no entry points found in the header"
+    library = hip_backend.library()
+    assert library.ep_hip_abi_version() == hip_backend.ABI_VERSION
+    for name in declared:
+        assert hasattr(library, name), f"{name} is declared in include/entropack_hip.h but not exported"
+    assert sorted(hip_backend.EXPORTED_SYMBOLS) == declared
+    assert library.ep_hip_error_string(1) == b"invalid argument"
+
+
+def _describe(meta, freq, prob_bits, force=-1, lds=160 * 1024, tile_elements=16384):
+    desc = hip_backend.PlanDesc()
+    meta = np.ascontiguousarray(meta, dtype=np.int32)
+    freq = np.ascontiguousarray(freq, dtype=np.uint16)
+    status = hip_backend.library().ep_hip_plan_describe(
+        meta.ctypes.data, freq.ctypes.data if freq.size else None, freq.size, prob_bits, tile_elements, lds, force, ctypes.byref(desc))
+    return status, desc
+
+
+def test_plan_choice_is_pure_host_logic(golden):
+    prob_bits = int(golden.buffers["layout"][1])
+    status, desc = _describe(golden.buffers["stream_meta"], golden.buffers["freq_tables"], prob_bits,
+                             tile_elements=int(golden.buffers["layout"][2]))
+    assert status == hip_backend.OK
+    alphabets = golden.buffers["stream_meta"][:, 3]
+    assert desc.max_alphabet == alphabets.max() and desc.alphabet_sum == alphabets.sum() and desc.prob_bits == prob_bits
+    if prob_bits > 11:
+        assert desc.table_kind == hip_backend.TABLE_GLOBAL64 and desc.lds_bytes == 0
+        assert desc.table_bytes == 256 + 17 * (1 << prob_bits) * 8
+    else:
+        assert desc.table_kind in (hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE)
+        assert desc.table_bytes == 256 + 16 * (1 << prob_bits) * 4
+    if golden.name.startswith("huge_alpha"):
+        assert desc.table_kind == hip_backend.TABLE_LDS_WIDE          # a 769-symbol alphabet cannot use byte values
+    if golden.name.startswith("c1_"):
+        assert desc.table_kind == hip_backend.TABLE_LDS_BYTE
+
+
+def test_plan_describe_rejects_inconsistent_tables():
+    golden = Golden("c1_256x256_bf16_3p5")
+    meta, freq = golden.buffers["stream_meta"].copy(), golden.buffers["freq_tables"].copy()
+    assert _describe(meta, freq, 11)[0] == hip_backend.OK
+    assert _describe(meta, freq, 8)[0] == hip_backend.EINVAL
+    broken = freq.copy()
+    broken[4] += 1
+    assert _describe(meta, broken, 11)[0] == hip_backend.EINVAL                # sum != 2**11
+    shifted = meta.copy()
+    shifted[3, 2] += 1
+    assert _describe(shifted, freq, 11)[0] == hip_backend.EINVAL               # offsets not contiguous
+    assert _describe(meta, freq[:-1], 11)[0] == hip_backend.EINVAL
+    assert _describe(meta, freq, 11, lds=64 * 1024)[1].table_kind == hip_backend.TABLE_GLOBAL64
+    assert _describe(meta, freq, 11, force=hip_backend.TABLE_GLOBAL64)[1].table_kind == hip_backend.TABLE_GLOBAL64
+    assert _describe(meta, freq, 11, tile_elements=0)[0] == hip_backend.EINVAL
+    wide_only = Golden("huge_alpha_16x1024_bf16_7p0")
+    assert _describe(wide_only.buffers["stream_meta"], wide_only.buffers["freq_tables"], 11,
+                     force=hip_backend.TABLE_LDS_BYTE)[0] == hip_backend.EUNSUPPORTED

@@ -1,0 +1,69 @@
+"""The package's CPU encoder against the containers the reference encoder wrote: same input + config -> same bytes."""
+import numpy as np
+import pytest
+import torch
+
+import entropack_amd as ep
+from entropack_amd.schemes.lattice_rans import eager
+from conftest import Golden
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32, "int8": torch.int8}
+
+
+def _weight(golden):
+    dtype = _DTYPES[golden.dtype]
+    bits = torch.from_numpy(golden.weight_bits.copy())
+    return bits.view(torch.int8) if dtype == torch.int8 else bits.view(dtype)
+
+
+def test_compress_reproduces_the_reference_container(golden):
+    container = ep.compress(_weight(golden), ep.EntroPackLossyConfig(execution_backend="eager", **golden.config_kwargs))
+    assert container.compress_method == "lattice_rans"
+    assert torch.equal(container.entropack_quant_state, torch.from_numpy(golden.quant_state))
+    assert container.actual_bpp == golden.actual_bpp
+
+
+def test_config_1_rate_and_error_window():
+    """BASELINE config 1: 256x256 bf16 N(0, 0.02), seed 0, 3.5 bpp -> actual_bpp in [3.5, 3.6], rel-L2 near the
+    E8 high-rate closed form 1.1065 * 2**-R for the payload rate R (container overhead excluded)."""
+    golden = Golden("c1_256x256_bf16_3p5")
+    torch.manual_seed(0)
+    weight = (torch.randn(256, 256) * 0.02).to(torch.bfloat16)
+    assert np.array_equal(weight.view(torch.int16).numpy(), golden.weight_bits)
+    assert 3.5 <= golden.actual_bpp <= 3.6
+    restored = torch.from_numpy(golden.restored_bits.copy()).view(torch.bfloat16).float()
+    rel = ((restored - weight.float()).norm() / weight.float().norm()).item()
+    payload_rate = 8 * 2 * golden.buffers["payload"].size / weight.numel()
+    assert 0.9 * 1.1065 * 2 ** -payload_rate < rel < 1.35 * 1.1065 * 2 ** -payload_rate
+    assert 0.11 < rel < 0.14
+
+
+def test_hamilton_normalisation_properties():
+    rng = np.random.default_rng(1)
+    for size in (512, 2048):
+        for _ in range(20):
+            counts = rng.integers(0, 50, size=rng.integers(1, 60)).astype(np.int64)
+            counts[rng.integers(0, counts.size)] += 1
+            freq = eager.normalize_counts(counts, size).astype(np.int64)
+            assert freq.sum() == size
+            assert np.all((freq > 0) == (counts > 0))
+    skew = np.array([1] * 600 + [10 ** 6], dtype=np.int64)                  # deficit path: 601 symbols into 512 slots fails
+    with pytest.raises(ValueError):
+        eager.normalize_counts(skew, 512)
+    tight = np.array([1] * 500 + [10 ** 6], dtype=np.int64)
+    freq = eager.normalize_counts(tight, 512)
+    assert freq.sum() == 512 and freq[:500].tolist() == [1] * 500 and freq[500] == 12
+    with pytest.raises(ValueError):
+        eager.normalize_counts(np.zeros(4, dtype=np.int64), 512)
+
+
+def test_encoder_rejects_what_the_reference_rejects():
+    with pytest.raises(ValueError):
+        ep.registry.get_scheme("lattice_rans").encode(torch.zeros(4, 4, 4), ep.EntroPackLossyConfig(execution_backend="eager"))
+    with pytest.warns(ep.CompressionFallbackWarning):
+        raw = ep.compress(torch.tensor([[float("inf")] * 8]), ep.EntroPackLossyConfig(execution_backend="eager"))
+    assert raw.compress_method == "raw" and raw.header["requested"] == "lattice_rans"
+    with pytest.raises(TypeError):
+        ep.compress(raw, ep.EntroPackLossyConfig())
+    with pytest.warns(ep.CompressionFallbackWarning):
+        ep.compress(torch.randn(8, 16), ep.EntroPackLossyConfig(execution_backend="eager", row_rdo_iterations=1))
