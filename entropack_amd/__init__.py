@@ -4,12 +4,13 @@ Drop-in names: `compress`, `decompress`, `CompressedTensor`, `EntroPackLossyConf
 `CompressedINT8Linear`. Decoding runs on the `hip` backend only.
 """
 from .compression import CompressedTensor, CompressionFallbackWarning, compress, decompress
+from .linear import CompressedINT8Linear, CompressedLinear
 from .registry import DispatchError
 from .schemes import CompressionConfig, EntroPackLossyConfig, LatticeRANSConfig, RawConfig
 
 __version__ = "0.1.0"
 
 __all__ = [
-    "CompressedTensor", "CompressionConfig", "CompressionFallbackWarning", "DispatchError", "EntroPackLossyConfig",
+    "CompressedINT8Linear", "CompressedLinear", "CompressedTensor", "CompressionConfig", "CompressionFallbackWarning", "DispatchError", "EntroPackLossyConfig",
     "LatticeRANSConfig", "RawConfig", "__version__", "compress", "decompress",
 ]

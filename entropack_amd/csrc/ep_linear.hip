@@ -1,0 +1,289 @@
+// The consumers of decoded weights: MFMA GEMMs for gfx950 and the activation row quantiser.
+//
+//   gemm_bf16_nt_kernel   y[M,N] = x[M,K] . w[N,K]^T (+ bias[N]), bf16 operands, f32 accumulation in
+//                         v_mfma_f32_32x32x16_bf16, one bf16 rounding at the end (what F.linear does in the
+//                         reference's forward, entropack/linear/linear.py:163-165).
+//   gemm_i8_nt_kernel     y[M,N] = (a[M,K] . b[N,K]^T)_i32 -> f32 * sa[m] * sb[n] (+ bias[n]) -> out dtype, with
+//                         v_mfma_i32_32x32x32_i8 (semantics of the reference's Triton kernel,
+//                         entropack/linear/quant_kernels.py:15-54).
+//   quantize_rows_kernel  per row: scale = max(absmax / 127, eps_f32), code = clamp(rint(x / scale), +-127)
+//                         (entropack/linear/quant_kernels.py:56-79).
+//
+// Both GEMMs are "NT": each operand row is contiguous in K, which is exactly the MFMA fragment shape (a lane holds
+// 8 bf16 / 16 int8 consecutive in K of one row), so tiles go global -> LDS -> fragment with 16-byte accesses only.
+// Block tile 128 x 128 x 64 (bf16) or 128 x 128 x 128 (int8), 4 waves in a 2 x 2 arrangement, each wave 64 x 64 as
+// 2 x 2 MFMA tiles; the next K tile is fetched into registers while the current one is multiplied.
+#include "ep_common.hpp"
+
+namespace ep {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kBlockM = 128, kBlockN = 128;
+constexpr int kTileBytesK = 128;                 // bytes of K per tile row: 64 bf16 or 128 int8
+constexpr int kRowStride = kTileBytesK + 16;     // padded LDS row: 16-byte reads of 32 consecutive rows spread over banks
+constexpr int kChunksPerRow = kTileBytesK / 16;
+
+enum : int { kOutBF16 = 0, kOutF16 = 1, kOutF32 = 2 };
+
+__device__ __forceinline__ uint32_t bf16_bits_of(float v) {
+  typedef float float2v __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const float2v two = {v, 0.0f};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(two, bf16x2)) & 0xFFFFu;
+}
+
+__device__ __forceinline__ void store_out(void* y, int kind, int64_t at, float v) {
+  if (kind == kOutBF16) reinterpret_cast<uint16_t*>(y)[at] = static_cast<uint16_t>(bf16_bits_of(v));
+  else if (kind == kOutF16) reinterpret_cast<_Float16*>(y)[at] = static_cast<_Float16>(v);
+  else reinterpret_cast<float*>(y)[at] = v;
+}
+
+__device__ __forceinline__ float load_bias(const void* bias, int kind, int n) {
+  if (kind == kOutBF16) return __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(bias)[n]) << 16);
+  if (kind == kOutF16) return static_cast<float>(reinterpret_cast<const _Float16*>(bias)[n]);
+  return reinterpret_cast<const float*>(bias)[n];
+}
+
+// Shared skeleton. ELEM = bytes per operand element (2 = bf16, 1 = int8). Operand rows are `ld*` elements apart.
+template <int ELEM>
+struct TileLoader {
+  // Each of the 256 threads moves 4 chunks of 16 bytes per operand tile: chunk c covers row c / 8, bytes 16 (c % 8).
+  uint4 reg[4];
+
+  __device__ __forceinline__ void fetch(const uint8_t* base, int64_t ld_bytes, int row0, int rows, int64_t k_byte0,
+                                        int64_t k_bytes, int tid) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = tid + 256 * i;
+      const int r = chunk / kChunksPerRow;
+      const int64_t kb = k_byte0 + 16 * (chunk % kChunksPerRow);
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (row0 + r < rows && kb < k_bytes) v = *reinterpret_cast<const uint4*>(base + (row0 + r) * ld_bytes + kb);
+      reg[i] = v;
+    }
+  }
+
+  __device__ __forceinline__ void stash(uint8_t* tile, int tid) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = tid + 256 * i;
+      *reinterpret_cast<uint4*>(tile + (chunk / kChunksPerRow) * kRowStride + 16 * (chunk % kChunksPerRow)) = reg[i];
+    }
+  }
+};
+
+__global__ __launch_bounds__(256) void gemm_bf16_nt_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                           const void* __restrict__ bias, void* __restrict__ y, int M,
+                                                           int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
+                                                           int out_kind) {
+  __shared__ __align__(16) uint8_t tile_a[kBlockM * kRowStride];
+  __shared__ __align__(16) uint8_t tile_b[kBlockN * kRowStride];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int m0 = blockIdx.y * kBlockM, n0 = blockIdx.x * kBlockN;
+  const uint8_t* xa = reinterpret_cast<const uint8_t*>(x);
+  const uint8_t* wb = reinterpret_cast<const uint8_t*>(w);
+  const int64_t k_bytes = static_cast<int64_t>(K) * 2;
+
+  f32x16 acc[2][2] = {};
+  TileLoader<2> la, lb;
+  la.fetch(xa, ldx * 2, m0, M, 0, k_bytes, tid);
+  lb.fetch(wb, ldw * 2, n0, N, 0, k_bytes, tid);
+  const int frag_row = lane & 31;
+  const int frag_k = (lane >> 5) * 16;             // byte offset of this lane's 8 bf16 inside a 16-element K step
+
+  for (int64_t kb = 0; kb < k_bytes; kb += kTileBytesK) {
+    __syncthreads();                                // everyone is done reading the previous tile
+    la.stash(tile_a, tid);
+    lb.stash(tile_b, tid);
+    __syncthreads();
+    if (kb + kTileBytesK < k_bytes) {               // fetch the next tile while this one is multiplied
+      la.fetch(xa, ldx * 2, m0, M, kb + kTileBytesK, k_bytes, tid);
+      lb.fetch(wb, ldw * 2, n0, N, kb + kTileBytesK, k_bytes, tid);
+    }
+#pragma unroll
+    for (int kk = 0; kk < kTileBytesK / 32; ++kk) {
+      bf16x8 fa[2], fb[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        fa[t] = *reinterpret_cast<const bf16x8*>(tile_a + (wave_m * 64 + t * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+        fb[t] = *reinterpret_cast<const bf16x8*>(tile_b + (wave_n * 64 + t * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // Accumulator layout of a 32 x 32 tile: register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wave_n * 64 + j * 32 + (lane & 31);
+      if (n >= N) continue;
+      const float b = bias != nullptr ? load_bias(bias, out_kind, n) : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wave_m * 64 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+        if (m < M) store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, acc[i][j][r] + b);
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void gemm_i8_nt_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ b,
+                                                         const float* __restrict__ scale_a, const float* __restrict__ scale_b,
+                                                         const void* __restrict__ bias, void* __restrict__ y, int M, int N,
+                                                         int K, int64_t lda, int64_t ldb, int64_t ldy, int out_kind) {
+  __shared__ __align__(16) uint8_t tile_a[kBlockM * kRowStride];
+  __shared__ __align__(16) uint8_t tile_b[kBlockN * kRowStride];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int m0 = blockIdx.y * kBlockM, n0 = blockIdx.x * kBlockN;
+  const uint8_t* pa = reinterpret_cast<const uint8_t*>(a);
+  const uint8_t* pb = reinterpret_cast<const uint8_t*>(b);
+  const int64_t k_bytes = K;
+
+  i32x16 acc[2][2] = {};
+  TileLoader<1> la, lb;
+  la.fetch(pa, lda, m0, M, 0, k_bytes, tid);
+  lb.fetch(pb, ldb, n0, N, 0, k_bytes, tid);
+  const int frag_row = lane & 31;
+  const int frag_k = (lane >> 5) * 16;             // this lane's 16 int8 inside a 32-element K step
+
+  for (int64_t kb = 0; kb < k_bytes; kb += kTileBytesK) {
+    __syncthreads();
+    la.stash(tile_a, tid);
+    lb.stash(tile_b, tid);
+    __syncthreads();
+    if (kb + kTileBytesK < k_bytes) {
+      la.fetch(pa, lda, m0, M, kb + kTileBytesK, k_bytes, tid);
+      lb.fetch(pb, ldb, n0, N, kb + kTileBytesK, k_bytes, tid);
+    }
+#pragma unroll
+    for (int kk = 0; kk < kTileBytesK / 32; ++kk) {
+      i32x4 fa[2], fb[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        fa[t] = *reinterpret_cast<const i32x4*>(tile_a + (wave_m * 64 + t * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+        fb[t] = *reinterpret_cast<const i32x4*>(tile_b + (wave_n * 64 + t * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wave_n * 64 + j * 32 + (lane & 31);
+      if (n >= N) continue;
+      const float sb = scale_b[n];
+      const bool has_bias = bias != nullptr;
+      const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wave_m * 64 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+        if (m < M) {
+          // int32 -> f32, times the activation row scale, times the weight row scale, plus bias: in that order,
+          // each a single rounded float operation.
+          float v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[m]), sb);
+          if (has_bias) v = __fadd_rn(v, bv);
+          store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, v);
+        }
+      }
+    }
+  }
+}
+
+// One block per row. in_kind: kOutBF16 / kOutF16 / kOutF32 naming the activation dtype.
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const void* __restrict__ x, int in_kind, int64_t ldx, int K,
+                                                            int8_t* __restrict__ codes, float* __restrict__ scales) {
+  __shared__ float partial[4];
+  const int64_t row = blockIdx.x;
+  auto value = [&](int k) -> float {
+    if (in_kind == kOutBF16) return __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(x)[row * ldx + k]) << 16);
+    if (in_kind == kOutF16) return static_cast<float>(reinterpret_cast<const _Float16*>(x)[row * ldx + k]);
+    return reinterpret_cast<const float*>(x)[row * ldx + k];
+  };
+  float top = 0.0f;
+  for (int k = threadIdx.x; k < K; k += blockDim.x) top = __builtin_fmaxf(top, __builtin_fabsf(value(k)));
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) top = __builtin_fmaxf(top, __shfl_xor(top, offset));
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = top;
+  __syncthreads();
+  top = __builtin_fmaxf(__builtin_fmaxf(partial[0], partial[1]), __builtin_fmaxf(partial[2], partial[3]));
+  const float scale = __builtin_fmaxf(top / 127.0f, 1.1920928955078125e-07f);
+  for (int k = threadIdx.x; k < K; k += blockDim.x) {
+    const float q = __builtin_fminf(__builtin_fmaxf(__builtin_rintf(value(k) / scale), -127.0f), 127.0f);
+    codes[row * K + k] = static_cast<int8_t>(q);
+  }
+  if (threadIdx.x == 0) scales[row] = scale;
+}
+
+static int out_kind_valid(int kind) { return kind == kOutBF16 || kind == kOutF16 || kind == kOutF32; }
+
+}  // namespace ep
+
+extern "C" {
+
+int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
+                     int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, void* stream) {
+  using namespace ep;
+  if (x_dev == nullptr || w_dev == nullptr || y_dev == nullptr) return EP_HIP_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return EP_HIP_EINVAL;
+  if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0) return EP_HIP_EINVAL;
+  if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
+  if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
+  hipLaunchKernelGGL(gemm_bf16_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(x_dev), static_cast<const uint16_t*>(w_dev), bias_dev, y_dev,
+                     static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), ldx, ldw, ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_a_dev, const float* scale_b_dev,
+                   const void* bias_dev, void* y_dev, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                   int64_t ldy, int out_kind, void* stream) {
+  using namespace ep;
+  if (a_dev == nullptr || b_dev == nullptr || scale_a_dev == nullptr || scale_b_dev == nullptr || y_dev == nullptr) return EP_HIP_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return EP_HIP_EINVAL;
+  if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0) return EP_HIP_EINVAL;
+  if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
+  if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
+  hipLaunchKernelGGL(gemm_i8_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a_dev, b_dev, scale_a_dev,
+                     scale_b_dev, bias_dev, y_dev, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), lda, ldb,
+                     ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K, int64_t ldx, int8_t* codes_dev,
+                         float* scales_dev, void* stream) {
+  using namespace ep;
+  if (x_dev == nullptr || codes_dev == nullptr || scales_dev == nullptr) return EP_HIP_EINVAL;
+  if (rows <= 0 || K <= 0 || rows > 0x7FFFFFFF || K > 0x7FFFFFFF || ldx < K || !out_kind_valid(in_kind)) return EP_HIP_EINVAL;
+  hipLaunchKernelGGL(quantize_rows_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     x_dev, in_kind, ldx, static_cast<int>(K), codes_dev, scales_dev);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,3 @@
+from .linear import CompressedINT8Linear, CompressedLinear, QuantizedLinear
+
+__all__ = ["CompressedINT8Linear", "CompressedLinear", "QuantizedLinear"]

@@ -1,0 +1,94 @@
+"""Python face of the HIP linear kernels (libentropack_hip.so): MFMA GEMMs and the activation row quantiser.
+
+Same call shapes as the reference's Triton wrappers (entropack/linear/quant_kernels.py:81-106). Everything runs on the
+tensors' device and torch's current stream; nothing here has a CPU or library fallback.
+"""
+import torch
+
+from ..backends import hip as _hip
+
+
+def _require_device(*tensors: torch.Tensor) -> torch.device:
+    device = tensors[0].device
+    if device.type != "cuda":
+        raise RuntimeError(f"the HIP linear kernels need device tensors, got {device}")
+    for tensor in tensors:
+        if tensor is not None and tensor.device != device:
+            raise ValueError("all operands must be on one device")
+    return device
+
+
+def _rows(tensor: torch.Tensor) -> torch.Tensor:
+    """2-D view with unit inner stride (copying only if the layout forces it)."""
+    flat = tensor.reshape(-1, tensor.shape[-1])
+    return flat if flat.stride(-1) == 1 and flat.data_ptr() % 16 == 0 and flat.stride(0) % 16 == 0 else flat.contiguous()
+
+
+def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x[..., K] @ weight[N, K].T (+ bias): bf16 operands, f32 accumulation on the matrix cores."""
+    device = _require_device(x, weight)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("gemm_bf16 takes bfloat16 operands")
+    out_dtype = out_dtype or x.dtype
+    flat, w = _rows(x), _rows(weight)
+    if w.shape[1] != flat.shape[1]:
+        raise ValueError(f"inner sizes differ: {flat.shape[1]} vs {w.shape[1]}")
+    rows, inner, outer = flat.shape[0], flat.shape[1], w.shape[0]
+    out = torch.empty(rows, outer, dtype=out_dtype, device=device)
+    if rows == 0:
+        return out.reshape(*x.shape[:-1], outer)
+    bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
+    with torch.cuda.device(device):
+        _hip.check("ep_hip_gemm_bf16", _hip.library().ep_hip_gemm_bf16(
+            flat.data_ptr(), w.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(),
+            rows, outer, inner, flat.stride(0), w.stride(0), out.stride(0), _hip.FLOAT_KINDS[out_dtype],
+            _hip.current_stream(device)))
+    return out.reshape(*x.shape[:-1], outer)
+
+
+def quantize_rows(tensor: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-row symmetric int8 codes and float32 scales of a [rows, K] activation."""
+    device = _require_device(tensor)
+    if tensor.dtype not in _hip.FLOAT_KINDS:
+        raise TypeError(f"quantize_rows takes bf16/f16/f32 activations, got {tensor.dtype}")
+    flat = tensor.reshape(-1, tensor.shape[-1])
+    if flat.stride(-1) != 1:
+        flat = flat.contiguous()
+    rows, inner = flat.shape
+    codes = torch.empty(rows, inner, dtype=torch.int8, device=device)
+    scale = torch.empty(rows, dtype=torch.float32, device=device)
+    if rows:
+        with torch.cuda.device(device):
+            _hip.check("ep_hip_quantize_rows", _hip.library().ep_hip_quantize_rows(
+                flat.data_ptr(), _hip.FLOAT_KINDS[tensor.dtype], rows, inner, flat.stride(0), codes.data_ptr(),
+                scale.data_ptr(), _hip.current_stream(device)))
+    return codes, scale
+
+
+def int8_gemm(activation: torch.Tensor, codes: torch.Tensor, activation_scale: torch.Tensor, weight_scale: torch.Tensor,
+              bias: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
+    """(activation[M, K] @ codes[N, K].T) in int32, times both row scales, plus bias, as `out_dtype`."""
+    device = _require_device(activation, codes, activation_scale, weight_scale)
+    if activation.dtype != torch.int8 or codes.dtype != torch.int8:
+        raise TypeError("int8_gemm takes int8 operands")
+    rows, inner = activation.shape
+    outer = codes.shape[0]
+    if codes.shape[1] != inner:
+        raise ValueError(f"inner sizes differ: {inner} vs {codes.shape[1]}")
+    a, b = activation, codes
+    if inner % 16:                                   # the int8 matrix-core step is 32 wide; rows must be 16-byte multiples
+        pad = 16 - inner % 16
+        a = torch.nn.functional.pad(a, (0, pad))
+        b = torch.nn.functional.pad(b, (0, pad))
+    a, b = _rows(a), _rows(b)
+    out = torch.empty(rows, outer, dtype=out_dtype, device=device)
+    if rows == 0:
+        return out
+    bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
+    with torch.cuda.device(device):
+        _hip.check("ep_hip_gemm_i8", _hip.library().ep_hip_gemm_i8(
+            a.data_ptr(), b.data_ptr(), activation_scale.float().contiguous().data_ptr(),
+            weight_scale.float().contiguous().data_ptr(), None if bias_ready is None else bias_ready.data_ptr(),
+            out.data_ptr(), rows, outer, a.shape[1], a.stride(0), b.stride(0), out.stride(0),
+            _hip.FLOAT_KINDS[out_dtype], _hip.current_stream(device)))
+    return out

@@ -116,6 +116,29 @@ int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, c
                           const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows,
                           int64_t cols_padded, int tile_elements, int32_t* error_dev, void* stream);
 
+/* Linear ---------------------------------------------------------------------------------------------------- */
+
+/* Element kinds of GEMM outputs, biases and quantiser inputs. */
+enum ep_hip_float_kind { EP_FLOAT_BF16 = 0, EP_FLOAT_F16 = 1, EP_FLOAT_F32 = 2 };
+
+/* y[M][N] = x[M][K] . w[N][K]^T (+ bias[N]): bf16 operands (rows ldx / ldw elements apart, 16-byte aligned, K a
+ * multiple of 8), f32 accumulation on the matrix cores, result and bias of kind `out_kind`.
+ * Reference: the F.linear call of CompressedLinear.forward, entropack/linear/linear.py:163-165. */
+int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
+                     int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, void* stream);
+
+/* y[M][N] = (a[M][K] . b[N][K]^T)_int32 -> f32 * scale_a[m] * scale_b[n] (+ bias[n]) -> out_kind. K a multiple of 16.
+ * Reference: int8_gemm / _int8_gemm_kernel, entropack/linear/quant_kernels.py:15-54,81-93. */
+int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_a_dev, const float* scale_b_dev,
+                   const void* bias_dev, void* y_dev, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                   int64_t ldy, int out_kind, void* stream);
+
+/* Per-row symmetric int8 quantisation of activations: scale = max(absmax / 127, FLT_EPSILON),
+ * code = clamp(rint(x / scale), -127, 127). codes_dev is [rows][K] contiguous.
+ * Reference: quantize_rows / _quantize_rows_kernel, entropack/linear/quant_kernels.py:56-79,95-106. */
+int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K, int64_t ldx, int8_t* codes_dev,
+                         float* scales_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

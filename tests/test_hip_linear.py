@@ -1,0 +1,176 @@
+"""GPU parity, part 3: the MFMA GEMMs, the row quantiser and the compressed linear layers."""
+import io
+
+import numpy as np
+import pytest
+import torch
+from torch.nn import functional as F
+
+import entropack_amd as ep
+from entropack_amd.linear import kernels
+
+pytestmark = pytest.mark.gpu
+REL_L2 = 1e-3          # tolerance BASELINE states for linear outputs (bf16 accumulate-order differences)
+
+
+def rel_l2(got, expect):
+    got, expect = got.double(), expect.double()
+    return ((got - expect).norm() / expect.norm().clamp_min(1e-30)).item()
+
+
+@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (1, 256, 512), (17, 100, 72), (130, 129, 264), (128, 8192, 1024)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
+    print("case", shape, with_bias, flush=True)
+    m, n, k = shape
+    torch.manual_seed(5)
+    x = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(n, k, device="cuda") * 0.02).to(torch.bfloat16)
+    b = (torch.randn(n, device="cuda") * 0.01).to(torch.bfloat16) if with_bias else None
+    got = kernels.gemm_bf16(x, w, b)
+    expect = x.float() @ w.float().T + (b.float() if with_bias else 0.0)
+    assert got.dtype == torch.bfloat16 and got.shape == (m, n)
+    assert rel_l2(got, expect) <= REL_L2
+    # one bf16 rounding of an f32-accumulated result: elementwise within half a bf16 ulp (+ accumulation noise) of fp32
+    assert (got.float() - expect).abs().max() <= 2.0 ** -8 * expect.abs().max() + 1e-6
+    as_f32 = kernels.gemm_bf16(x, w, b, out_dtype=torch.float32)
+    assert rel_l2(as_f32, expect) <= 1e-5
+
+
+def test_gemm_bf16_takes_strided_rows_and_batches():
+    torch.manual_seed(6)
+    big = torch.randn(64, 512, device="cuda").to(torch.bfloat16)
+    x = big[:, :256]                                   # row stride 512, 256 used
+    w = (torch.randn(96, 256, device="cuda") * 0.1).to(torch.bfloat16)
+    assert rel_l2(kernels.gemm_bf16(x, w, None), x.float() @ w.float().T) <= REL_L2
+    batched = torch.randn(3, 5, 256, device="cuda").to(torch.bfloat16)
+    out = kernels.gemm_bf16(batched, w, None)
+    assert out.shape == (3, 5, 96)
+    assert rel_l2(out, batched.float() @ w.float().T) <= REL_L2
+    with pytest.raises(TypeError):
+        kernels.gemm_bf16(x.float(), w, None)
+    with pytest.raises(ValueError):
+        kernels.gemm_bf16(x, w[:, :128], None)
+
+
+@pytest.mark.parametrize("rows,inner,dtype", [(4096, 3072, torch.bfloat16), (3, 1000, torch.float32), (1, 8, torch.float16), (257, 4100, torch.bfloat16)])
+def test_quantize_rows_is_exact(rows, inner, dtype):
+    torch.manual_seed(7)
+    x = (torch.randn(rows, inner, device="cuda") * 3).to(dtype)
+    x[0, :] = 0                                        # an all-zero row takes the epsilon scale
+    codes, scale = kernels.quantize_rows(x)
+    flat = x.float()
+    expect_scale = (flat.abs().amax(dim=1) / 127.0).clamp(min=torch.finfo(torch.float32).eps)
+    expect_codes = (flat / expect_scale.unsqueeze(1)).round().clamp(-127, 127).to(torch.int8)
+    assert torch.equal(scale, expect_scale)
+    assert torch.equal(codes, expect_codes)
+    assert codes[0].abs().max() == 0
+
+
+@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040)])
+def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
+    print("case", shape, flush=True)
+    m, n, k = shape
+    torch.manual_seed(8)
+    a = torch.randint(-127, 128, (m, k), device="cuda", dtype=torch.int8)
+    b = torch.randint(-127, 128, (n, k), device="cuda", dtype=torch.int8)
+    sa = torch.rand(m, device="cuda") * 0.05 + 1e-3
+    sb = torch.rand(n, device="cuda") * 0.01 + 1e-4
+    bias = (torch.randn(n, device="cuda") * 0.01).to(torch.bfloat16)
+    exact = (a.double() @ b.double().T)                # |sum| < 2^31 here, exact in float64
+    assert exact.abs().max() < 2 ** 31
+    product = exact.float()                             # int32 -> f32 conversion (round to nearest), as the kernel does
+    expect = product * sa.unsqueeze(1) * sb.unsqueeze(0)
+    got = kernels.int8_gemm(a, b, sa, sb, None, torch.float32)
+    assert torch.equal(got, expect)
+    with_bias = kernels.int8_gemm(a, b, sa, sb, bias.float(), torch.float32)
+    assert torch.equal(with_bias, expect + bias.float().unsqueeze(0))
+    as_bf16 = kernels.int8_gemm(a, b, sa, sb, bias, torch.bfloat16)
+    assert torch.equal(as_bf16, (expect + bias.float().unsqueeze(0)).to(torch.bfloat16))
+
+
+def _c3_layer(mode, rows=3072, cols=3072, cls=None, bpp=4.0):
+    torch.manual_seed(2)
+    weight = (torch.randn(rows, cols) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(rows) * 0.01).to(torch.bfloat16)
+    dense = torch.nn.Linear(cols, rows, dtype=torch.bfloat16)
+    dense.weight.data.copy_(weight)
+    dense.bias.data.copy_(bias)
+    cls = cls or ep.CompressedLinear
+    layer = cls.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=bpp), forward_mode=mode)
+    return layer.to("cuda"), weight, bias
+
+
+@pytest.mark.parametrize("mode", ["decode_then_gemm", "fused"])
+def test_compressed_linear_forward_config_3(mode):
+    """BASELINE config 3: W 3072x3072 @ 4 bpp, bias, X [4096, 3072]; output rel-L2 vs F.linear(x, W_dec, b) <= 1e-3."""
+    layer, weight, bias = _c3_layer(mode)
+    torch.manual_seed(2)
+    x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
+    y = layer(x)
+    decoded = layer.dequantize("cuda")
+    assert decoded.dtype == torch.bfloat16 and decoded.shape == (3072, 3072)
+    expect = F.linear(x.float(), decoded.float(), bias.cuda().float())
+    assert y.shape == (4096, 3072) and y.dtype == torch.bfloat16
+    assert rel_l2(y, expect) <= REL_L2
+    assert 0.05 < rel_l2(decoded.cpu(), weight) < 0.09           # ~7 % at 4 bpp (E8 high-rate closed form 6.9 %)
+    assert 3.9 < layer.compressed_bits < 4.1
+
+
+@pytest.mark.parametrize("m", [1, 16, 128])
+def test_compressed_linear_small_m_both_modes_agree(m):
+    layer_a, _, bias = _c3_layer("decode_then_gemm", rows=512, cols=2048)
+    layer_b, _, _ = _c3_layer("fused", rows=512, cols=2048)
+    torch.manual_seed(9)
+    x = torch.randn(2, m, 2048).to(torch.bfloat16).cuda()
+    expect = F.linear(x.float(), layer_a.dequantize("cuda").float(), bias.cuda().float())
+    for layer in (layer_a, layer_b):
+        y = layer(x)
+        assert y.shape == (2, m, 512)
+        assert rel_l2(y, expect) <= REL_L2
+
+
+@pytest.mark.parametrize("mode", ["decode_then_gemm", "fused"])
+def test_int8_linear_forward_matches_its_definition(mode):
+    layer, weight, bias = _c3_layer(mode, rows=1024, cols=1536, cls=ep.CompressedINT8Linear)
+    torch.manual_seed(3)
+    x = torch.randn(300, 1536).to(torch.bfloat16).cuda()
+    y = layer(x)
+    codes = layer.codes("cuda")
+    assert codes.dtype == torch.int8 and codes.shape == (1024, 1536)
+    flat = x.float()
+    sa = (flat.abs().amax(dim=1) / 127.0).clamp(min=torch.finfo(torch.float32).eps)
+    qa = (flat / sa.unsqueeze(1)).round().clamp(-127, 127)
+    expect = ((qa.double() @ codes.double().T).float() * sa.unsqueeze(1) * layer.weight_quant_scale.cuda().unsqueeze(0)
+              + bias.cuda().float().unsqueeze(0)).to(torch.bfloat16)
+    assert torch.equal(y, expect)
+    # and the quantised layer still approximates the dense one
+    assert rel_l2(y, F.linear(x.float(), weight.cuda().float(), bias.cuda().float())) < 0.15
+    assert layer.weight_quant_scale.dtype == torch.float32
+    layer.to(torch.float16)
+    assert layer.weight_quant_scale.dtype == torch.float32        # Module.to must not cast the row scales
+
+
+def test_state_dict_round_trip_through_torch_save():
+    """Usage/Linear-layers doc flow: save state_dict -> fresh layers -> torch.load(weights_only=True) -> same outputs."""
+    layer, _, _ = _c3_layer("decode_then_gemm", rows=256, cols=512)
+    model = torch.nn.Sequential(layer)
+    state = model.state_dict()
+    assert sorted(state) == ["0.bias", "0.weight.entropack_quant_state"]
+    assert state["0.weight.entropack_quant_state"].dtype == torch.uint8 and state["0.weight.entropack_quant_state"].ndim == 1
+    buffer = io.BytesIO()
+    torch.save(state, buffer)
+    buffer.seek(0)
+    loaded = torch.load(buffer, weights_only=True)
+    fresh = torch.nn.Sequential(ep.CompressedLinear(512, 256, config=ep.EntroPackLossyConfig(target_bpp=4.0), device="cuda"))
+    result = fresh.load_state_dict(loaded)
+    assert not result.missing_keys and not result.unexpected_keys
+    x = torch.randn(8, 512, device="cuda").to(torch.bfloat16)
+    assert torch.equal(fresh(x), model(x))
+    assert fresh[0].weight.device.type == "cuda"
+    empty = ep.CompressedLinear(512, 256, device="cuda")
+    with pytest.raises(RuntimeError, match="nothing to decode"):
+        empty(x)
+    wrong = ep.CompressedLinear(256, 512, device="cuda")
+    with pytest.raises(RuntimeError):
+        torch.nn.Sequential(wrong).load_state_dict(loaded)
