@@ -130,7 +130,7 @@ def test_full_size_target_8192x28672():
     for bpp in (4.0, 2.0, 8.0):
         print("case bpp", bpp, flush=True)
         container, used = decode_and_check(weight, target_bpp=bpp)
-        assert abs(container.actual_bpp - bpp) < 0.05
+        assert abs(container.actual_bpp - bpp) < 0.1
         on_gpu = container.to("cuda")
         first = ep.decompress(on_gpu, ep.EntroPackLossyConfig(execution_backend="hip"))
         second = ep.decompress(on_gpu, ep.EntroPackLossyConfig())          # "auto" resolves to hip on this box
