@@ -22,6 +22,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+#: HBM bytes per decode launch measured with two rocprofv3 --pmc runs of this script (FETCH_SIZE, scaled by the 2.0
+#: a plain 512 MiB copy calibrates it to, plus WRITE_SIZE, factor 1.0). Only the default workload has been measured.
+MEASURED_TRAFFIC_BYTES = {"target": 599_500_000}
+
 WORKLOADS = {
     # name: (rows, cols, sigma, seed, target_bpp, outliers)
     "target": (8192, 28672, 0.015, 4, 4.0, False),     # the shape/rate the 60 %-of-HBM target is quoted on
@@ -92,6 +96,49 @@ def python_loop_baseline(host, rows, cols_padded, alg_bytes, tiles_sampled=8):
             "sample": f"{take} of {tiles} tiles through the per-symbol Python loop, {seconds:.2f} s, scaled linearly in tiles"}
 
 
+MFMA_PEAK_BF16_TFLOPS = 2500.0
+
+
+def _median_ms(fn, steps, warmup=5):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for begin, end in events:
+        begin.record()
+        fn()
+        end.record()
+    torch.cuda.synchronize()
+    times = sorted(begin.elapsed_time(end) for begin, end in events)
+    return times[len(times) // 2]
+
+
+def linear_section(ep, steps):
+    """BASELINE config 3: W 3072x3072 @ 4 bpp + bias, X [4096, 3072] bf16, seed 2; whole forward (decode + GEMM)."""
+    from torch.nn import functional as F
+    torch.manual_seed(2)
+    dense = torch.nn.Linear(3072, 3072, dtype=torch.bfloat16)
+    dense.weight.data.copy_((torch.randn(3072, 3072) * 0.02).to(torch.bfloat16))
+    dense.bias.data.copy_((torch.randn(3072) * 0.01).to(torch.bfloat16))
+    x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
+    flops = 2.0 * 4096 * 3072 * 3072
+    out = {"workload": "CompressedLinear 3072x3072 @ 4.0 bpp + bias, X [4096, 3072] bf16, seed 2", "flops": flops}
+    reference = None
+    for mode in ("decode_then_gemm", "fused"):
+        layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
+        y = layer(x)
+        if reference is None:
+            weight = layer.dequantize("cuda")
+            reference = F.linear(x.float(), weight.float(), layer.bias.float()).to(torch.bfloat16).double()
+            decode_ms = _median_ms(lambda: layer.dequantize("cuda"), steps)
+            out["decode_ms"] = round(decode_ms, 5)
+        rel = ((y.double() - reference).norm() / reference.norm()).item()
+        ms = _median_ms(lambda: layer(x), steps)
+        out[mode] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2),
+                     "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5), "rel_l2_vs_f32_reference": rel}
+    return out
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -99,6 +146,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
+    parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
+    parser.add_argument("--copy-probe-mib", type=int, default=0,
+                        help="also run one plain device copy of this many MiB (calibrates FETCH_SIZE / WRITE_SIZE counters)")
     parser.add_argument("--table-kind", type=int, default=None, help="force an ep_hip_table_kind (debugging)")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -127,6 +177,13 @@ def main():
 
     def step():
         return hip_lane.decode(lattice, shape=(rows, cols), dtype=torch.bfloat16)
+
+    if args.copy_probe_mib:
+        probe = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=device)
+        probe.zero_()
+        torch.empty_like(probe).copy_(probe)          # reads and writes exactly copy_probe_mib MiB
+        torch.cuda.synchronize()
+        del probe
 
     for _ in range(max(args.warmup, 1)):
         dense = step()
@@ -164,10 +221,14 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9, 3), "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s", "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": None,
+            "unit": "GB/s", "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.table_kind is None else None,
             "kernel_ms_avg": round(kernel_avg_ms, 5), "kernel_ms_median": round(kernel_ms[len(kernel_ms) // 2], 5),
         },
     }
+
+    if not args.no_linear:
+        result["linear"] = linear_section(ep, args.steps)
 
     if not args.no_cpu:
         host = host_arrays(container.buffers)
