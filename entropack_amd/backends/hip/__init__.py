@@ -16,8 +16,8 @@ LIBRARY_PATH = os.path.join(_PACKAGE_DIR, "libentropack_hip.so")
 ABI_VERSION = 1
 
 OK, EINVAL, EUNSUPPORTED, ERUNTIME, ENODEVICE = range(5)
-TABLE_GLOBAL64, TABLE_LDS_BYTE, TABLE_LDS_WIDE = range(3)
-TABLE_KIND_NAMES = {TABLE_GLOBAL64: "global64", TABLE_LDS_BYTE: "lds_byte", TABLE_LDS_WIDE: "lds_wide"}
+TABLE_GLOBAL64, TABLE_LDS_BYTE, TABLE_LDS_WIDE, TABLE_LDS_RANK = range(4)
+TABLE_KIND_NAMES = {TABLE_GLOBAL64: "global64", TABLE_LDS_BYTE: "lds_byte", TABLE_LDS_WIDE: "lds_wide", TABLE_LDS_RANK: "lds_rank"}
 DECODE_ERRORS = {
     2: "a renormalisation read passed the start of a tile's payload (truncated or corrupt payload)",
     3: "a tile ended with unread payload words or a lane state other than 2**15 (corrupt payload, states or tables)",
@@ -43,6 +43,7 @@ class PlanDesc(ctypes.Structure):
     _fields_ = [
         ("table_kind", ctypes.c_int), ("prob_bits", ctypes.c_int), ("table_bytes", ctypes.c_size_t),
         ("lds_bytes", ctypes.c_int), ("max_alphabet", ctypes.c_int), ("alphabet_sum", ctypes.c_int),
+        ("present_offset", ctypes.c_int * 18),
     ]
 
 

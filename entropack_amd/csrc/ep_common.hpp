@@ -46,9 +46,25 @@ inline int tile_vectors_of(int tile_elements) {
   return v > 32 ? v : 32;
 }
 
+// LDS_RANK plan layout after the header: FB u32[P] | VAL i16[P] | RS {u32 bits, u32 count}[16][2^pb / 32], each part
+// starting on a multiple of 16 bytes and RS on a multiple of one stream's RS size (its base is OR-ed with word offsets).
+inline size_t rank_fb_bytes(int present) { return (static_cast<size_t>(present) * 4 + 15) / 16 * 16; }
+inline size_t rank_val_bytes(int present) { return (static_cast<size_t>(present) * 2 + 15) / 16 * 16; }
+inline size_t rank_rs_stream_bytes(int prob_bits) { return (size_t{1} << prob_bits) / 32 * 8; }
+inline size_t rank_rs_offset(int present, int prob_bits) {
+  const size_t unit = rank_rs_stream_bytes(prob_bits);
+  return (rank_fb_bytes(present) + rank_val_bytes(present) + unit - 1) / unit * unit;
+}
+inline size_t rank_table_bytes(int present, int prob_bits) {
+  return rank_rs_offset(present, prob_bits) + kFieldStreams * rank_rs_stream_bytes(prob_bits);
+}
+
 // LDS bytes the LDS-table decode kernel needs for `waves` wavefronts each carrying `ilp` tile pairs.
 inline int lds_decode_bytes(int prob_bits, int waves, int ilp) {
   return (kFieldStreams << prob_bits) * 4 + waves * ilp * 2 * kRingBytes + 256;
+}
+inline int lds_rank_decode_bytes(int present, int prob_bits, int waves) {
+  return static_cast<int>((rank_table_bytes(present, prob_bits) + 255) / 256 * 256) + waves * 2 * kRingBytes + 256;
 }
 
 }  // namespace ep

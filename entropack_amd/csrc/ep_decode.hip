@@ -140,6 +140,7 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   args.tile_vectors = tv;
   args.num_tiles = static_cast<int>(tiles);
   args.error = error_dev;
+  args.lut_bytes = args.rank_val_offset = args.rank_rs_offset = 0;
   // row = floor(v / d) for v < 2^31 as umulhi(v, ceil(2^p / d)) >> (p - 32), p = 31 + ceil(log2 d), d >= 2.
   // d == 1 is handled as floor(2 v / 2): umulhi(2 v, 2^31) is exact for every 32-bit 2 v.
   {
@@ -161,6 +162,14 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
     hipLaunchKernelGGL(decode_global64_kernel, dim3(blocks), dim3(waves_per_block * 64), 0, s, args);
     EP_HIP_TRY(hipGetLastError());
     return EP_HIP_OK;
+  }
+  if (desc->table_kind == EP_TABLE_LDS_RANK) {
+    const int present = desc->present_offset[kStreams];
+    if (present < 0 || present > 65535 || desc->lds_bytes != static_cast<int>(rank_table_bytes(present, desc->prob_bits))) return EP_HIP_EINVAL;
+    args.lut_bytes = static_cast<uint32_t>(desc->lds_bytes);
+    args.rank_val_offset = static_cast<uint32_t>(rank_fb_bytes(present));
+    args.rank_rs_offset = static_cast<uint32_t>(rank_rs_offset(present, desc->prob_bits));
+    return launch_lds_decode(args, *desc, pairs, s);
   }
   if (desc->table_kind != EP_TABLE_LDS_BYTE && desc->table_kind != EP_TABLE_LDS_WIDE) return EP_HIP_EINVAL;
   if (desc->prob_bits > 11) return EP_HIP_EINVAL;

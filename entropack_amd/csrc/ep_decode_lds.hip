@@ -23,8 +23,11 @@
 
 namespace ep {
 
-template <int PB, bool WIDE>
+constexpr int kModeByte = 0, kModeWide = 1, kModeRank = 2;
+
+template <int PB, int MODE>
 struct Layout {
+  static constexpr bool WIDE = MODE == kModeWide;
   static constexpr uint32_t kTable = 1u << PB;
   static constexpr uint32_t kTableBytes = 4u << PB;             // one stream's table
   static constexpr uint32_t kLutBytes = kFieldStreams * kTableBytes;
@@ -132,10 +135,10 @@ struct StepConsts {
   uint32_t f0s;      // wave-uniform
 };
 
-template <int PB, bool WIDE, bool MASKED>
+template <int PB, int MODE, bool MASKED>
 __device__ __forceinline__ void field_step_single(Pair& p, int field, uint32_t off, uint32_t cb, const StepConsts& k,
                                                   uint64_t valid) {
-  using L = Layout<PB, WIDE>;
+  using L = Layout<PB, MODE>;
   uint32_t t, h, d, e, na, nb;
   uint64_t sv;
   const uint32_t kslot = L::kSlotMask4, kring = 0xFEu;
@@ -167,10 +170,10 @@ __device__ __forceinline__ void field_step_single(Pair& p, int field, uint32_t o
   p.pos = pos;
 }
 
-template <int PB, bool WIDE, bool MASKED>
+template <int PB, int MODE, bool MASKED>
 __device__ __forceinline__ void field_step_dual(Pair& p0, Pair& p1, int field, uint32_t off, uint32_t cb0, uint32_t cb1,
                                                 const StepConsts& k, uint64_t valid) {
-  using L = Layout<PB, WIDE>;
+  using L = Layout<PB, MODE>;
   uint32_t t0, h0, d0, e0, t1, h1, d1, e1, na, nb;
   uint64_t sv, m0;
   const uint32_t kslot = L::kSlotMask4, kring = 0xFEu;
@@ -210,9 +213,9 @@ __device__ __forceinline__ void field_step_dual(Pair& p0, Pair& p1, int field, u
   p1.pos = pos1;
 }
 
-template <int PB, bool WIDE, bool MASKED>
+template <int PB, int MODE, bool MASKED>
 __device__ __forceinline__ void coset_step_single(Pair& p, const StepConsts& k, uint64_t valid) {
-  using L = Layout<PB, WIDE>;
+  using L = Layout<PB, MODE>;
   uint32_t t, h, d, cb, na, nb;
   uint64_t sv;
   const uint32_t kring = 0xFEu, f0s = k.f0s;
@@ -233,9 +236,9 @@ __device__ __forceinline__ void coset_step_single(Pair& p, const StepConsts& k, 
   p.pos = pos;
 }
 
-template <int PB, bool WIDE, bool MASKED>
+template <int PB, int MODE, bool MASKED>
 __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepConsts& k, uint64_t valid) {
-  using L = Layout<PB, WIDE>;
+  using L = Layout<PB, MODE>;
   uint32_t t0, h0, d0, cb0, t1, h1, d1, cb1, na, nb;
   uint64_t sv, m0;
   const uint32_t kring = 0xFEu, f0s = k.f0s;
@@ -264,12 +267,49 @@ __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepCo
   p1.pos = pos1;
 }
 
+// ---- rank/select tables (any prob_bits) ---------------------------------------------------------------------------
+//
+// A slot table of 2^PB entries per stream does not fit LDS beyond prob_bits 11, but the alphabet does. Per stream and
+// 32 slots the table keeps {bits, count}: bit b is set when slot 32 w + b is the last slot of its symbol, count is the
+// number of symbols (of all field streams before this one, plus this stream's) that end before slot 32 w. The symbol
+// of a slot is then count + popcount(bits below the slot): one 8-byte read, and a second read fetches that symbol's
+// freq | cdf << 16; its value (symbol + minimum, int16) is read off the critical path. The lookups are ordinary C++;
+// renormalisation is the same scalar vote as above.
+template <int PB, bool MASKED>
+__device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, uint32_t val0, const StepConsts& k,
+                                          bool valid_lane) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(3))) const u32x2* lds_u2;
+  typedef __attribute__((address_space(3))) const uint32_t* lds_u32;
+  typedef __attribute__((address_space(3))) const int16_t* lds_i16;
+  constexpr uint32_t kTable = 1u << PB;
+  const uint32_t x = p.x;
+  const uint32_t slot = x & (kTable - 1u);
+  const uint32_t word_at = (((x >> 5) & (kTable / 32u - 1u)) << 3) + rs_base;
+  const u32x2 rs = *reinterpret_cast<lds_u2>(static_cast<uintptr_t>(word_at));
+  const uint32_t index = static_cast<uint32_t>(__builtin_popcount(rs.x & ((1u << (x & 31u)) - 1u))) + rs.y;
+  const uint32_t fb = *reinterpret_cast<lds_u32>(static_cast<uintptr_t>(index << 2));
+  p.e[field] = static_cast<uint32_t>(static_cast<int32_t>(*reinterpret_cast<lds_i16>(static_cast<uintptr_t>((index << 1) + val0))));
+  const uint32_t next = __umul24(fb & 0xFFFFu, x >> PB) + slot - (fb >> 16);
+  p.x = (!MASKED || valid_lane) ? next : x;
+  uint32_t t, d, na, nb;
+  uint32_t pos = uniform(p.pos);
+  asm volatile(EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("0")
+               : [x0] "+v"(p.x), [pos0] "+s"(pos), [t0] "=&v"(t), [d0] "=&v"(d), [na] "=&s"(na), [nb] "=&s"(nb)
+               : [ring0] "v"(p.ring), [shv] "v"(k.shv)
+               : "vcc", "scc", "memory");
+  p.pos = pos;
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
-template <int PB, bool WIDE, int ILP, int KIND>
-__global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_pairs) {
+template <int PB, int MODE, int ILP, int KIND>
+__device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int num_pairs) {
   extern __shared__ __align__(16) uint8_t smem[];
-  using L = Layout<PB, WIDE>;
+  using L = Layout<PB, MODE>;
+  constexpr bool WIDE = MODE != kModeByte;      // symbols as integers (plus minima or already as values), not biased bytes
+  static_assert(MODE != kModeRank || ILP == 1, "the rank/select steps are single-pair");
+  const uint32_t lut_bytes = MODE == kModeRank ? (a.lut_bytes + 255u) / 256u * 256u : L::kLutBytes;
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
 
   const int waves = blockDim.x >> 6;
@@ -279,16 +319,17 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
   const int l32 = lane & 31;
   // Absolute LDS byte addresses: tables first (so that table bases have their low 13 bits clear), then the rings.
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr)smem));
-  const uint32_t rings0 = lds0 + L::kLutBytes;
+  const uint32_t rings0 = lds0 + lut_bytes;
   const uint32_t minima0 = rings0 + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes;
   auto lds_write32 = [](uint32_t at, uint32_t value) { *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(at)) = value; };
 
   {
     const uint4* src = reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.plan) + kHeaderBytes);
     uint4* dst = reinterpret_cast<uint4*>(smem);
-    for (uint32_t i = threadIdx.x; i < L::kLutBytes / 16; i += blockDim.x) dst[i] = src[i];
+    const uint32_t quads = (MODE == kModeRank ? a.lut_bytes : L::kLutBytes) / 16;
+    for (uint32_t i = threadIdx.x; i < quads; i += blockDim.x) dst[i] = src[i];
     if (threadIdx.x < kStreams) {
-      reinterpret_cast<int32_t*>(smem + L::kLutBytes + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes)[threadIdx.x] =
+      reinterpret_cast<int32_t*>(smem + lut_bytes + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes)[threadIdx.x] =
           static_cast<int32_t>(a.plan[kHdrSymMin + threadIdx.x]);
     }
   }
@@ -302,7 +343,8 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
   k.f0s = uniform(a.plan[kHdrCosetFreq0]);
   k.f0v = k.f0s;
   k.f1v = L::kTable - k.f0s;
-  k.ktab = L::kTableBytes;
+  k.ktab = MODE == kModeRank ? (L::kTable / 32u) * 8u : L::kTableBytes;    // byte distance between a field's two cosets
+  const uint32_t rank_val0 = uniform(a.rank_val_offset), rank_rs0 = uniform(a.rank_rs_offset);
   k.shv = half ? 16u : 0u;
   // Keep the per-lane constants in vector registers (the steps name them as VGPR operands).
   asm volatile("" : "+v"(k.f0v), "+v"(k.f1v), "+v"(k.ktab), "+v"(k.shv));
@@ -401,7 +443,10 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
         const int32_t* minima = reinterpret_cast<const int32_t*>(smem + (minima0 - lds0)) + 1 + (c ? 1 : 0);
         int z[8];
 #pragma unroll
-        for (int f = 0; f < 8; ++f) z[f] = static_cast<int>(s.e[f] >> L::kSymShift) + minima[2 * f];
+        for (int f = 0; f < 8; ++f) {
+          if constexpr (MODE == kModeRank) z[f] = static_cast<int>(s.e[f]);
+          else z[f] = static_cast<int>(s.e[f] >> L::kSymShift) + minima[2 * f];
+        }
         const int parity = (z[0] + z[1] + z[2] + z[3] + z[4] + z[5] + z[6]) & 1;
         z[7] = 2 * z[7] + parity;
         const float shift = c ? 0.5f : 0.0f;
@@ -445,8 +490,8 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
         vector[j] = st[j].vector0 + static_cast<uint32_t>(offset) + l32;
         scale[j] = valid_lane ? a.scales[row_of(a, vector[j])] : 0.0f;
       }
-      if constexpr (ILP == 2) coset_step_dual<PB, WIDE, MASKED>(st[0], st[ILP - 1], k, valid);
-      else coset_step_single<PB, WIDE, MASKED>(st[0], k, valid);
+      if constexpr (ILP == 2) coset_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], k, valid);
+      else coset_step_single<PB, MODE, MASKED>(st[0], k, valid);
 #pragma unroll
       for (int j = 0; j < ILP; ++j) top_up(st[j]);
       uint32_t high[ILP];
@@ -454,11 +499,14 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
       for (int j = 0; j < ILP; ++j) high[j] = st[j].coset_base + L::kHighBase;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
-        if constexpr (ILP == 2) {
-          field_step_dual<PB, WIDE, MASKED>(st[0], st[ILP - 1], f, f & 3, f < 4 ? st[0].coset_base : high[0],
+        if constexpr (MODE == kModeRank) {
+          rank_step<PB, MASKED>(st[0], f, st[0].coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)),
+                                rank_val0, k, valid_lane);
+        } else if constexpr (ILP == 2) {
+          field_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], f, f & 3, f < 4 ? st[0].coset_base : high[0],
                                             f < 4 ? st[ILP - 1].coset_base : high[ILP - 1], k, valid);
         } else {
-          field_step_single<PB, WIDE, MASKED>(st[0], f, f & 3, f < 4 ? st[0].coset_base : high[0], k, valid);
+          field_step_single<PB, MODE, MASKED>(st[0], f, f & 3, f < 4 ? st[0].coset_base : high[0], k, valid);
         }
 #pragma unroll
         for (int j = 0; j < ILP; ++j) top_up(st[j]);
@@ -474,12 +522,17 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
       const uint64_t valid = __builtin_amdgcn_ballot_w64(valid_lane);
       const uint32_t vector = s.vector0 + static_cast<uint32_t>(offset) + l32;
       const float scale = valid_lane ? a.scales[row_of(a, vector)] : 0.0f;
-      coset_step_single<PB, WIDE, true>(s, k, valid);
+      coset_step_single<PB, MODE, true>(s, k, valid);
       top_up(s);
       const uint32_t high = s.coset_base + L::kHighBase;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
-        field_step_single<PB, WIDE, true>(s, f, f & 3, f < 4 ? s.coset_base : high, k, valid);
+        if constexpr (MODE == kModeRank) {
+          rank_step<PB, true>(s, f, s.coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)), rank_val0, k,
+                              valid_lane);
+        } else {
+          field_step_single<PB, MODE, true>(s, f, f & 3, f < 4 ? s.coset_base : high, k, valid);
+        }
         top_up(s);
       }
       if (valid_lane) emit(s, vector, scale);
@@ -535,11 +588,43 @@ __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_
   }
 }
 
+template <int PB, int MODE, int ILP, int KIND>
+__global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_pairs) {
+  decode_lds_body<PB, MODE, ILP, KIND>(a, num_pairs);
+}
+
+// The rank/select tables are small enough for two workgroups per CU; eight waves per SIMD need at most 64 registers.
+template <int PB, int KIND>
+__global__ __launch_bounds__(1024, 8) void decode_rank_kernel(DecodeArgs a, int num_pairs) {
+  decode_lds_body<PB, kModeRank, 1, KIND>(a, num_pairs);
+}
+
 // ---- host side -------------------------------------------------------------------------------------------------------
 
-template <int PB, bool WIDE, int ILP, int KIND>
+template <int PB, int KIND>
+static int launch_rank_one(const DecodeArgs& args, int num_pairs, int blocks, int threads, int lds, hipStream_t stream) {
+  auto kernel = decode_rank_kernel<PB, KIND>;
+  static thread_local int configured_for = -1;
+  int device = 0;
+  EP_HIP_TRY(hipGetDevice(&device));
+  if (configured_for != device) {
+    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    configured_for = device;
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), lds, stream, args, num_pairs);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+template <int PB>
+static int launch_rank_pb(const DecodeArgs& args, int num_pairs, int blocks, int threads, int lds, hipStream_t stream) {
+  return args.store_kind == EP_STORE_BF16 ? launch_rank_one<PB, EP_STORE_BF16>(args, num_pairs, blocks, threads, lds, stream)
+                                          : launch_rank_one<PB, -1>(args, num_pairs, blocks, threads, lds, stream);
+}
+
+template <int PB, int MODE, int ILP, int KIND>
 static int launch_one(const DecodeArgs& args, int num_pairs, int blocks, int threads, hipStream_t stream) {
-  auto kernel = decode_lds_kernel<PB, WIDE, ILP, KIND>;
+  auto kernel = decode_lds_kernel<PB, MODE, ILP, KIND>;
   const int lds = lds_decode_bytes(PB, threads / 64, ILP);
   static thread_local int configured_for = -1;     // per instantiation: raise the dynamic LDS cap once per device
   int device = 0;
@@ -553,15 +638,15 @@ static int launch_one(const DecodeArgs& args, int num_pairs, int blocks, int thr
   return EP_HIP_OK;
 }
 
-template <int PB, bool WIDE>
+template <int PB, int MODE>
 static int launch_pb(const DecodeArgs& args, int num_pairs, int blocks, int threads, int ilp, hipStream_t stream) {
   const bool bf16 = args.store_kind == EP_STORE_BF16;
   if (ilp == 2) {
-    return bf16 ? launch_one<PB, WIDE, 2, EP_STORE_BF16>(args, num_pairs, blocks, threads, stream)
-                : launch_one<PB, WIDE, 2, -1>(args, num_pairs, blocks, threads, stream);
+    return bf16 ? launch_one<PB, MODE, 2, EP_STORE_BF16>(args, num_pairs, blocks, threads, stream)
+                : launch_one<PB, MODE, 2, -1>(args, num_pairs, blocks, threads, stream);
   }
-  return bf16 ? launch_one<PB, WIDE, 1, EP_STORE_BF16>(args, num_pairs, blocks, threads, stream)
-              : launch_one<PB, WIDE, 1, -1>(args, num_pairs, blocks, threads, stream);
+  return bf16 ? launch_one<PB, MODE, 1, EP_STORE_BF16>(args, num_pairs, blocks, threads, stream)
+              : launch_one<PB, MODE, 1, -1>(args, num_pairs, blocks, threads, stream);
 }
 
 int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int pairs, hipStream_t stream) {
@@ -569,6 +654,27 @@ int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int 
   EP_HIP_TRY(hipGetDevice(&device));
   EP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
   if (cus <= 0) cus = 256;
+  if (desc.table_kind == EP_TABLE_LDS_RANK) {
+    // As many waves as fit: 16 per block, and two blocks per CU when two copies of the tables fit its 160 KiB.
+    const int present = desc.present_offset[kStreams];
+    const int resident = 2 * lds_rank_decode_bytes(present, desc.prob_bits, 16) <= 160 * 1024 ? 2 : 1;
+    int waves = (pairs + cus * resident - 1) / (cus * resident);
+    waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
+    int blocks = (pairs + waves - 1) / waves;
+    blocks = blocks > cus * resident ? cus * resident : blocks;
+    const int lds = lds_rank_decode_bytes(present, desc.prob_bits, waves);
+    const int threads = waves * 64;
+    switch (desc.prob_bits) {
+      case 9: return launch_rank_pb<9>(args, pairs, blocks, threads, lds, stream);
+      case 10: return launch_rank_pb<10>(args, pairs, blocks, threads, lds, stream);
+      case 11: return launch_rank_pb<11>(args, pairs, blocks, threads, lds, stream);
+      case 12: return launch_rank_pb<12>(args, pairs, blocks, threads, lds, stream);
+      case 13: return launch_rank_pb<13>(args, pairs, blocks, threads, lds, stream);
+      case 14: return launch_rank_pb<14>(args, pairs, blocks, threads, lds, stream);
+      case 15: return launch_rank_pb<15>(args, pairs, blocks, threads, lds, stream);
+      default: return EP_HIP_EINVAL;
+    }
+  }
   // One resident block per CU (the tables fill most of its LDS). Two interleaved pairs per wave once 16 waves on
   // every CU cannot hold all pairs at once; otherwise spread the pairs over as many CUs as possible.
   const int ilp = pairs > cus * 16 ? 2 : 1;
@@ -579,9 +685,9 @@ int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int 
   const bool wide = desc.table_kind == EP_TABLE_LDS_WIDE;
   const int threads = waves * 64;
   switch (desc.prob_bits) {
-    case 9: return wide ? launch_pb<9, true>(args, pairs, blocks, threads, ilp, stream) : launch_pb<9, false>(args, pairs, blocks, threads, ilp, stream);
-    case 10: return wide ? launch_pb<10, true>(args, pairs, blocks, threads, ilp, stream) : launch_pb<10, false>(args, pairs, blocks, threads, ilp, stream);
-    case 11: return wide ? launch_pb<11, true>(args, pairs, blocks, threads, ilp, stream) : launch_pb<11, false>(args, pairs, blocks, threads, ilp, stream);
+    case 9: return wide ? launch_pb<9, kModeWide>(args, pairs, blocks, threads, ilp, stream) : launch_pb<9, kModeByte>(args, pairs, blocks, threads, ilp, stream);
+    case 10: return wide ? launch_pb<10, kModeWide>(args, pairs, blocks, threads, ilp, stream) : launch_pb<10, kModeByte>(args, pairs, blocks, threads, ilp, stream);
+    case 11: return wide ? launch_pb<11, kModeWide>(args, pairs, blocks, threads, ilp, stream) : launch_pb<11, kModeByte>(args, pairs, blocks, threads, ilp, stream);
     default: return EP_HIP_EINVAL;
   }
 }

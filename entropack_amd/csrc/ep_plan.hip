@@ -12,10 +12,21 @@ void set_runtime_error(hipError_t e) { g_last_runtime_error = static_cast<int>(e
 
 // One block per stream. Threads split the alphabet into contiguous chunks, scan the chunk sums, then each
 // thread writes the slot entries of its own symbols, so slot ranges are disjoint and no atomics are needed.
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint4* __restrict__ p, size_t quads) {
+  for (size_t i = blockIdx.x * size_t{256} + threadIdx.x; i < quads; i += gridDim.x * size_t{256}) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+struct RankLayout {
+  int present_offset[18];
+  uint32_t val_offset;     // byte offsets inside the table area
+  uint32_t rs_offset;
+};
+
 __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __restrict__ meta,
                                                            const uint16_t* __restrict__ freq_tables, int kind,
-                                                           int prob_bits, uint32_t* __restrict__ plan) {
+                                                           int prob_bits, uint32_t* __restrict__ plan, RankLayout rank) {
   __shared__ uint32_t chunk_sum[256];
+  __shared__ uint32_t chunk_present[256];
   const int stream = blockIdx.x;
   const int tid = threadIdx.x;
   const uint32_t size = 1u << prob_bits;
@@ -41,21 +52,54 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
   const int per = (alphabet + 255) / 256;
   const int first = tid * per;
   const int last = first + per < alphabet ? first + per : alphabet;
-  uint32_t local = 0;
-  for (int s = first; s < last; ++s) local += freq[s];
+  uint32_t local = 0, local_present = 0;
+  for (int s = first; s < last; ++s) {
+    local += freq[s];
+    local_present += freq[s] != 0;
+  }
   chunk_sum[tid] = local;
+  chunk_present[tid] = local_present;
   __syncthreads();
   if (tid == 0) {
-    uint32_t running = 0;
+    uint32_t running = 0, seen = 0;
     for (int i = 0; i < 256; ++i) {
-      const uint32_t v = chunk_sum[i];
+      const uint32_t v = chunk_sum[i], n = chunk_present[i];
       chunk_sum[i] = running;
+      chunk_present[i] = seen;
       running += v;
+      seen += n;
     }
   }
   __syncthreads();
   uint32_t running = chunk_sum[tid];
   uint8_t* tables = reinterpret_cast<uint8_t*>(plan) + kHeaderBytes;
+  if (kind == EP_TABLE_LDS_RANK) {
+    // Symbol-end bitmap + running symbol count per 32 slots, and per present symbol freq | cdf << 16 and its value.
+    uint32_t* fb = reinterpret_cast<uint32_t*>(tables);
+    int16_t* val = reinterpret_cast<int16_t*>(tables + rank.val_offset);
+    uint32_t* rs = reinterpret_cast<uint32_t*>(tables + rank.rs_offset) + (static_cast<size_t>(stream - 1) << prob_bits) / 32 * 2;
+    uint32_t index = static_cast<uint32_t>(rank.present_offset[stream]) + chunk_present[tid];
+    for (int s = first; s < last; ++s) {
+      const uint32_t f = freq[s];
+      if (f == 0) continue;
+      fb[index] = f | (running << 16);
+      val[index] = static_cast<int16_t>(s + sym_min);
+      const uint32_t end = running + f - 1;
+      if (end < size) atomicOr(&rs[(end >> 5) * 2], 1u << (end & 31));
+      running += f;
+      ++index;
+    }
+    __threadfence_block();
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t before = static_cast<uint32_t>(rank.present_offset[stream]);
+      for (uint32_t w = 0; w < size / 32; ++w) {
+        rs[w * 2 + 1] = before;
+        before += __popc(rs[w * 2]);
+      }
+    }
+    return;
+  }
   for (int s = first; s < last; ++s) {
     const uint32_t f = freq[s];
     for (uint32_t d = 0; d < f && running + d < size; ++d) {
@@ -123,7 +167,8 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   const int64_t size = int64_t{1} << prob_bits;
   int64_t cursor = 0;
   int max_alphabet = 0;
-  bool byte_ok = true, wide_ok = true;
+  bool byte_ok = true, wide_ok = true, rank_ok = true;
+  int64_t present = 0;       // symbols with non-zero frequency in the field streams so far
   for (int s = 0; s < ep::kStreams; ++s) {
     const int64_t sym_min = meta[s * 4 + 1], off = meta[s * 4 + 2], alphabet = meta[s * 4 + 3];
     if (meta[s * 4 + 0] < 0 || alphabet < 0 || off != cursor || off + alphabet > static_cast<int64_t>(n_freq)) return EP_HIP_EINVAL;
@@ -140,8 +185,11 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
       } else {
         if (sym_min < -128 || sym_min + alphabet - 1 > 127) byte_ok = false;
         if (alphabet > 1024 || top > 2047) wide_ok = false;
+        if (sym_min < -32768 || sym_min + alphabet - 1 > 32767) rank_ok = false;
+        for (int64_t i = 0; i < alphabet; ++i) present += freq[off + i] != 0;
       }
     }
+    desc->present_offset[s + 1] = static_cast<int>(present);
     if (alphabet > max_alphabet) max_alphabet = static_cast<int>(alphabet);
     cursor += alphabet;
   }
@@ -149,15 +197,18 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   if (meta[0 * 4 + 3] == 0) return EP_HIP_EINVAL;
 
   const bool lds_fits = prob_bits <= 11 && ep::lds_decode_bytes(prob_bits, 1, 1) <= lds_limit_bytes;
+  rank_ok = rank_ok && present <= 65535 && ep::lds_rank_decode_bytes(static_cast<int>(present), prob_bits, 4) <= lds_limit_bytes;
   int kind = EP_TABLE_GLOBAL64;
   if (lds_fits && byte_ok) kind = EP_TABLE_LDS_BYTE;
   else if (lds_fits && wide_ok) kind = EP_TABLE_LDS_WIDE;
+  else if (rank_ok) kind = EP_TABLE_LDS_RANK;
   if (force_kind >= 0) {
     const bool allowed = force_kind == EP_TABLE_GLOBAL64 || (force_kind == EP_TABLE_LDS_BYTE && lds_fits && byte_ok) ||
-                         (force_kind == EP_TABLE_LDS_WIDE && lds_fits && wide_ok);
+                         (force_kind == EP_TABLE_LDS_WIDE && lds_fits && wide_ok) || (force_kind == EP_TABLE_LDS_RANK && rank_ok);
     if (!allowed) return EP_HIP_EUNSUPPORTED;
     kind = force_kind;
   }
+  if (kind != EP_TABLE_LDS_RANK) memset(desc->present_offset, 0, sizeof(desc->present_offset));
   desc->table_kind = kind;
   desc->prob_bits = prob_bits;
   desc->max_alphabet = max_alphabet;
@@ -165,6 +216,9 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   if (kind == EP_TABLE_GLOBAL64) {
     desc->table_bytes = ep::kHeaderBytes + (static_cast<size_t>(ep::kStreams) << prob_bits) * 8;
     desc->lds_bytes = 0;
+  } else if (kind == EP_TABLE_LDS_RANK) {
+    desc->lds_bytes = static_cast<int>(ep::rank_table_bytes(static_cast<int>(present), prob_bits));
+    desc->table_bytes = ep::kHeaderBytes + static_cast<size_t>(desc->lds_bytes);
   } else {
     desc->table_bytes = ep::kHeaderBytes + (static_cast<size_t>(ep::kFieldStreams) << prob_bits) * 4;
     desc->lds_bytes = (ep::kFieldStreams << prob_bits) * 4;
@@ -177,12 +231,28 @@ int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_table
   if (stream_meta_dev == nullptr || desc == nullptr || tables_dev == nullptr) return EP_HIP_EINVAL;
   if (freq_tables_dev == nullptr && desc->alphabet_sum != 0) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(tables_dev) % 256 != 0) return EP_HIP_EINVAL;
-  if (desc->prob_bits < 9 || desc->prob_bits > 15 || desc->table_kind < 0 || desc->table_kind > EP_TABLE_LDS_WIDE) return EP_HIP_EINVAL;
+  if (desc->prob_bits < 9 || desc->prob_bits > 15 || desc->table_kind < 0 || desc->table_kind > EP_TABLE_LDS_RANK) return EP_HIP_EINVAL;
+  if (desc->table_bytes < ep::kHeaderBytes || desc->table_bytes % 16 != 0) return EP_HIP_EINVAL;
+  ep::RankLayout rank = {};
+  if (desc->table_kind == EP_TABLE_LDS_RANK) {
+    const int present = desc->present_offset[ep::kStreams];
+    if (present < 0 || present > 65535 || desc->table_bytes != ep::kHeaderBytes + ep::rank_table_bytes(present, desc->prob_bits)) return EP_HIP_EINVAL;
+    for (int i = 0; i < 18; ++i) {
+      if (desc->present_offset[i] < 0 || desc->present_offset[i] > present) return EP_HIP_EINVAL;
+      rank.present_offset[i] = desc->present_offset[i];
+    }
+    rank.val_offset = static_cast<uint32_t>(ep::rank_fb_bytes(present));
+    rank.rs_offset = static_cast<uint32_t>(ep::rank_rs_offset(present, desc->prob_bits));
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // Slots of empty streams are never read, but keep the buffer deterministic.
-  EP_HIP_TRY(hipMemsetAsync(tables_dev, 0, desc->table_bytes, s));
+  // Slots of empty streams are never read, but keep the buffer deterministic; the rank form ORs into zeroed bitmaps.
+  // A fill kernel rather than a memset node, so the call can be captured into a graph.
+  const size_t quads = desc->table_bytes / 16;
+  hipLaunchKernelGGL(ep::zero_fill_kernel, dim3(static_cast<unsigned>((quads + 255) / 256 < 1024 ? (quads + 255) / 256 : 1024)),
+                     dim3(256), 0, s, static_cast<uint4*>(tables_dev), quads);
+  EP_HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(ep::build_tables_kernel, dim3(ep::kStreams), dim3(256), 0, s, stream_meta_dev, freq_tables_dev,
-                     desc->table_kind, desc->prob_bits, static_cast<uint32_t*>(tables_dev));
+                     desc->table_kind, desc->prob_bits, static_cast<uint32_t*>(tables_dev), rank);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }

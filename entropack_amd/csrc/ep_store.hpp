@@ -22,6 +22,9 @@ struct DecodeArgs {
   int tile_vectors;
   int num_tiles;
   int* error;
+  uint32_t lut_bytes;       // LDS_RANK: bytes of tables to stage, and where the value and rank/select parts start
+  uint32_t rank_val_offset;
+  uint32_t rank_rs_offset;
 };
 
 __device__ __forceinline__ void flag_error(int* error, int code) { atomicCAS(error, 0, code); }

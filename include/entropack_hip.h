@@ -44,7 +44,9 @@ enum ep_hip_store_kind {
 enum ep_hip_table_kind {
   EP_TABLE_GLOBAL64 = 0,    /* u64 per slot in HBM/L2, any prob_bits 9..15, any alphabet */
   EP_TABLE_LDS_BYTE = 1,    /* u32 per slot, LDS-resident; prob_bits <= 11, every field value in [-128, 127] */
-  EP_TABLE_LDS_WIDE = 2     /* u32 per slot, LDS-resident; prob_bits <= 11, alphabets <= 1024, frequencies < 2048 */
+  EP_TABLE_LDS_WIDE = 2,    /* u32 per slot, LDS-resident; prob_bits <= 11, alphabets <= 1024, frequencies < 2048 */
+  EP_TABLE_LDS_RANK = 3     /* LDS-resident rank/select form: per 32 slots a bitmap of symbol ends + running symbol count,
+                               per present symbol freq | cdf << 16 and an int16 value; any prob_bits whose tables fit LDS */
 };
 
 /* Device-side error flag values written (first one wins) to *error_dev by the decode kernels; same meaning as the
@@ -72,6 +74,8 @@ typedef struct ep_hip_plan_desc {
   int lds_bytes;              /* dynamic LDS the decode kernel will request (0 for GLOBAL64) */
   int max_alphabet;
   int alphabet_sum;
+  int present_offset[18];     /* LDS_RANK: symbols with non-zero frequency in field streams before stream s (index s),
+                                 [17] = their total; zero for the other kinds */
 } ep_hip_plan_desc;
 
 /* Library / device ------------------------------------------------------------------------------------------ */

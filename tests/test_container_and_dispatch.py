@@ -187,8 +187,20 @@ def test_plan_choice_is_pure_host_logic(golden):
     alphabets = golden.buffers["stream_meta"][:, 3]
     assert desc.max_alphabet == alphabets.max() and desc.alphabet_sum == alphabets.sum() and desc.prob_bits == prob_bits
     if prob_bits > 11:
-        assert desc.table_kind == hip_backend.TABLE_GLOBAL64 and desc.lds_bytes == 0
-        assert desc.table_bytes == 256 + 17 * (1 << prob_bits) * 8
+        # Slot tables of 2**prob_bits entries no longer fit LDS; the rank/select form indexes the present symbols.
+        assert desc.table_kind == hip_backend.TABLE_LDS_RANK
+        freq = golden.buffers["freq_tables"]
+        meta = golden.buffers["stream_meta"]
+        present = [int(np.count_nonzero(freq[meta[s, 2]:meta[s, 2] + meta[s, 3]])) for s in range(1, 17)]
+        assert list(desc.present_offset) == [0, 0] + list(np.cumsum(present))
+        total = sum(present)
+        rs_unit = (1 << prob_bits) // 32 * 8
+        rs_at = -(-(-(-total * 4 // 16) * 16 + -(-total * 2 // 16) * 16) // rs_unit) * rs_unit
+        assert desc.lds_bytes == rs_at + 16 * rs_unit and desc.table_bytes == 256 + desc.lds_bytes
+        status, forced = _describe(golden.buffers["stream_meta"], golden.buffers["freq_tables"], prob_bits,
+                                   force=hip_backend.TABLE_GLOBAL64)
+        assert status == hip_backend.OK and forced.lds_bytes == 0 and forced.table_bytes == 256 + 17 * (1 << prob_bits) * 8
+        assert not any(forced.present_offset)
     else:
         assert desc.table_kind in (hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE)
         assert desc.table_bytes == 256 + 16 * (1 << prob_bits) * 4
@@ -210,7 +222,8 @@ def test_plan_describe_rejects_inconsistent_tables():
     shifted[3, 2] += 1
     assert _describe(shifted, freq, 11)[0] == hip_backend.EINVAL               # offsets not contiguous
     assert _describe(meta, freq[:-1], 11)[0] == hip_backend.EINVAL
-    assert _describe(meta, freq, 11, lds=64 * 1024)[1].table_kind == hip_backend.TABLE_GLOBAL64
+    assert _describe(meta, freq, 11, lds=64 * 1024)[1].table_kind == hip_backend.TABLE_LDS_RANK
+    assert _describe(meta, freq, 11, lds=2 * 1024)[1].table_kind == hip_backend.TABLE_GLOBAL64
     assert _describe(meta, freq, 11, force=hip_backend.TABLE_GLOBAL64)[1].table_kind == hip_backend.TABLE_GLOBAL64
     assert _describe(meta, freq, 11, tile_elements=0)[0] == hip_backend.EINVAL
     wide_only = Golden("huge_alpha_16x1024_bf16_7p0")

@@ -13,7 +13,7 @@ from oracle import c_oracle
 pytestmark = pytest.mark.gpu
 
 _VIEW = {"bfloat16": torch.int16, "float16": torch.int16, "float32": torch.int32, "int8": torch.uint8}
-KINDS = [hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE]
+KINDS = [hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE, hip_backend.TABLE_LDS_RANK]
 
 
 def _container(golden, device="cuda"):
@@ -26,7 +26,7 @@ def _reset_force():
     hip_lane.FORCE_TABLE_KIND = None
 
 
-@pytest.mark.parametrize("kind", KINDS, ids=["global64", "lds_byte", "lds_wide"])
+@pytest.mark.parametrize("kind", KINDS, ids=["global64", "lds_byte", "lds_wide", "lds_rank"])
 @pytest.mark.parametrize("name", golden_names())
 def test_decompress_matches_reference_bits(name, kind):
     print(f"case {name} kind {kind}", flush=True)
@@ -51,9 +51,11 @@ def test_decompress_matches_reference_bits(name, kind):
 @pytest.mark.parametrize("name", ["outlier_128x256_bf16_4p0", "hi_96x512_bf16_8p0", "pb9_64x128_bf16_1p5"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.int8, torch.uint8, torch.int16,
                                    torch.int32, torch.int64, torch.bool, torch.float8_e4m3fn, torch.float8_e5m2])
-def test_every_store_kind_matches_oracle(name, dtype):
-    print(f"case {name} dtype {dtype}", flush=True)
+@pytest.mark.parametrize("kind", [None, hip_backend.TABLE_LDS_RANK], ids=["auto", "lds_rank"])
+def test_every_store_kind_matches_oracle(name, dtype, kind):
+    print(f"case {name} dtype {dtype} kind {kind}", flush=True)
     golden = Golden(name)
+    hip_lane.FORCE_TABLE_KIND = kind
     compressed = _container(golden)
     buffers = {k: v for k, v in compressed.buffers.items()}
     if dtype in (torch.int8, torch.uint8, torch.int16, torch.int32, torch.int64, torch.bool):
@@ -85,7 +87,7 @@ def test_every_store_kind_matches_oracle(name, dtype):
 
 def test_corrupt_payload_sets_the_error_flag_and_stays_in_bounds():
     golden = Golden("ragged_66x200_bf16_4p0")
-    for kind in (hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE):
+    for kind in (hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_RANK):
         hip_lane.FORCE_TABLE_KIND = kind
         compressed = _container(golden)
         buffers = dict(compressed.buffers)

@@ -68,7 +68,7 @@ def decode_and_check(weight, kinds=(None,), dtype=torch.bfloat16, **options):
     return container, used
 
 
-ALL_KINDS = (None, hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE)
+ALL_KINDS = (None, hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE, hip_backend.TABLE_LDS_RANK)
 
 
 def test_config_2_outliers_4096x4096():
@@ -84,7 +84,7 @@ def test_dit_like_layer_at_each_rate(bpp):
     print("case bpp", bpp, flush=True)
     container, used = decode_and_check(gauss(3, 3840, 3840), kinds=(None, hip_backend.TABLE_GLOBAL64), target_bpp=bpp)
     assert abs(container.actual_bpp - bpp) < 0.12
-    assert used[0] == ("global64" if bpp > 7.0 else "lds_byte")
+    assert used[0] == ("lds_rank" if bpp > 7.0 else "lds_byte")
 
 
 @pytest.mark.parametrize("shape", [(3840, 11520), (10240, 3840)])
