@@ -139,16 +139,113 @@ def linear_section(ep, steps):
     return out
 
 
+STACK_SHAPES = ((11520, 3840), (3840, 3840), (10240, 3840), (3840, 10240))      # qkv, out, ffn-up, ffn-down as [out, in]
+STACK_RATES = (2.3, 4.0, 5.0, 6.0, 8.0)
+
+
+def stack_workload(args, ep):
+    """BASELINE config 4: `--stack-blocks` blocks x 4 layers, N(0, 0.02) seed 3, rates round-robin; one pass decodes all."""
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    torch.manual_seed(3)
+    containers, params, alg_bytes, kinds, check = [], 0, 0, {}, []
+    started = time.perf_counter()
+    for index in range(args.stack_blocks * 4):
+        rows, cols = STACK_SHAPES[index % 4]
+        rate = STACK_RATES[index % 5]
+        weight = (torch.randn(rows, cols) * 0.02).to(torch.bfloat16)
+        container = ep.compress(weight, ep.EntroPackLossyConfig(target_bpp=rate, execution_backend="eager"))
+        params += rows * cols
+        layer_bytes = algorithmic_bytes(container.buffers, rows, int(container.buffers["layout"][0]), 2)
+        alg_bytes += layer_bytes
+        if index < 5 and not args.no_cpu:
+            check.append((index, host_arrays(container.buffers), rows, int(container.buffers["layout"][0]), layer_bytes))
+        containers.append(container.to(device))
+        if index % 10 == 9:
+            print(f"encoded {index + 1} layers, {time.perf_counter() - started:.0f} s", file=sys.stderr, flush=True)
+    encode_seconds = time.perf_counter() - started
+
+    config = ep.EntroPackLossyConfig(execution_backend="hip")
+    batch = ep.BatchDecompressor(containers, config)
+    arena = torch.empty(batch.arena_bytes, dtype=torch.uint8, device=device)
+    for container in containers:
+        lattice = LatticeBuffers(**{key: container.buffers[key] for key in LatticeBuffers._fields})
+        kind = hip_lane.plan_of(lattice).table_kind
+        kinds[kind] = kinds.get(kind, 0) + 1
+
+    def timed(fn, steps, warmup):
+        for _ in range(max(warmup, 1)):
+            out = fn()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        wall = time.perf_counter()
+        for begin, end in events:
+            begin.record()
+            out = fn()
+            end.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - wall) / steps
+        device_ms = sorted(begin.elapsed_time(end) for begin, end in events)
+        return out, wall, sum(device_ms) / len(device_ms)
+
+    steps = min(args.steps, 20)
+    dense, wall, device_ms = timed(lambda: batch(arena), steps, args.warmup)
+    batch.check_errors()
+    _, layer_wall, layer_ms = timed(lambda: [ep.decompress(c, config) for c in containers], max(2, steps // 4), 1)
+
+    result = {
+        "metric": "lossy decode GB/s (+% HBM roofline); CompressedLinear TFLOPS @ M=4096, 4 bpp",
+        "value": round(alg_bytes / wall / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"lattice_rans decode to bf16 of a DiT-like stack in one pass: {args.stack_blocks} blocks x "
+                        f"{{11520x3840, 3840x3840, 10240x3840, 3840x10240}} N(0,0.02) seed 3, rates {list(STACK_RATES)} round-robin",
+            "layers": len(containers), "params": params, "algorithmic_bytes": alg_bytes, "table_kinds": kinds,
+            "params_per_s": round(params / wall, 1), "encode_seconds_cpu": round(encode_seconds, 1),
+            "layer_by_layer": {"ms_per_pass": round(layer_wall * 1e3, 4), "device_ms": round(layer_ms, 4),
+                               "GBps": round(alg_bytes / layer_wall / 1e9, 3)},
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(alg_bytes / (device_ms * 1e-3) / 1e9, 3), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(alg_bytes / (device_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": None,
+            "kernel_ms_avg": round(device_ms, 5),
+        },
+    }
+    if check:
+        from oracle import c_oracle
+        c_oracle.load()
+        exact = True
+        cpu_seconds, cpu_bytes = 0.0, 0
+        for index, host, rows, cols_padded, layer_bytes in check:
+            begin = time.perf_counter()
+            expect = c_oracle.decode(host, (rows, cols_padded), "bfloat16", threads=min(16, os.cpu_count() or 1))
+            cpu_seconds += time.perf_counter() - begin
+            cpu_bytes += layer_bytes
+            got = dense[index].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+            exact = exact and bool(np.array_equal(got, expect[:, :got.shape[1]]))
+        result["config"]["bit_exact_vs_oracle_first_5_layers"] = exact
+        result["cpu_baseline"] = {
+            "value": round(cpu_bytes / cpu_seconds / 1e9, 4), "unit": "GB/s", "cores": min(16, os.cpu_count() or 1), "kind": "port",
+            "sample": f"the first 5 layers (one per rate), C port of the reference CPU decoder, OpenMP, {cpu_seconds:.2f} s"}
+    print(json.dumps(result))
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4"])
+    parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
     parser.add_argument("--copy-probe-mib", type=int, default=0,
                         help="also run one plain device copy of this many MiB (calibrates FETCH_SIZE / WRITE_SIZE counters)")
+    parser.add_argument("--prob-bits", type=int, default=None, help="encode with this prob_bits instead of the rate's default")
     parser.add_argument("--table-kind", type=int, default=None, help="force an ep_hip_table_kind (debugging)")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -159,10 +256,12 @@ def main():
     from entropack_amd.schemes.lattice_rans import hip as hip_lane
     from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
 
+    if args.workload == "c4":
+        return stack_workload(args, ep)
     rows, cols, sigma, seed, bpp, outliers = WORKLOADS[args.workload]
     started = time.perf_counter()
     weight = make_weight(rows, cols, sigma, seed, outliers)
-    config = ep.EntroPackLossyConfig(target_bpp=bpp, execution_backend="eager")
+    config = ep.EntroPackLossyConfig(target_bpp=bpp, execution_backend="eager", prob_bits=args.prob_bits)
     container = ep.compress(weight, config)
     encode_seconds = time.perf_counter() - started
     del weight
@@ -188,8 +287,7 @@ def main():
     for _ in range(max(args.warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
-    if not os.environ.get("EP_HIP_DEBUG"):
-        hip_lane.check_errors(lattice)
+    hip_lane.check_errors(lattice)
 
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     torch.cuda.synchronize()

@@ -3,7 +3,7 @@
 Drop-in names: `compress`, `decompress`, `CompressedTensor`, `EntroPackLossyConfig`, `CompressedLinear`,
 `CompressedINT8Linear`. Decoding runs on the `hip` backend only.
 """
-from .compression import CompressedTensor, CompressionFallbackWarning, compress, decompress
+from .compression import BatchDecompressor, CompressedTensor, CompressionFallbackWarning, compress, decompress, decompress_many
 from .linear import CompressedINT8Linear, CompressedLinear
 from .registry import DispatchError
 from .schemes import CompressionConfig, EntroPackLossyConfig, LatticeRANSConfig, RawConfig
@@ -11,6 +11,6 @@ from .schemes import CompressionConfig, EntroPackLossyConfig, LatticeRANSConfig,
 __version__ = "0.1.0"
 
 __all__ = [
-    "CompressedINT8Linear", "CompressedLinear", "CompressedTensor", "CompressionConfig", "CompressionFallbackWarning", "DispatchError", "EntroPackLossyConfig",
-    "LatticeRANSConfig", "RawConfig", "__version__", "compress", "decompress",
+    "BatchDecompressor", "CompressedINT8Linear", "CompressedLinear", "CompressedTensor", "CompressionConfig", "CompressionFallbackWarning", "DispatchError", "EntroPackLossyConfig",
+    "LatticeRANSConfig", "RawConfig", "__version__", "compress", "decompress", "decompress_many",
 ]

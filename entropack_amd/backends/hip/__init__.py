@@ -47,6 +47,17 @@ class PlanDesc(ctypes.Structure):
     ]
 
 
+class DecodeJob(ctypes.Structure):
+    """ep_hip_decode_job: one container of a batched decode."""
+    _fields_ = [
+        ("payload_dev", ctypes.c_void_p), ("payload_words", ctypes.c_uint64), ("offsets_dev", ctypes.c_void_p),
+        ("states_dev", ctypes.c_void_p), ("scales_dev", ctypes.c_void_p), ("tables_dev", ctypes.c_void_p),
+        ("desc", ctypes.POINTER(PlanDesc)), ("out_offset", ctypes.c_uint64), ("store_kind", ctypes.c_int),
+        ("tile_elements", ctypes.c_int), ("rows", ctypes.c_int64), ("cols_padded", ctypes.c_int64),
+        ("error_dev", ctypes.c_void_p),
+    ]
+
+
 class HipError(RuntimeError):
     """A C-ABI call returned a non-zero status."""
 
@@ -68,6 +79,9 @@ _SIGNATURES = {
         ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
         ctypes.POINTER(PlanDesc), ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_void_p]),
+    "ep_hip_batch_plan": (ctypes.c_int, [
+        ctypes.POINTER(DecodeJob), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_size_t)]),
+    "ep_hip_decode_lattice_batch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "ep_hip_gemm_bf16": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
         ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),

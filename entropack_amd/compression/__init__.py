@@ -1,4 +1,4 @@
-from .api import CompressionFallbackWarning, compress, decompress
+from .api import BatchDecompressor, CompressionFallbackWarning, compress, decompress, decompress_many
 from .compressed_tensor import CompressedTensor
 
-__all__ = ["CompressedTensor", "CompressionFallbackWarning", "compress", "decompress"]
+__all__ = ["BatchDecompressor", "CompressedTensor", "CompressionFallbackWarning", "compress", "decompress", "decompress_many"]

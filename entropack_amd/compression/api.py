@@ -49,3 +49,46 @@ def decompress(compressed: CompressedTensor, config: CompressionConfig) -> torch
     dense = compressed.scheme.decode(
         compressed.buffers, shape=tuple(compressed.shape), dtype=compressed.encoded_dtype, config=config)
     return dense.to(compressed.dtype)
+
+
+class BatchDecompressor:
+    """`decompress` for a whole list of `lattice_rans` containers (a model's layers) in one pass on the hip lane.
+
+    Planning happens once here; every call decodes all containers with a handful of launches and returns tensors with
+    the containers' shapes and dtypes, views into one output arena. The reference has no counterpart: its callers
+    decode layer by layer (entropack/linear/linear.py:125-130).
+    """
+
+    def __init__(self, containers, config: CompressionConfig):
+        from ..schemes.base import packed_buffers
+        from ..schemes.lattice_rans import hip as hip_lane
+        from ..schemes.lattice_rans.format import LatticeBuffers
+        validate_config(config)
+        if config.execution_backend not in (None, "auto", "hip"):
+            raise DispatchError(f"batched decode runs on the hip backend only, not {config.execution_backend!r}")
+        self._containers = list(containers)
+        items = []
+        for compressed in self._containers:
+            if compressed.compress_method != "lattice_rans":
+                raise ValueError(f"batched decode handles lattice_rans containers, got {compressed.compress_method!r}")
+            buffers = packed_buffers(compressed.buffers, LatticeBuffers)
+            items.append((buffers, tuple(compressed.shape), compressed.encoded_dtype))
+        self._decoder = hip_lane.BatchDecoder(items)
+        self.arena_bytes = self._decoder.arena_bytes
+
+    def __call__(self, arena: torch.Tensor | None = None) -> list[torch.Tensor]:
+        outputs = []
+        for compressed, dense in zip(self._containers, self._decoder.decode(arena)):
+            rows, cols = compressed.shape
+            if tuple(dense.shape) != (rows, cols):
+                dense = dense[:rows, :cols]
+            outputs.append(dense.to(compressed.dtype))
+        return outputs
+
+    def check_errors(self) -> None:
+        self._decoder.check_errors()
+
+
+def decompress_many(containers, config: CompressionConfig) -> list[torch.Tensor]:
+    """Decode every container of a list in one device pass; see `BatchDecompressor` to reuse the plan."""
+    return BatchDecompressor(containers, config)()

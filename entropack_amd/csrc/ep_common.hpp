@@ -63,8 +63,11 @@ inline size_t rank_table_bytes(int present, int prob_bits) {
 inline int lds_decode_bytes(int prob_bits, int waves, int ilp) {
   return (kFieldStreams << prob_bits) * 4 + waves * ilp * 2 * kRingBytes + 256;
 }
+inline int lds_rank_decode_bytes_of(int table_bytes, int waves) {
+  return (table_bytes + 255) / 256 * 256 + waves * 2 * kRingBytes + 256;
+}
 inline int lds_rank_decode_bytes(int present, int prob_bits, int waves) {
-  return static_cast<int>((rank_table_bytes(present, prob_bits) + 255) / 256 * 256) + waves * 2 * kRingBytes + 256;
+  return lds_rank_decode_bytes_of(static_cast<int>(rank_table_bytes(present, prob_bits)), waves);
 }
 
 }  // namespace ep

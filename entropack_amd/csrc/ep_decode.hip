@@ -9,6 +9,8 @@
 //   decode_lds_kernel (ep_decode_lds)  prob_bits <= 11: u32 slot table staged in LDS, payload streamed through an
 //                                      LDS ring.
 // Both produce bit-identical output.
+#include <string.h>
+
 #include "ep_store.hpp"
 
 namespace ep {
@@ -105,13 +107,15 @@ __global__ __launch_bounds__(256) void decode_global64_kernel(DecodeArgs a) {
 
 }  // namespace ep
 
-extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, const uint32_t* offsets_dev,
-                                     const uint32_t* states_dev, const float* scales_dev, const void* tables_dev,
-                                     const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows,
-                                     int64_t cols_padded, int tile_elements, int32_t* error_dev, void* stream) {
-  using namespace ep;
+namespace ep {
+
+// Validates one container's arguments and fills the kernels' argument block. `pairs` = wave-sized tile pairs.
+static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words, const uint32_t* offsets_dev,
+                            const uint32_t* states_dev, const float* scales_dev, const void* tables_dev,
+                            const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows, int64_t cols_padded,
+                            int tile_elements, int32_t* error_dev, DecodeArgs& args, int& pairs) {
   if (offsets_dev == nullptr || states_dev == nullptr || scales_dev == nullptr || tables_dev == nullptr ||
-      desc == nullptr || out_dev == nullptr || error_dev == nullptr) return EP_HIP_EINVAL;
+      desc == nullptr || error_dev == nullptr) return EP_HIP_EINVAL;
   if (payload_dev == nullptr && payload_words != 0) return EP_HIP_EINVAL;
   if (rows <= 0 || cols_padded <= 0 || cols_padded % 8 != 0 || tile_elements <= 0) return EP_HIP_EINVAL;
   if (store_kind < EP_STORE_F32 || store_kind > EP_STORE_BF16) return EP_HIP_EINVAL;
@@ -126,7 +130,6 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   const int64_t tiles = (vectors + tv - 1) / tv;
   if (vectors >= (int64_t{1} << 31) || tiles >= (int64_t{1} << 30)) return EP_HIP_EUNSUPPORTED;
 
-  DecodeArgs args;
   args.payload = payload_dev;
   args.payload_words = payload_words;
   args.offsets = offsets_dev;
@@ -153,26 +156,222 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
     args.row_shift = p - 32;
     args.row_pre = vecs_per_row > 1 ? 0 : 1;
   }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int pairs = static_cast<int>((tiles + 1) / 2);
+  pairs = static_cast<int>((tiles + 1) / 2);
 
-  if (desc->table_kind == EP_TABLE_GLOBAL64) {
-    const int waves_per_block = 4;
-    const int blocks = (pairs + waves_per_block - 1) / waves_per_block;
-    hipLaunchKernelGGL(decode_global64_kernel, dim3(blocks), dim3(waves_per_block * 64), 0, s, args);
-    EP_HIP_TRY(hipGetLastError());
+  switch (desc->table_kind) {
+    case EP_TABLE_GLOBAL64:
+      return EP_HIP_OK;
+    case EP_TABLE_LDS_RANK: {
+      const int present = desc->present_offset[kStreams];
+      if (present < 0 || present > 65535 || desc->lds_bytes != static_cast<int>(rank_table_bytes(present, desc->prob_bits))) return EP_HIP_EINVAL;
+      args.lut_bytes = static_cast<uint32_t>(desc->lds_bytes);
+      args.rank_val_offset = static_cast<uint32_t>(rank_fb_bytes(present));
+      args.rank_rs_offset = static_cast<uint32_t>(rank_rs_offset(present, desc->prob_bits));
+      return EP_HIP_OK;
+    }
+    case EP_TABLE_LDS_BYTE:
+    case EP_TABLE_LDS_WIDE:
+      return desc->prob_bits <= 11 ? EP_HIP_OK : EP_HIP_EINVAL;
+    default:
+      return EP_HIP_EINVAL;
+  }
+}
+
+static int launch_global64(const DecodeArgs& args, int pairs, hipStream_t s) {
+  const int waves_per_block = 4;
+  const int blocks = (pairs + waves_per_block - 1) / waves_per_block;
+  hipLaunchKernelGGL(decode_global64_kernel, dim3(blocks), dim3(waves_per_block * 64), 0, s, args);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+// ---- batch plan: a position-independent blob, identical on host and device -------------------------------------------
+
+constexpr uint32_t kBatchMagic = 0x45504254u;
+constexpr int kBatchMaxLaunches = 64;       // (table kind, prob_bits, bf16 or not) combinations, far below this in practice
+
+struct BatchLaunch {
+  LdsLaunch cfg;            // cfg.blocks = number of block jobs; for GLOBAL64: cfg.blocks = job index
+  int first_block;
+  int pairs;                // GLOBAL64 only
+};
+
+struct BatchHeader {
+  uint32_t magic;
+  int n_jobs;
+  int n_launches;
+  int n_blocks;
+  uint64_t args_offset;     // DecodeArgs[n_jobs]; `out` holds the byte offset into the arena
+  uint64_t blocks_offset;   // BlockJob[n_blocks]
+  uint64_t total_bytes;
+  BatchLaunch launches[kBatchMaxLaunches];
+};
+
+static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace ep
+
+extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, const uint32_t* offsets_dev,
+                                     const uint32_t* states_dev, const float* scales_dev, const void* tables_dev,
+                                     const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows,
+                                     int64_t cols_padded, int tile_elements, int32_t* error_dev, void* stream) {
+  using namespace ep;
+  if (out_dev == nullptr) return EP_HIP_EINVAL;
+  DecodeArgs args;
+  int pairs = 0;
+  const int status = fill_decode_args(payload_dev, payload_words, offsets_dev, states_dev, scales_dev, tables_dev, desc, out_dev,
+                                      store_kind, rows, cols_padded, tile_elements, error_dev, args, pairs);
+  if (status != EP_HIP_OK) return status;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (desc->table_kind == EP_TABLE_GLOBAL64) return launch_global64(args, pairs, s);
+  return launch_lds_decode(args, *desc, pairs, s);
+}
+
+extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int compute_units, void* blob_host, size_t* blob_bytes) {
+  using namespace ep;
+  if (jobs == nullptr || n_jobs <= 0 || blob_bytes == nullptr || compute_units <= 0) return EP_HIP_EINVAL;
+
+  struct Group { int table_kind, prob_bits, bf16, lut_bytes; int64_t pairs; };
+  Group groups[kBatchMaxLaunches];
+  int n_groups = 0;
+  auto group_of = [&](const ep_hip_plan_desc& d, int store_kind) {
+    const int bf16 = store_kind == EP_STORE_BF16;
+    for (int g = 0; g < n_groups; ++g) {
+      if (groups[g].table_kind == d.table_kind && groups[g].prob_bits == d.prob_bits && groups[g].bf16 == bf16) return g;
+    }
+    return -1;
+  };
+
+  // Pass 1: validate every job, count GLOBAL64 jobs (one launch each) and the pairs of each LDS group.
+  int n_global = 0;
+  for (int i = 0; i < n_jobs; ++i) {
+    const ep_hip_decode_job& j = jobs[i];
+    if (j.out_offset % 16 != 0) return EP_HIP_EINVAL;
+    DecodeArgs args;
+    int pairs = 0;
+    const int status = fill_decode_args(j.payload_dev, j.payload_words, j.offsets_dev, j.states_dev, j.scales_dev, j.tables_dev, j.desc,
+                                        nullptr, j.store_kind, j.rows, j.cols_padded, j.tile_elements, j.error_dev, args, pairs);
+    if (status != EP_HIP_OK) return status;
+    if (j.desc->table_kind == EP_TABLE_GLOBAL64) {
+      ++n_global;
+      continue;
+    }
+    int g = group_of(*j.desc, j.store_kind);
+    if (g < 0) {
+      if (n_groups == kBatchMaxLaunches) return EP_HIP_EUNSUPPORTED;
+      g = n_groups++;
+      groups[g] = {j.desc->table_kind, j.desc->prob_bits, j.store_kind == EP_STORE_BF16, 0, 0};
+    }
+    groups[g].pairs += pairs;
+    if (j.desc->lds_bytes > groups[g].lut_bytes) groups[g].lut_bytes = j.desc->lds_bytes;
+  }
+  if (n_groups + n_global > kBatchMaxLaunches) return EP_HIP_EUNSUPPORTED;
+
+  // Slice size per group: full blocks (16 waves x ilp pairs per round), about eight slices per resident block so the
+  // tail of the launch stays short whatever the mix of tile lengths.
+  LdsLaunch cfgs[kBatchMaxLaunches];
+  int slice[kBatchMaxLaunches];
+  for (int g = 0; g < n_groups; ++g) {
+    const int big = groups[g].pairs > 0x7FFFFFFF ? 0x7FFFFFFF : static_cast<int>(groups[g].pairs);
+    cfgs[g] = choose_lds_launch(groups[g].table_kind, groups[g].prob_bits, groups[g].lut_bytes, groups[g].bf16 != 0, big, compute_units);
+    const int per_round = (cfgs[g].threads / 64) * cfgs[g].ilp;
+    const int resident = lds_resident_blocks(groups[g].table_kind, groups[g].prob_bits, groups[g].lut_bytes) * compute_units;
+    int64_t rounds = groups[g].pairs / (static_cast<int64_t>(per_round) * resident * 8);
+    rounds = rounds < 1 ? 1 : (rounds > 64 ? 64 : rounds);
+    slice[g] = per_round * static_cast<int>(rounds);
+  }
+
+  // Pass 2: count (sizing) or emit block jobs.
+  int64_t n_blocks = 0;
+  for (int i = 0; i < n_jobs; ++i) {
+    const ep_hip_decode_job& j = jobs[i];
+    if (j.desc->table_kind == EP_TABLE_GLOBAL64) continue;
+    const int g = group_of(*j.desc, j.store_kind);
+    const int64_t vectors = j.rows * (j.cols_padded / 8);
+    const int tv = tile_vectors_of(j.tile_elements);
+    const int64_t pairs = ((vectors + tv - 1) / tv + 1) / 2;
+    n_blocks += (pairs + slice[g] - 1) / slice[g];
+  }
+  if (n_blocks > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
+  const size_t args_offset = align_up(sizeof(BatchHeader), 256);
+  const size_t blocks_offset = align_up(args_offset + sizeof(DecodeArgs) * static_cast<size_t>(n_jobs), 256);
+  const size_t total = align_up(blocks_offset + sizeof(BlockJob) * static_cast<size_t>(n_blocks > 0 ? n_blocks : 1), 256);
+  if (blob_host == nullptr) {
+    *blob_bytes = total;
     return EP_HIP_OK;
   }
-  if (desc->table_kind == EP_TABLE_LDS_RANK) {
-    const int present = desc->present_offset[kStreams];
-    if (present < 0 || present > 65535 || desc->lds_bytes != static_cast<int>(rank_table_bytes(present, desc->prob_bits))) return EP_HIP_EINVAL;
-    args.lut_bytes = static_cast<uint32_t>(desc->lds_bytes);
-    args.rank_val_offset = static_cast<uint32_t>(rank_fb_bytes(present));
-    args.rank_rs_offset = static_cast<uint32_t>(rank_rs_offset(present, desc->prob_bits));
-    return launch_lds_decode(args, *desc, pairs, s);
-  }
-  if (desc->table_kind != EP_TABLE_LDS_BYTE && desc->table_kind != EP_TABLE_LDS_WIDE) return EP_HIP_EINVAL;
-  if (desc->prob_bits > 11) return EP_HIP_EINVAL;
+  if (*blob_bytes < total) return EP_HIP_EINVAL;
 
-  return launch_lds_decode(args, *desc, pairs, s);
+  memset(blob_host, 0, total);
+  BatchHeader* header = static_cast<BatchHeader*>(blob_host);
+  DecodeArgs* args_out = reinterpret_cast<DecodeArgs*>(static_cast<uint8_t*>(blob_host) + args_offset);
+  BlockJob* blocks_out = reinterpret_cast<BlockJob*>(static_cast<uint8_t*>(blob_host) + blocks_offset);
+  header->magic = kBatchMagic;
+  header->n_jobs = n_jobs;
+  header->n_blocks = static_cast<int>(n_blocks);
+  header->args_offset = args_offset;
+  header->blocks_offset = blocks_offset;
+  header->total_bytes = total;
+  for (int i = 0; i < n_jobs; ++i) {
+    const ep_hip_decode_job& j = jobs[i];
+    int pairs = 0;
+    fill_decode_args(j.payload_dev, j.payload_words, j.offsets_dev, j.states_dev, j.scales_dev, j.tables_dev, j.desc, nullptr,
+                     j.store_kind, j.rows, j.cols_padded, j.tile_elements, j.error_dev, args_out[i], pairs);
+    args_out[i].out = reinterpret_cast<void*>(static_cast<uintptr_t>(j.out_offset));
+  }
+  int n_launches = 0, cursor = 0;
+  for (int g = 0; g < n_groups; ++g) {       // block jobs grouped by launch, containers in caller order inside a group
+    BatchLaunch& launch = header->launches[n_launches++];
+    launch.cfg = cfgs[g];
+    launch.first_block = cursor;
+    for (int i = 0; i < n_jobs; ++i) {
+      const ep_hip_decode_job& j = jobs[i];
+      if (j.desc->table_kind == EP_TABLE_GLOBAL64 || group_of(*j.desc, j.store_kind) != g) continue;
+      const int pairs = (args_out[i].num_tiles + 1) / 2;
+      for (int first = 0; first < pairs; first += slice[g]) {
+        BlockJob& b = blocks_out[cursor++];
+        b.job = i;
+        b.first_pair = first;
+        b.n_pairs = pairs - first < slice[g] ? pairs - first : slice[g];
+      }
+    }
+    launch.cfg.blocks = cursor - launch.first_block;      // threads and LDS stay as chosen for the group's total
+  }
+  for (int i = 0; i < n_jobs; ++i) {
+    if (jobs[i].desc->table_kind != EP_TABLE_GLOBAL64) continue;
+    BatchLaunch& launch = header->launches[n_launches++];
+    launch.cfg.table_kind = EP_TABLE_GLOBAL64;
+    launch.cfg.blocks = i;
+    launch.pairs = (args_out[i].num_tiles + 1) / 2;
+  }
+  header->n_launches = n_launches;
+  *blob_bytes = total;
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_decode_lattice_batch(const void* blob_host, const void* blob_dev, void* out_arena_dev, void* stream) {
+  using namespace ep;
+  if (blob_host == nullptr || blob_dev == nullptr || out_arena_dev == nullptr) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(out_arena_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(blob_dev) % 256 != 0) return EP_HIP_EINVAL;
+  const BatchHeader* header = static_cast<const BatchHeader*>(blob_host);
+  if (header->magic != kBatchMagic || header->n_launches < 0 || header->n_launches > kBatchMaxLaunches) return EP_HIP_EINVAL;
+  const DecodeArgs* args_host = reinterpret_cast<const DecodeArgs*>(static_cast<const uint8_t*>(blob_host) + header->args_offset);
+  const DecodeArgs* args_dev = reinterpret_cast<const DecodeArgs*>(static_cast<const uint8_t*>(blob_dev) + header->args_offset);
+  const BlockJob* blocks_dev = reinterpret_cast<const BlockJob*>(static_cast<const uint8_t*>(blob_dev) + header->blocks_offset);
+  uint8_t* arena = static_cast<uint8_t*>(out_arena_dev);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  for (int l = 0; l < header->n_launches; ++l) {
+    const BatchLaunch& launch = header->launches[l];
+    if (launch.cfg.table_kind == EP_TABLE_GLOBAL64) {
+      DecodeArgs args = args_host[launch.cfg.blocks];
+      args.out = arena + reinterpret_cast<uintptr_t>(args.out);
+      const int status = launch_global64(args, launch.pairs, s);
+      if (status != EP_HIP_OK) return status;
+      continue;
+    }
+    if (launch.cfg.blocks == 0) continue;
+    const int status = launch_lds(launch.cfg, args_host[0], 0, args_dev, blocks_dev + launch.first_block, arena, s);
+    if (status != EP_HIP_OK) return status;
+  }
+  return EP_HIP_OK;
 }

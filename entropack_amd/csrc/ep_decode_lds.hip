@@ -304,7 +304,7 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, 
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
 template <int PB, int MODE, int ILP, int KIND>
-__device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int num_pairs) {
+__device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_begin, int pair_end, int pair_stride) {
   extern __shared__ __align__(16) uint8_t smem[];
   using L = Layout<PB, MODE>;
   constexpr bool WIDE = MODE != kModeByte;      // symbols as integers (plus minima or already as values), not biased bytes
@@ -351,8 +351,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int num_pai
   const uint32_t* payload32 = reinterpret_cast<const uint32_t*>(a.payload);
   const uint64_t all_lanes = ~0ull;
 
-  const int stride = gridDim.x * waves * ILP;
-  for (int first_pair = (blockIdx.x * waves + wave) * ILP; first_pair < num_pairs; first_pair += stride) {
+  for (int first_pair = pair_begin + wave * ILP; first_pair < pair_end; first_pair += pair_stride) {
     Pair st[ILP];
     bool full = true;
 
@@ -367,7 +366,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int num_pai
       s.x = kStateMin;
       s.vector0 = 0;
       s.coset_base = 0;
-      if (first_pair + j < num_pairs && tile < a.num_tiles) {
+      if (first_pair + j < pair_end && tile < a.num_tiles) {
         word_begin = a.offsets[tile];
         word_end = a.offsets[tile + 1];
         const int64_t v0 = tile * a.tile_vectors;
@@ -588,65 +587,146 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int num_pai
   }
 }
 
+// One container spread over the whole grid.
 template <int PB, int MODE, int ILP, int KIND>
 __global__ __launch_bounds__(1024) void decode_lds_kernel(DecodeArgs a, int num_pairs) {
-  decode_lds_body<PB, MODE, ILP, KIND>(a, num_pairs);
+  const int per_block = static_cast<int>(blockDim.x >> 6) * ILP;
+  decode_lds_body<PB, MODE, ILP, KIND>(a, static_cast<int>(blockIdx.x) * per_block, num_pairs, static_cast<int>(gridDim.x) * per_block);
 }
 
 // The rank/select tables are small enough for two workgroups per CU; eight waves per SIMD need at most 64 registers.
 template <int PB, int KIND>
 __global__ __launch_bounds__(1024, 8) void decode_rank_kernel(DecodeArgs a, int num_pairs) {
-  decode_lds_body<PB, kModeRank, 1, KIND>(a, num_pairs);
+  const int per_block = static_cast<int>(blockDim.x >> 6);
+  decode_lds_body<PB, kModeRank, 1, KIND>(a, static_cast<int>(blockIdx.x) * per_block, num_pairs, static_cast<int>(gridDim.x) * per_block);
+}
+
+// Batch: each block decodes its slice of one of many containers. The argument block is read with every word made
+// wave-uniform, so that it lives in scalar registers exactly as kernel arguments do.
+__device__ __forceinline__ DecodeArgs load_job(const DecodeArgs* __restrict__ jobs, const BlockJob& mine, uint8_t* arena) {
+  static_assert(sizeof(DecodeArgs) % 4 == 0, "DecodeArgs is copied as 32-bit words");
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(jobs + uniform(static_cast<uint32_t>(mine.job)));
+  uint32_t words[sizeof(DecodeArgs) / 4];
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(DecodeArgs) / 4; ++i) words[i] = uniform(src[i]);
+  DecodeArgs a;
+  __builtin_memcpy(&a, words, sizeof(a));
+  a.out = arena + reinterpret_cast<uintptr_t>(a.out);       // batch jobs carry the byte offset of their output
+  return a;
+}
+
+template <int PB, int MODE, int ILP, int KIND>
+__global__ __launch_bounds__(1024) void decode_lds_batch_kernel(const DecodeArgs* __restrict__ jobs,
+                                                                const BlockJob* __restrict__ block_jobs, uint8_t* arena) {
+  const BlockJob mine = block_jobs[blockIdx.x];
+  const DecodeArgs a = load_job(jobs, mine, arena);
+  const int first = static_cast<int>(uniform(static_cast<uint32_t>(mine.first_pair)));
+  const int count = static_cast<int>(uniform(static_cast<uint32_t>(mine.n_pairs)));
+  decode_lds_body<PB, MODE, ILP, KIND>(a, first, first + count, static_cast<int>(blockDim.x >> 6) * ILP);
+}
+
+template <int PB, int KIND>
+__global__ __launch_bounds__(1024, 8) void decode_rank_batch_kernel(const DecodeArgs* __restrict__ jobs,
+                                                                    const BlockJob* __restrict__ block_jobs, uint8_t* arena) {
+  const BlockJob mine = block_jobs[blockIdx.x];
+  const DecodeArgs a = load_job(jobs, mine, arena);
+  const int first = static_cast<int>(uniform(static_cast<uint32_t>(mine.first_pair)));
+  const int count = static_cast<int>(uniform(static_cast<uint32_t>(mine.n_pairs)));
+  decode_lds_body<PB, kModeRank, 1, KIND>(a, first, first + count, static_cast<int>(blockDim.x >> 6));
 }
 
 // ---- host side -------------------------------------------------------------------------------------------------------
 
-template <int PB, int KIND>
-static int launch_rank_one(const DecodeArgs& args, int num_pairs, int blocks, int threads, int lds, hipStream_t stream) {
-  auto kernel = decode_rank_kernel<PB, KIND>;
-  static thread_local int configured_for = -1;
+template <typename Single, typename Batch>
+static int launch_configured(Single single, Batch batch, int* configured_for, const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs,
+                             const DecodeArgs* jobs, const BlockJob* block_jobs, uint8_t* arena, hipStream_t stream) {
   int device = 0;
   EP_HIP_TRY(hipGetDevice(&device));
-  if (configured_for != device) {
-    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    configured_for = device;
+  const int which = block_jobs != nullptr ? 1 : 0;
+  if (configured_for[which] != device) {      // per instantiation and thread: raise the dynamic LDS cap once per device
+    const void* function = which ? reinterpret_cast<const void*>(batch) : reinterpret_cast<const void*>(single);
+    EP_HIP_TRY(hipFuncSetAttribute(function, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    configured_for[which] = device;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), lds, stream, args, num_pairs);
+  if (which) hipLaunchKernelGGL(batch, dim3(cfg.blocks), dim3(cfg.threads), cfg.lds_bytes, stream, jobs, block_jobs, arena);
+  else hipLaunchKernelGGL(single, dim3(cfg.blocks), dim3(cfg.threads), cfg.lds_bytes, stream, args, num_pairs);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }
 
-template <int PB>
-static int launch_rank_pb(const DecodeArgs& args, int num_pairs, int blocks, int threads, int lds, hipStream_t stream) {
-  return args.store_kind == EP_STORE_BF16 ? launch_rank_one<PB, EP_STORE_BF16>(args, num_pairs, blocks, threads, lds, stream)
-                                          : launch_rank_one<PB, -1>(args, num_pairs, blocks, threads, lds, stream);
+template <int PB, int KIND>
+static int launch_rank_one(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs,
+                           const BlockJob* block_jobs, uint8_t* arena, hipStream_t stream) {
+  static thread_local int configured_for[2] = {-1, -1};
+  return launch_configured(decode_rank_kernel<PB, KIND>, decode_rank_batch_kernel<PB, KIND>, configured_for, cfg, args, num_pairs, jobs, block_jobs, arena, stream);
 }
 
 template <int PB, int MODE, int ILP, int KIND>
-static int launch_one(const DecodeArgs& args, int num_pairs, int blocks, int threads, hipStream_t stream) {
-  auto kernel = decode_lds_kernel<PB, MODE, ILP, KIND>;
-  const int lds = lds_decode_bytes(PB, threads / 64, ILP);
-  static thread_local int configured_for = -1;     // per instantiation: raise the dynamic LDS cap once per device
-  int device = 0;
-  EP_HIP_TRY(hipGetDevice(&device));
-  if (configured_for != device) {
-    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    configured_for = device;
-  }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), lds, stream, args, num_pairs);
-  EP_HIP_TRY(hipGetLastError());
-  return EP_HIP_OK;
+static int launch_one(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs,
+                      const BlockJob* block_jobs, uint8_t* arena, hipStream_t stream) {
+  static thread_local int configured_for[2] = {-1, -1};
+  return launch_configured(decode_lds_kernel<PB, MODE, ILP, KIND>, decode_lds_batch_kernel<PB, MODE, ILP, KIND>, configured_for, cfg, args, num_pairs, jobs, block_jobs, arena, stream);
+}
+
+#define EP_LAUNCH_ARGS cfg, args, num_pairs, jobs, block_jobs, arena, stream
+
+template <int PB>
+static int launch_rank_pb(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs,
+                          const BlockJob* block_jobs, uint8_t* arena, hipStream_t stream) {
+  return cfg.bf16 ? launch_rank_one<PB, EP_STORE_BF16>(EP_LAUNCH_ARGS) : launch_rank_one<PB, -1>(EP_LAUNCH_ARGS);
 }
 
 template <int PB, int MODE>
-static int launch_pb(const DecodeArgs& args, int num_pairs, int blocks, int threads, int ilp, hipStream_t stream) {
-  const bool bf16 = args.store_kind == EP_STORE_BF16;
-  if (ilp == 2) {
-    return bf16 ? launch_one<PB, MODE, 2, EP_STORE_BF16>(args, num_pairs, blocks, threads, stream)
-                : launch_one<PB, MODE, 2, -1>(args, num_pairs, blocks, threads, stream);
+static int launch_pb(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs,
+                     const BlockJob* block_jobs, uint8_t* arena, hipStream_t stream) {
+  if (cfg.ilp == 2) return cfg.bf16 ? launch_one<PB, MODE, 2, EP_STORE_BF16>(EP_LAUNCH_ARGS) : launch_one<PB, MODE, 2, -1>(EP_LAUNCH_ARGS);
+  return cfg.bf16 ? launch_one<PB, MODE, 1, EP_STORE_BF16>(EP_LAUNCH_ARGS) : launch_one<PB, MODE, 1, -1>(EP_LAUNCH_ARGS);
+}
+
+int lds_resident_blocks(int table_kind, int prob_bits, int lut_bytes) {
+  const int one = table_kind == EP_TABLE_LDS_RANK ? lds_rank_decode_bytes_of(lut_bytes, 16) : lds_decode_bytes(prob_bits, 16, 1);
+  return 2 * one <= 160 * 1024 ? 2 : 1;
+}
+
+LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, bool bf16, int pairs, int cus) {
+  LdsLaunch cfg;
+  cfg.table_kind = table_kind;
+  cfg.prob_bits = prob_bits;
+  cfg.bf16 = bf16 ? 1 : 0;
+  // Tables that leave room for two blocks per CU run one pair per wave on twice the waves, which hides latency best.
+  // Otherwise one block per CU, and two interleaved pairs per wave once 16 waves on every CU cannot hold all pairs.
+  const int resident = lds_resident_blocks(table_kind, prob_bits, lut_bytes);
+  cfg.ilp = table_kind != EP_TABLE_LDS_RANK && resident == 1 && pairs > cus * 16 ? 2 : 1;
+  int waves = (pairs + cus * resident * cfg.ilp - 1) / (cus * resident * cfg.ilp);
+  waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
+  int blocks = (pairs + waves * cfg.ilp - 1) / (waves * cfg.ilp);
+  cfg.blocks = blocks > cus * resident ? cus * resident : blocks;
+  cfg.threads = waves * 64;
+  cfg.lds_bytes = table_kind == EP_TABLE_LDS_RANK ? lds_rank_decode_bytes_of(lut_bytes, waves) : lds_decode_bytes(prob_bits, waves, cfg.ilp);
+  return cfg;
+}
+
+int launch_lds(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs, const BlockJob* block_jobs,
+               uint8_t* arena, hipStream_t stream) {
+  if (cfg.table_kind == EP_TABLE_LDS_RANK) {
+    switch (cfg.prob_bits) {
+      case 9: return launch_rank_pb<9>(EP_LAUNCH_ARGS);
+      case 10: return launch_rank_pb<10>(EP_LAUNCH_ARGS);
+      case 11: return launch_rank_pb<11>(EP_LAUNCH_ARGS);
+      case 12: return launch_rank_pb<12>(EP_LAUNCH_ARGS);
+      case 13: return launch_rank_pb<13>(EP_LAUNCH_ARGS);
+      case 14: return launch_rank_pb<14>(EP_LAUNCH_ARGS);
+      case 15: return launch_rank_pb<15>(EP_LAUNCH_ARGS);
+      default: return EP_HIP_EINVAL;
+    }
   }
-  return bf16 ? launch_one<PB, MODE, 1, EP_STORE_BF16>(args, num_pairs, blocks, threads, stream)
-              : launch_one<PB, MODE, 1, -1>(args, num_pairs, blocks, threads, stream);
+  const bool wide = cfg.table_kind == EP_TABLE_LDS_WIDE;
+  switch (cfg.prob_bits) {
+    case 9: return wide ? launch_pb<9, kModeWide>(EP_LAUNCH_ARGS) : launch_pb<9, kModeByte>(EP_LAUNCH_ARGS);
+    case 10: return wide ? launch_pb<10, kModeWide>(EP_LAUNCH_ARGS) : launch_pb<10, kModeByte>(EP_LAUNCH_ARGS);
+    case 11: return wide ? launch_pb<11, kModeWide>(EP_LAUNCH_ARGS) : launch_pb<11, kModeByte>(EP_LAUNCH_ARGS);
+    default: return EP_HIP_EINVAL;
+  }
 }
 
 int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int pairs, hipStream_t stream) {
@@ -654,42 +734,8 @@ int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int 
   EP_HIP_TRY(hipGetDevice(&device));
   EP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
   if (cus <= 0) cus = 256;
-  if (desc.table_kind == EP_TABLE_LDS_RANK) {
-    // As many waves as fit: 16 per block, and two blocks per CU when two copies of the tables fit its 160 KiB.
-    const int present = desc.present_offset[kStreams];
-    const int resident = 2 * lds_rank_decode_bytes(present, desc.prob_bits, 16) <= 160 * 1024 ? 2 : 1;
-    int waves = (pairs + cus * resident - 1) / (cus * resident);
-    waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
-    int blocks = (pairs + waves - 1) / waves;
-    blocks = blocks > cus * resident ? cus * resident : blocks;
-    const int lds = lds_rank_decode_bytes(present, desc.prob_bits, waves);
-    const int threads = waves * 64;
-    switch (desc.prob_bits) {
-      case 9: return launch_rank_pb<9>(args, pairs, blocks, threads, lds, stream);
-      case 10: return launch_rank_pb<10>(args, pairs, blocks, threads, lds, stream);
-      case 11: return launch_rank_pb<11>(args, pairs, blocks, threads, lds, stream);
-      case 12: return launch_rank_pb<12>(args, pairs, blocks, threads, lds, stream);
-      case 13: return launch_rank_pb<13>(args, pairs, blocks, threads, lds, stream);
-      case 14: return launch_rank_pb<14>(args, pairs, blocks, threads, lds, stream);
-      case 15: return launch_rank_pb<15>(args, pairs, blocks, threads, lds, stream);
-      default: return EP_HIP_EINVAL;
-    }
-  }
-  // One resident block per CU (the tables fill most of its LDS). Two interleaved pairs per wave once 16 waves on
-  // every CU cannot hold all pairs at once; otherwise spread the pairs over as many CUs as possible.
-  const int ilp = pairs > cus * 16 ? 2 : 1;
-  int waves = (pairs + cus * ilp - 1) / (cus * ilp);
-  waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
-  int blocks = (pairs + waves * ilp - 1) / (waves * ilp);
-  blocks = blocks > cus ? cus : blocks;
-  const bool wide = desc.table_kind == EP_TABLE_LDS_WIDE;
-  const int threads = waves * 64;
-  switch (desc.prob_bits) {
-    case 9: return wide ? launch_pb<9, kModeWide>(args, pairs, blocks, threads, ilp, stream) : launch_pb<9, kModeByte>(args, pairs, blocks, threads, ilp, stream);
-    case 10: return wide ? launch_pb<10, kModeWide>(args, pairs, blocks, threads, ilp, stream) : launch_pb<10, kModeByte>(args, pairs, blocks, threads, ilp, stream);
-    case 11: return wide ? launch_pb<11, kModeWide>(args, pairs, blocks, threads, ilp, stream) : launch_pb<11, kModeByte>(args, pairs, blocks, threads, ilp, stream);
-    default: return EP_HIP_EINVAL;
-  }
+  const LdsLaunch cfg = choose_lds_launch(desc.table_kind, desc.prob_bits, desc.lds_bytes, args.store_kind == EP_STORE_BF16, pairs, cus);
+  return launch_lds(cfg, args, pairs, nullptr, nullptr, nullptr, stream);
 }
 
 }  // namespace ep

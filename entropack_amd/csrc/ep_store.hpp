@@ -156,6 +156,29 @@ __device__ __forceinline__ uint32_t row_of(const DecodeArgs& a, uint32_t vector)
 }
 
 // Launches the LDS-table decode kernel (ep_decode_lds.hip) for an EP_TABLE_LDS_* plan.
+// A block's share of a batch: pairs [first_pair, first_pair + n_pairs) of container `job`.
+struct BlockJob {
+  int job;
+  int first_pair;
+  int n_pairs;
+  int reserved;
+};
+
+// Launch shape of the LDS-table kernels for one container, or for the containers of a batch that share it.
+struct LdsLaunch {
+  int table_kind;
+  int prob_bits;
+  int bf16;         // BF16 output takes the specialised store
+  int ilp;          // tile pairs per wave
+  int threads;
+  int lds_bytes;
+  int blocks;
+};
+
+int lds_resident_blocks(int table_kind, int prob_bits, int lut_bytes);
+LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, bool bf16, int pairs, int cus);
+int launch_lds(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs, const BlockJob* block_jobs,
+               uint8_t* arena, hipStream_t stream);
 int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int num_pairs, hipStream_t stream);
 
 }  // namespace ep

@@ -66,14 +66,13 @@ def _plan_for(buffers: LatticeBuffers, info: dict) -> DecodePlan:
     return plan
 
 
-def decode(buffers: LatticeBuffers, *, shape, dtype, threads_per_block=None, l2_prefetch=True) -> torch.Tensor:
-    payload = buffers.payload
-    device = payload.device
+def _checked_geometry(buffers: LatticeBuffers, shape, dtype):
+    """(geometry, dtype the kernel stores, decoded via float32?) of one container, after the lane's argument checks."""
+    device = buffers.payload.device
     if device.type != "cuda":
         raise RuntimeError(f"the hip lane decodes device buffers only, got {device}")
     info = decode_geometry(buffers._asdict(), shape)
-    rows, cols = info["rows"], info["cols"]
-    if buffers.scales.numel() != rows or buffers.states.numel() != max(1, info["total_tiles"]) * 32 \
+    if buffers.scales.numel() != info["rows"] or buffers.states.numel() != max(1, info["total_tiles"]) * 32 \
             or buffers.offsets.numel() != max(1, info["total_tiles"]) + 1:
         raise ValueError("lattice_rans buffers do not match the container geometry")
     for tensor in buffers:
@@ -83,6 +82,14 @@ def decode(buffers: LatticeBuffers, *, shape, dtype, threads_per_block=None, l2_
     out_dtype = torch.float32 if via_float32 else dtype
     if out_dtype not in _hip.STORE_KINDS:
         raise ValueError(f"lattice_rans does not support output dtype {dtype}")
+    return info, out_dtype, via_float32
+
+
+def decode(buffers: LatticeBuffers, *, shape, dtype, threads_per_block=None, l2_prefetch=True) -> torch.Tensor:
+    payload = buffers.payload
+    device = payload.device
+    info, out_dtype, via_float32 = _checked_geometry(buffers, shape, dtype)
+    rows, cols = info["rows"], info["cols"]
     with torch.cuda.device(device):
         plan = _plan_for(buffers, info)
         out = torch.empty((rows, cols), dtype=out_dtype, device=device)
@@ -92,6 +99,81 @@ def decode(buffers: LatticeBuffers, *, shape, dtype, threads_per_block=None, l2_
             _hip.STORE_KINDS[out_dtype], rows, cols, info["tile_elements"], plan.error.data_ptr(),
             _hip.current_stream(device)))
     return snap_to_container(out, dtype) if via_float32 else out
+
+
+class BatchDecoder:
+    """Decodes many containers (a model's layers) in one pass: ep_hip_batch_plan / ep_hip_decode_lattice_batch.
+
+    Containers that share a kernel variant go into one launch whose workgroups each take a slice of one container, so
+    layers too small to fill the device on their own run side by side. The plan (argument blocks and the block map)
+    is built once and reused for every pass, like the per-container plans it refers to. The reference decodes layer
+    by layer (entropack/linear/linear.py:125-130 called from each module's forward) and has no batched entry.
+    """
+
+    def __init__(self, items):
+        """items: iterable of (LatticeBuffers, shape, dtype); all on one device."""
+        items = list(items)
+        if not items:
+            raise ValueError("BatchDecoder needs at least one container")
+        self.device = items[0][0].payload.device
+        self._keep = []                       # plans, descs and buffers the device-side argument blocks point into
+        self._views = []                      # (byte offset, rows, cols, out dtype, final dtype or None)
+        jobs = (_hip.DecodeJob * len(items))()
+        cursor = 0
+        with torch.cuda.device(self.device):
+            for job, (buffers, shape, dtype) in zip(jobs, items):
+                if buffers.payload.device != self.device:
+                    raise ValueError("every container of a batch must live on the same device")
+                info, out_dtype, via_float32 = _checked_geometry(buffers, shape, dtype)
+                plan = _plan_for(buffers, info)
+                rows, cols = info["rows"], info["cols"]
+                job.payload_dev = _hip.pointer(buffers.payload)
+                job.payload_words = buffers.payload.numel()
+                job.offsets_dev = buffers.offsets.data_ptr()
+                job.states_dev = buffers.states.data_ptr()
+                job.scales_dev = buffers.scales.data_ptr()
+                job.tables_dev = plan.tables.data_ptr()
+                job.desc = ctypes.pointer(plan.desc)
+                job.out_offset = cursor
+                job.store_kind = _hip.STORE_KINDS[out_dtype]
+                job.tile_elements = info["tile_elements"]
+                job.rows, job.cols_padded = rows, cols
+                job.error_dev = plan.error.data_ptr()
+                self._keep.append((plan, buffers))
+                self._views.append((cursor, rows, cols, out_dtype, dtype if via_float32 else None))
+                cursor += -(-rows * cols * out_dtype.itemsize // 256) * 256
+            self.arena_bytes = cursor
+            lib = _hip.library()
+            caps = _hip.device_info(self.device.index if self.device.index is not None else torch.cuda.current_device())
+            size = ctypes.c_size_t(0)
+            _hip.check("ep_hip_batch_plan", lib.ep_hip_batch_plan(jobs, len(items), caps.compute_units, None, ctypes.byref(size)))
+            self._blob_host = torch.zeros(size.value, dtype=torch.uint8)
+            _hip.check("ep_hip_batch_plan", lib.ep_hip_batch_plan(
+                jobs, len(items), caps.compute_units, self._blob_host.data_ptr(), ctypes.byref(size)))
+            self._blob_dev = self._blob_host.to(self.device)
+
+    def decode(self, arena: torch.Tensor | None = None) -> list[torch.Tensor]:
+        """One pass over every container on torch's current stream; returns `[rows, padded cols]` views of the arena.
+
+        `arena` (uint8, at least `arena_bytes`, 256-byte aligned) lets a caller reuse one output buffer pass after pass.
+        """
+        with torch.cuda.device(self.device):
+            if arena is None:
+                arena = torch.empty(self.arena_bytes, dtype=torch.uint8, device=self.device)
+            elif arena.device != self.device or arena.dtype != torch.uint8 or arena.numel() < self.arena_bytes \
+                    or not arena.is_contiguous() or arena.data_ptr() % 256:
+                raise ValueError("arena must be a contiguous, 256-byte aligned uint8 tensor of at least arena_bytes on the batch's device")
+            _hip.check("ep_hip_decode_lattice_batch", _hip.library().ep_hip_decode_lattice_batch(
+                self._blob_host.data_ptr(), self._blob_dev.data_ptr(), arena.data_ptr(), _hip.current_stream(self.device)))
+        outputs = []
+        for offset, rows, cols, out_dtype, final in self._views:
+            view = arena[offset:offset + rows * cols * out_dtype.itemsize].view(out_dtype).view(rows, cols)
+            outputs.append(snap_to_container(view, final) if final is not None else view)
+        return outputs
+
+    def check_errors(self) -> None:
+        for _, buffers in self._keep:
+            check_errors(buffers)
 
 
 def plan_of(buffers: LatticeBuffers) -> DecodePlan | None:

@@ -120,6 +120,40 @@ int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, c
                           const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows,
                           int64_t cols_padded, int tile_elements, int32_t* error_dev, void* stream);
 
+/* Batched decode --------------------------------------------------------------------------------------------- */
+
+/* One container of a batch: the arguments of ep_hip_decode_lattice, with the output given as a byte offset
+ * (a multiple of 16) into an arena the caller passes at launch time. */
+typedef struct ep_hip_decode_job {
+  const uint16_t* payload_dev;
+  uint64_t payload_words;
+  const uint32_t* offsets_dev;
+  const uint32_t* states_dev;
+  const float* scales_dev;
+  const void* tables_dev;
+  const ep_hip_plan_desc* desc;     /* host pointer, read only while planning */
+  uint64_t out_offset;
+  int store_kind;
+  int tile_elements;
+  int64_t rows;
+  int64_t cols_padded;
+  int32_t* error_dev;
+} ep_hip_decode_job;
+
+/* Plans one pass over many containers (a whole state_dict): containers that share a kernel variant are decoded
+ * by one launch whose workgroups each take a slice of one container, so small layers fill the device together
+ * instead of one under-filled launch each. Pure host code. With `blob_host` NULL only `*blob_bytes` is written
+ * (the size to allocate); otherwise `*blob_bytes` is the capacity of `blob_host`, which receives the plan. The
+ * caller uploads the same bytes to the device (256-byte aligned) and keeps both copies for every launch.
+ * `compute_units` sizes the slices (ep_hip_device_info.compute_units).
+ * Reference: the per-layer loop a caller of decode() writes, entropack/linear/linear.py:125-130 over a model;
+ * the reference has no batched entry. */
+int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int compute_units, void* blob_host, size_t* blob_bytes);
+
+/* Launches a planned batch on `stream`: job i writes at out_arena_dev + jobs[i].out_offset. Asynchronous. */
+int ep_hip_decode_lattice_batch(const void* blob_host, const void* blob_dev, void* out_arena_dev, void* stream);
+
+
 /* Linear ---------------------------------------------------------------------------------------------------- */
 
 /* Element kinds of GEMM outputs, biases and quantiser inputs. */
