@@ -139,6 +139,41 @@ def linear_section(ep, steps):
     return out
 
 
+def small_m_section(ep, on_gpu, rows, cols, bpp, steps):
+    """BASELINE config 5, linear part: X [M, cols] bf16 N(0, 1), M in {1, 16, 128}, on the container just decoded.
+
+    The weight stream bounds this regime, so each mode is priced in GB/s on the bytes it has to move: fused = the
+    compressed container + x + y; decode_then_gemm adds one write and one read of the dense weight.
+    """
+    from torch.nn import functional as F
+    compressed_bytes = sum(t.numel() * t.element_size() for t in on_gpu.buffers.values())
+    dense_bytes = rows * cols * 2
+    out = {"workload": f"CompressedLinear {rows}x{cols} @ {bpp} bpp, X [M, {cols}] bf16 N(0,1), seed 4"}
+    layers = {}
+    for mode in ("decode_then_gemm", "fused"):
+        layer = ep.CompressedLinear(cols, rows, bias=False, device="cuda", dtype=torch.bfloat16, forward_mode=mode)
+        layer.weight = torch.nn.Parameter(on_gpu, requires_grad=False)
+        layers[mode] = layer
+    weight = layers["fused"].dequantize("cuda")
+    torch.manual_seed(4)
+    for m in (1, 4, 16, 128):
+        x = torch.randn(m, cols).to(torch.bfloat16).cuda()
+        reference = F.linear(x.float(), weight.float()).to(torch.bfloat16).double()
+        entry = {}
+        for mode, layer in layers.items():
+            y = layer(x)
+            rel = ((y.double() - reference).norm() / reference.norm()).item()
+            ms = _median_ms(lambda: layer(x), max(5, steps // 2), warmup=2)
+            moved = compressed_bytes + 2 * m * cols + 2 * m * rows
+            if mode == "decode_then_gemm" or m > 4:
+                moved += 2 * dense_bytes
+            entry[mode] = {"ms": round(ms, 5), "GBps_on_bytes_moved": round(moved / ms / 1e6, 1),
+                           "tflops": round(2.0 * m * rows * cols / ms / 1e9, 3), "rel_l2_vs_f32_reference": rel}
+        out[f"M={m}"] = entry
+    del weight
+    return out
+
+
 STACK_SHAPES = ((11520, 3840), (3840, 3840), (10240, 3840), (3840, 10240))      # qkv, out, ffn-up, ffn-down as [out, in]
 STACK_RATES = (2.3, 4.0, 5.0, 6.0, 8.0)
 
@@ -327,6 +362,8 @@ def main():
 
     if not args.no_linear:
         result["linear"] = linear_section(ep, args.steps)
+        if rows * cols >= 1 << 27:
+            result["linear_small_m"] = small_m_section(ep, on_gpu, rows, cols, bpp, args.steps)
 
     if not args.no_cpu:
         host = host_arrays(container.buffers)

@@ -9,6 +9,7 @@
 //   decode_lds_kernel (ep_decode_lds)  prob_bits <= 11: u32 slot table staged in LDS, payload streamed through an
 //                                      LDS ring.
 // Both produce bit-identical output.
+#include <hip/hip_fp16.h>
 #include <string.h>
 
 #include "ep_store.hpp"
@@ -144,6 +145,10 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
   args.num_tiles = static_cast<int>(tiles);
   args.error = error_dev;
   args.lut_bytes = args.rank_val_offset = args.rank_rs_offset = 0;
+  args.m_rows = 0;
+  args.x = nullptr;
+  args.y32 = nullptr;
+  args.ldx = args.ldy32 = 0;
   // row = floor(v / d) for v < 2^31 as umulhi(v, ceil(2^p / d)) >> (p - 32), p = 31 + ceil(log2 d), d >= 2.
   // d == 1 is handled as floor(2 v / 2): umulhi(2 v, 2^31) is exact for every 32-bit 2 v.
   {
@@ -224,20 +229,20 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   if (status != EP_HIP_OK) return status;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (desc->table_kind == EP_TABLE_GLOBAL64) return launch_global64(args, pairs, s);
-  return launch_lds_decode(args, *desc, pairs, s);
+  return launch_lds_decode(args, *desc, store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, pairs, s);
 }
 
 extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int compute_units, void* blob_host, size_t* blob_bytes) {
   using namespace ep;
   if (jobs == nullptr || n_jobs <= 0 || blob_bytes == nullptr || compute_units <= 0) return EP_HIP_EINVAL;
 
-  struct Group { int table_kind, prob_bits, bf16, lut_bytes; int64_t pairs; };
+  struct Group { int table_kind, prob_bits, kind, lut_bytes; int64_t pairs; };
   Group groups[kBatchMaxLaunches];
   int n_groups = 0;
   auto group_of = [&](const ep_hip_plan_desc& d, int store_kind) {
-    const int bf16 = store_kind == EP_STORE_BF16;
+    const int kind = store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1;
     for (int g = 0; g < n_groups; ++g) {
-      if (groups[g].table_kind == d.table_kind && groups[g].prob_bits == d.prob_bits && groups[g].bf16 == bf16) return g;
+      if (groups[g].table_kind == d.table_kind && groups[g].prob_bits == d.prob_bits && groups[g].kind == kind) return g;
     }
     return -1;
   };
@@ -260,7 +265,7 @@ extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int 
     if (g < 0) {
       if (n_groups == kBatchMaxLaunches) return EP_HIP_EUNSUPPORTED;
       g = n_groups++;
-      groups[g] = {j.desc->table_kind, j.desc->prob_bits, j.store_kind == EP_STORE_BF16, 0, 0};
+      groups[g] = {j.desc->table_kind, j.desc->prob_bits, j.store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, 0, 0};
     }
     groups[g].pairs += pairs;
     if (j.desc->lds_bytes > groups[g].lut_bytes) groups[g].lut_bytes = j.desc->lds_bytes;
@@ -273,7 +278,7 @@ extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int 
   int slice[kBatchMaxLaunches];
   for (int g = 0; g < n_groups; ++g) {
     const int big = groups[g].pairs > 0x7FFFFFFF ? 0x7FFFFFFF : static_cast<int>(groups[g].pairs);
-    cfgs[g] = choose_lds_launch(groups[g].table_kind, groups[g].prob_bits, groups[g].lut_bytes, groups[g].bf16 != 0, big, compute_units);
+    cfgs[g] = choose_lds_launch(groups[g].table_kind, groups[g].prob_bits, groups[g].lut_bytes, groups[g].kind, big, compute_units);
     const int per_round = (cfgs[g].threads / 64) * cfgs[g].ilp;
     const int resident = lds_resident_blocks(groups[g].table_kind, groups[g].prob_bits, groups[g].lut_bytes) * compute_units;
     int64_t rounds = groups[g].pairs / (static_cast<int64_t>(per_round) * resident * 8);
@@ -373,5 +378,70 @@ extern "C" int ep_hip_decode_lattice_batch(const void* blob_host, const void* bl
     const int status = launch_lds(launch.cfg, args_host[0], 0, args_dev, blocks_dev + launch.first_block, arena, s);
     if (status != EP_HIP_OK) return status;
   }
+  return EP_HIP_OK;
+}
+
+// ---- fused linear for a few activation rows ----------------------------------------------------------------------------
+
+namespace ep {
+
+__global__ __launch_bounds__(256) void zero_f32_kernel(float* __restrict__ p, int64_t count) {
+  for (int64_t i = blockIdx.x * int64_t{256} + threadIdx.x; i < count; i += gridDim.x * int64_t{256}) p[i] = 0.0f;
+}
+
+// y[m][n] = cast(y32[m][n] + bias[n]); bias has the output's type.
+__global__ __launch_bounds__(256) void finish_linear_kernel(const float* __restrict__ y32, const void* __restrict__ bias, void* __restrict__ y,
+                                                            int rows, int64_t outer, int64_t ldy, int out_kind) {
+  const int64_t n = blockIdx.x * int64_t{256} + threadIdx.x;
+  if (n >= outer) return;
+  float add = 0.0f;
+  if (bias != nullptr) {
+    if (out_kind == EP_FLOAT_BF16) add = __uint_as_float(static_cast<uint32_t>(static_cast<const uint16_t*>(bias)[n]) << 16);
+    else if (out_kind == EP_FLOAT_F16) add = __half2float(static_cast<const __half*>(bias)[n]);
+    else add = static_cast<const float*>(bias)[n];
+  }
+  for (int m = 0; m < rows; ++m) {
+    const float v = __fadd_rn(y32[m * outer + n], add);
+    if (out_kind == EP_FLOAT_BF16) static_cast<uint16_t*>(y)[m * ldy + n] = static_cast<uint16_t>(bf16_bits_rne(v));
+    else if (out_kind == EP_FLOAT_F16) static_cast<__half*>(y)[m * ldy + n] = __float2half_rn(v);
+    else static_cast<float*>(y)[m * ldy + n] = v;
+  }
+}
+
+}  // namespace ep
+
+extern "C" int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
+                                        const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, float* workspace_dev,
+                                        void* stream) {
+  using namespace ep;
+  if (weight == nullptr || x_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
+  if (out_kind < EP_FLOAT_BF16 || out_kind > EP_FLOAT_F32 || m_rows <= 0) return EP_HIP_EINVAL;
+  if (weight->desc == nullptr) return EP_HIP_EINVAL;
+  const int64_t outer = weight->rows, inner = weight->cols_padded;
+  if (ldx < inner || ldy < outer || reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || ldx % 8 != 0) return EP_HIP_EINVAL;
+  // The kernels carry at most four activation rows in registers, need whole weight rows of at least 32 vectors (a
+  // group of 32 vectors then touches at most two rows), bf16 weights, and an LDS-table plan.
+  if (m_rows > 4 || inner < 256 || weight->store_kind != EP_STORE_BF16 || weight->desc->table_kind == EP_TABLE_GLOBAL64) return EP_HIP_EUNSUPPORTED;
+  DecodeArgs args;
+  int pairs = 0;
+  const int status = fill_decode_args(weight->payload_dev, weight->payload_words, weight->offsets_dev, weight->states_dev, weight->scales_dev,
+                                      weight->tables_dev, weight->desc, nullptr, weight->store_kind, weight->rows, weight->cols_padded,
+                                      weight->tile_elements, weight->error_dev, args, pairs);
+  if (status != EP_HIP_OK) return status;
+  args.m_rows = static_cast<int>(m_rows);
+  args.x = static_cast<const uint16_t*>(x_dev);
+  args.ldx = ldx;
+  args.y32 = workspace_dev;
+  args.ldy32 = outer;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t cells = m_rows * outer;
+  hipLaunchKernelGGL(zero_f32_kernel, dim3(static_cast<unsigned>((cells + 255) / 256 < 1024 ? (cells + 255) / 256 : 1024)), dim3(256), 0, s,
+                     workspace_dev, cells);
+  EP_HIP_TRY(hipGetLastError());
+  const int launched = launch_lds_decode(args, *weight->desc, m_rows == 1 ? -2 : -3, pairs, s);
+  if (launched != EP_HIP_OK) return launched;
+  hipLaunchKernelGGL(finish_linear_kernel, dim3(static_cast<unsigned>((outer + 255) / 256)), dim3(256), 0, s, workspace_dev, bias_dev, y_dev,
+                     static_cast<int>(m_rows), outer, ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }

@@ -234,6 +234,122 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const void* __restri
   if (threadIdx.x == 0) scales[row] = scale;
 }
 
+
+// ---- few activation rows (M <= 128): the weight stream bounds the product ---------------------------------------------------
+//
+// y = x W^T reads every weight exactly once, so the kernel is built around that stream: a block owns 128 weight rows
+// and one slice of K and moves 128 x 64 weight tiles from memory to LDS with fully coalesced 16-byte loads (eight
+// lanes per 128-byte row segment), the next tile always in flight in registers. Its four waves each multiply 32 of
+// the rows with all activation rows (at most four 32-row tiles, also staged in LDS). Small tiles keep many blocks
+// resident per CU, which is what keeps enough bytes in flight; K is split across blocks so that every CU streams.
+// The partial sums land in f32 slabs [slice][M][N] and a second kernel adds them, the bias, and rounds once.
+constexpr int kSkinnyBlockN = 128;
+constexpr int kSkinnyChunk = 64;                              // K elements per step (128 bytes per row)
+
+template <int MT>     // number of 32-row activation tiles, 1..4
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                               float* __restrict__ partial, int M, int N, int K, int64_t ldx,
+                                                               int64_t ldw, int chunks_per_slice) {
+  __shared__ __align__(16) uint8_t tile_w[kSkinnyBlockN * kRowStride];
+  __shared__ __align__(16) uint8_t tile_x[MT * 32 * kRowStride];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int frag_row = lane & 31;
+  const int frag_k = (lane >> 5) * 16;             // byte offset of this lane's 8 bf16 inside a 16-element K step
+  const int n0 = blockIdx.x * kSkinnyBlockN;
+  const int k_begin = blockIdx.y * chunks_per_slice * kSkinnyChunk;
+  const int k_end = min(K, k_begin + chunks_per_slice * kSkinnyChunk);
+
+  // Tiles are rows of 8 chunks of 16 bytes; thread t moves chunks t, t + 256, ... (chunk c: row c / 8, bytes 16 (c % 8)).
+  uint4 w_next[4], x_next[MT];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = tid + 256 * i;
+      const int n = n0 + (chunk >> 3), k = k0 + 8 * (chunk & 7);
+      w_next[i] = make_uint4(0, 0, 0, 0);
+      if (n < N && k < k_end) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w + static_cast<int64_t>(n) * ldw + k));   // read once
+        w_next[i] = make_uint4(v.x, v.y, v.z, v.w);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int chunk = tid + 256 * i;
+      const int m = chunk >> 3, k = k0 + 8 * (chunk & 7);
+      x_next[i] = make_uint4(0, 0, 0, 0);
+      if (m < M && k < k_end) x_next[i] = *reinterpret_cast<const uint4*>(x + static_cast<int64_t>(m) * ldx + k);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = tid + 256 * i;
+      *reinterpret_cast<uint4*>(tile_w + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = w_next[i];
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int chunk = tid + 256 * i;
+      *reinterpret_cast<uint4*>(tile_x + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = x_next[i];
+    }
+  };
+
+  f32x16 acc[MT] = {};
+  fetch(k_begin);
+  for (int k0 = k_begin; k0 < k_end; k0 += kSkinnyChunk) {
+    __syncthreads();                                 // every wave is done with the previous tiles
+    stash();
+    __syncthreads();
+    if (k0 + kSkinnyChunk < k_end) fetch(k0 + kSkinnyChunk);
+#pragma unroll
+    for (int kk = 0; kk < kSkinnyChunk / 16; ++kk) {
+      const bf16x8 fb = *reinterpret_cast<const bf16x8*>(tile_w + (wave * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const bf16x8 fa = *reinterpret_cast<const bf16x8*>(tile_x + (t * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[t], 0, 0, 0);
+      }
+    }
+  }
+
+  // Register r of lane l holds activation row 8 (r / 4) + 4 (l / 32) + r % 4 of its tile, weight row l % 32.
+  const int n = n0 + wave * 32 + frag_row;
+  if (n >= N) return;
+  float* slab = partial + static_cast<int64_t>(blockIdx.y) * M * N;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = t * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+      if (m < M) slab[static_cast<int64_t>(m) * N + n] = acc[t][r];
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void gemm_skinny_finish_kernel(const float* __restrict__ partial, int slices, const void* __restrict__ bias,
+                                                                 void* __restrict__ y, int M, int N, int64_t ldy, int out_kind) {
+  const int64_t cell = blockIdx.x * int64_t{256} + threadIdx.x;
+  if (cell >= static_cast<int64_t>(M) * N) return;
+  const int m = static_cast<int>(cell / N), n = static_cast<int>(cell % N);
+  float sum = 0.0f;
+  for (int s = 0; s < slices; ++s) sum += partial[static_cast<int64_t>(s) * M * N + cell];
+  if (bias != nullptr) sum += load_bias(bias, out_kind, n);
+  store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, sum);
+}
+
+// K slices for M x N x K on `cus` compute units: enough blocks for about four per CU, at least one chunk each.
+static int skinny_slices(int64_t N, int64_t K, int cus) {
+  const int64_t n_blocks = (N + kSkinnyBlockN - 1) / kSkinnyBlockN;
+  const int64_t chunks = (K + kSkinnyChunk - 1) / kSkinnyChunk;
+  int64_t slices = (4 * static_cast<int64_t>(cus) + n_blocks - 1) / n_blocks;
+  slices = slices < 1 ? 1 : (slices > chunks ? chunks : slices);
+  slices = slices > 64 ? 64 : slices;
+  const int64_t per = (chunks + slices - 1) / slices;
+  return static_cast<int>((chunks + per - 1) / per);
+}
+
 static int out_kind_valid(int kind) { return kind == kOutBF16 || kind == kOutF16 || kind == kOutF32; }
 
 }  // namespace ep
@@ -253,6 +369,45 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   hipLaunchKernelGGL(gemm_bf16_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint16_t*>(x_dev), static_cast<const uint16_t*>(w_dev), bias_dev, y_dev,
                      static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), ldx, ldw, ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+size_t ep_hip_gemm_bf16_skinny_workspace(int64_t M, int64_t N, int64_t K, int compute_units) {
+  using namespace ep;
+  if (M <= 0 || N <= 0 || K <= 0 || compute_units <= 0) return 0;
+  return static_cast<size_t>(skinny_slices(N, K, compute_units)) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+}
+
+int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
+                            int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, int compute_units,
+                            void* workspace_dev, size_t workspace_bytes, void* stream) {
+  using namespace ep;
+  if (x_dev == nullptr || w_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0 || N > 0x7FFFFFFF || K > 0x7FFFFFFF - kSkinnyChunk || compute_units <= 0) return EP_HIP_EINVAL;
+  if (M > 128) return EP_HIP_EUNSUPPORTED;
+  if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0) return EP_HIP_EINVAL;
+  if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  const int slices = skinny_slices(N, K, compute_units);
+  if (workspace_bytes < static_cast<size_t>(slices) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float)) return EP_HIP_EINVAL;
+  const int chunks = static_cast<int>((K + kSkinnyChunk - 1) / kSkinnyChunk);
+  const int per = (chunks + slices - 1) / slices;
+  const dim3 grid(static_cast<unsigned>((N + kSkinnyBlockN - 1) / kSkinnyBlockN), static_cast<unsigned>(slices));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint16_t* x = static_cast<const uint16_t*>(x_dev);
+  const uint16_t* w = static_cast<const uint16_t*>(w_dev);
+  float* partial = static_cast<float*>(workspace_dev);
+  const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
+  if (M <= 32) hipLaunchKernelGGL(gemm_bf16_skinny_kernel<1>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
+  else if (M <= 64) hipLaunchKernelGGL(gemm_bf16_skinny_kernel<2>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
+  else if (M <= 96) hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
+  else hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
+  EP_HIP_TRY(hipGetLastError());
+  const int64_t cells = M * N;
+  hipLaunchKernelGGL(gemm_skinny_finish_kernel, dim3(static_cast<unsigned>((cells + 255) / 256)), dim3(256), 0, s, partial, slices, bias_dev,
+                     y_dev, m, n, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }

@@ -25,6 +25,12 @@ struct DecodeArgs {
   uint32_t lut_bytes;       // LDS_RANK: bytes of tables to stage, and where the value and rank/select parts start
   uint32_t rank_val_offset;
   uint32_t rank_rs_offset;
+  // Multiply-on-the-fly kernels only: activations x[m_rows][ldx] (bf16) and the f32 accumulator y32[m_rows][ldy32].
+  int m_rows;
+  const uint16_t* x;
+  int64_t ldx;
+  float* y32;
+  int64_t ldy32;
 };
 
 __device__ __forceinline__ void flag_error(int* error, int code) { atomicCAS(error, 0, code); }
@@ -168,7 +174,7 @@ struct BlockJob {
 struct LdsLaunch {
   int table_kind;
   int prob_bits;
-  int bf16;         // BF16 output takes the specialised store
+  int kind;         // EP_STORE_BF16 (specialised store), -1 (any container), -2 / -3 (multiply on the fly, 1 / up to 4 rows)
   int ilp;          // tile pairs per wave
   int threads;
   int lds_bytes;
@@ -176,9 +182,12 @@ struct LdsLaunch {
 };
 
 int lds_resident_blocks(int table_kind, int prob_bits, int lut_bytes);
-LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, bool bf16, int pairs, int cus);
+LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, int kind, int pairs, int cus);
 int launch_lds(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs, const BlockJob* block_jobs,
                uint8_t* arena, hipStream_t stream);
-int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int num_pairs, hipStream_t stream);
+int launch_rank(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs, const BlockJob* block_jobs,
+                uint8_t* arena, hipStream_t stream);
+int launch_dot(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, hipStream_t stream);
+int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int kind, int num_pairs, hipStream_t stream);
 
 }  // namespace ep

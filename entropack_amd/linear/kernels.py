@@ -8,6 +8,10 @@ import torch
 from ..backends import hip as _hip
 
 
+#: Up to this many activation rows the product is bound by the weight stream and takes the split-K kernel.
+SKINNY_MAX_ROWS = 128
+
+
 def _require_device(*tensors: torch.Tensor) -> torch.device:
     device = tensors[0].device
     if device.type != "cuda":
@@ -38,6 +42,16 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
     if rows == 0:
         return out.reshape(*x.shape[:-1], outer)
     bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
+    if rows <= SKINNY_MAX_ROWS:
+        with torch.cuda.device(device):
+            lib = _hip.library()
+            cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
+            workspace = torch.empty(lib.ep_hip_gemm_bf16_skinny_workspace(rows, outer, inner, cus), dtype=torch.uint8, device=device)
+            _hip.check("ep_hip_gemm_bf16_skinny", lib.ep_hip_gemm_bf16_skinny(
+                flat.data_ptr(), w.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(),
+                rows, outer, inner, flat.stride(0), w.stride(0), out.stride(0), _hip.FLOAT_KINDS[out_dtype], cus,
+                workspace.data_ptr(), workspace.numel(), _hip.current_stream(device)))
+        return out.reshape(*x.shape[:-1], outer)
     with torch.cuda.device(device):
         _hip.check("ep_hip_gemm_bf16", _hip.library().ep_hip_gemm_bf16(
             flat.data_ptr(), w.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(),

@@ -101,6 +101,61 @@ def decode(buffers: LatticeBuffers, *, shape, dtype, threads_per_block=None, l2_
     return snap_to_container(out, dtype) if via_float32 else out
 
 
+def _job_of(buffers: LatticeBuffers, info: dict, plan: DecodePlan, store_kind: int, out_offset: int = 0) -> "_hip.DecodeJob":
+    job = _hip.DecodeJob()
+    job.payload_dev = _hip.pointer(buffers.payload)
+    job.payload_words = buffers.payload.numel()
+    job.offsets_dev = buffers.offsets.data_ptr()
+    job.states_dev = buffers.states.data_ptr()
+    job.scales_dev = buffers.scales.data_ptr()
+    job.tables_dev = plan.tables.data_ptr()
+    job.desc = ctypes.pointer(plan.desc)
+    job.out_offset = out_offset
+    job.store_kind = store_kind
+    job.tile_elements = info["tile_elements"]
+    job.rows, job.cols_padded = info["rows"], info["cols"]
+    job.error_dev = plan.error.data_ptr()
+    return job
+
+
+#: Activation rows the multiply-on-the-fly kernels take at most, and the shortest weight row they handle.
+FUSED_MAX_ROWS = 4
+FUSED_MIN_COLS = 256
+
+
+def fused_linear_usable(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
+    """Can `linear_rows` take this container and activation? (Otherwise: decode, then multiply.)"""
+    rows = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    return (x.dtype == torch.bfloat16 and 0 < rows <= FUSED_MAX_ROWS and shape[1] % 8 == 0 and shape[1] >= FUSED_MIN_COLS
+            and x.shape[-1] == shape[1] and buffers.payload.device.type == "cuda")
+
+
+def linear_rows(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
+    """x[..., K] @ W.T (+ bias) for up to four activation rows, W = this bf16 container, without ever writing W.
+
+    ep_hip_linear_fused_bf16: the decode kernel multiplies each decoded vector with the activations in registers.
+    The reference decodes the whole weight and calls F.linear (entropack/linear/linear.py:163-165).
+    """
+    device = buffers.payload.device
+    info, out_dtype, _ = _checked_geometry(buffers, shape, torch.bfloat16)
+    if not fused_linear_usable(buffers, shape, x):
+        raise ValueError("linear_rows takes 1..4 bfloat16 activation rows and weight rows of a multiple of 8, at least 256, columns")
+    flat = x.reshape(-1, x.shape[-1])
+    if flat.stride(-1) != 1 or flat.stride(0) % 8 or flat.data_ptr() % 16:
+        flat = flat.contiguous()
+    outer = info["rows"]
+    with torch.cuda.device(device):
+        plan = _plan_for(buffers, info)
+        job = _job_of(buffers, info, plan, _hip.STORE_KINDS[torch.bfloat16])
+        out = torch.empty(flat.shape[0], outer, dtype=x.dtype, device=device)
+        workspace = torch.empty(flat.shape[0] * outer, dtype=torch.float32, device=device)
+        bias_ready = None if bias is None else bias.to(device=device, dtype=x.dtype).contiguous()
+        _hip.check("ep_hip_linear_fused_bf16", _hip.library().ep_hip_linear_fused_bf16(
+            ctypes.byref(job), flat.data_ptr(), flat.shape[0], flat.stride(0), None if bias_ready is None else bias_ready.data_ptr(),
+            out.data_ptr(), out.stride(0), _hip.FLOAT_KINDS[x.dtype], workspace.data_ptr(), _hip.current_stream(device)))
+    return out.reshape(*x.shape[:-1], outer)
+
+
 class BatchDecoder:
     """Decodes many containers (a model's layers) in one pass: ep_hip_batch_plan / ep_hip_decode_lattice_batch.
 
@@ -127,18 +182,8 @@ class BatchDecoder:
                 info, out_dtype, via_float32 = _checked_geometry(buffers, shape, dtype)
                 plan = _plan_for(buffers, info)
                 rows, cols = info["rows"], info["cols"]
-                job.payload_dev = _hip.pointer(buffers.payload)
-                job.payload_words = buffers.payload.numel()
-                job.offsets_dev = buffers.offsets.data_ptr()
-                job.states_dev = buffers.states.data_ptr()
-                job.scales_dev = buffers.scales.data_ptr()
-                job.tables_dev = plan.tables.data_ptr()
-                job.desc = ctypes.pointer(plan.desc)
-                job.out_offset = cursor
-                job.store_kind = _hip.STORE_KINDS[out_dtype]
-                job.tile_elements = info["tile_elements"]
-                job.rows, job.cols_padded = rows, cols
-                job.error_dev = plan.error.data_ptr()
+                filled = _job_of(buffers, info, plan, _hip.STORE_KINDS[out_dtype], cursor)
+                ctypes.memmove(ctypes.byref(job), ctypes.byref(filled), ctypes.sizeof(_hip.DecodeJob))
                 self._keep.append((plan, buffers))
                 self._views.append((cursor, rows, cols, out_dtype, dtype if via_float32 else None))
                 cursor += -(-rows * cols * out_dtype.itemsize // 256) * 256

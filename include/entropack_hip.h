@@ -165,6 +165,17 @@ enum ep_hip_float_kind { EP_FLOAT_BF16 = 0, EP_FLOAT_F16 = 1, EP_FLOAT_F32 = 2 }
 int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
                      int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, void* stream);
 
+/* The same product for at most 128 activation rows, where reading W once bounds the time: K is split over blocks so
+ * that every CU streams weights, partial sums go to `workspace_dev` (f32, 16-byte aligned, at least
+ * ep_hip_gemm_bf16_skinny_workspace(M, N, K, compute_units) bytes, contents irrelevant on entry) and a second kernel
+ * adds them and the bias and rounds once. Same operand rules as ep_hip_gemm_bf16; M > 128 returns
+ * EP_HIP_EUNSUPPORTED. Reference: the F.linear call of CompressedLinear.forward at small batch,
+ * entropack/linear/linear.py:163-165. */
+size_t ep_hip_gemm_bf16_skinny_workspace(int64_t M, int64_t N, int64_t K, int compute_units);
+int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
+                            int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, int compute_units,
+                            void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* y[M][N] = (a[M][K] . b[N][K]^T)_int32 -> f32 * scale_a[m] * scale_b[n] (+ bias[n]) -> out_kind. K a multiple of 16.
  * Reference: int8_gemm / _int8_gemm_kernel, entropack/linear/quant_kernels.py:15-54,81-93. */
 int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_a_dev, const float* scale_b_dev,
@@ -176,6 +187,20 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
  * Reference: quantize_rows / _quantize_rows_kernel, entropack/linear/quant_kernels.py:56-79,95-106. */
 int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K, int64_t ldx, int8_t* codes_dev,
                          float* scales_dev, void* stream);
+
+/* y[m_rows][rows] = x[m_rows][cols_padded] * W^T (+ bias) for one to four activation rows, W given as a compressed
+ * container (`weight`: the arguments of ep_hip_decode_lattice; out_offset is ignored, store_kind must be
+ * EP_STORE_BF16): every decoded vector is rounded to bf16 as the store would, multiplied with the matching
+ * activations in registers and reduced into `workspace_dev` (m_rows * rows floats, zeroed here), so the dense weight is
+ * never written or re-read. x is bf16 with row stride `ldx` elements (a multiple of 8, 16-byte aligned base); bias
+ * (may be NULL) and y have type `out_kind` (ep_hip_float_kind), y with row stride `ldy`. Returns EP_HIP_EUNSUPPORTED
+ * for more than four rows, fewer than 256 columns, non-bf16 weights or a GLOBAL64 plan: the caller then decodes and
+ * multiplies separately. Sums are accumulated with floating-point atomics, so the last bits can vary from run to run.
+ * Reference: the memory-bound use of CompressedLinear.forward, entropack/linear/linear.py:163-165 (decode, then
+ * F.linear); the reference has no fused form. */
+int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
+                             const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, float* workspace_dev,
+                             void* stream);
 
 #ifdef __cplusplus
 }

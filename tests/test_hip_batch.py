@@ -12,7 +12,7 @@ from conftest import Golden, golden_names
 
 class _Launch(ctypes.Structure):
     _fields_ = [(name, ctypes.c_int) for name in
-                ("table_kind", "prob_bits", "bf16", "ilp", "threads", "lds_bytes", "blocks", "first_block", "pairs")]
+                ("table_kind", "prob_bits", "kind", "ilp", "threads", "lds_bytes", "blocks", "first_block", "pairs")]
 
 
 class _Header(ctypes.Structure):
@@ -80,7 +80,7 @@ def test_batch_plan_covers_every_pair_exactly_once(compute_units):
         for job, first, count, _ in blocks[launch.first_block:launch.first_block + launch.blocks]:
             desc = descs[job]
             bf16 = jobs[job].store_kind == hip_backend.STORE_KINDS[torch.bfloat16]
-            assert (desc.table_kind, desc.prob_bits, int(bf16)) == (launch.table_kind, launch.prob_bits, launch.bf16)
+            assert (desc.table_kind, desc.prob_bits, 13 if bf16 else -1) == (launch.table_kind, launch.prob_bits, launch.kind)
             assert count > 0 and count % 1 == 0
             covered[job][first:first + count] += 1
         seen_blocks += launch.blocks

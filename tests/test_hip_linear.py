@@ -29,7 +29,8 @@ def within_one_ulp(got, rounded):
     return bool(((a - b).abs() <= 2.0 ** -7 * torch.maximum(torch.maximum(a.abs(), b.abs()), floor)).all())
 
 
-@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (1, 256, 512), (17, 100, 72), (130, 129, 264), (128, 8192, 1024)])
+@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (1, 256, 512), (17, 100, 72), (130, 129, 264), (128, 8192, 1024),
+                                   (5, 300, 1000), (64, 257, 4104), (100, 128, 128), (33, 1000, 28672), (96, 640, 8)])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
     print("case", shape, with_bias, flush=True)
@@ -147,6 +148,61 @@ def test_compressed_linear_small_m_both_modes_agree(m):
         assert y.shape == (2, m, 512)
         assert within_one_ulp(y, expect.to(torch.bfloat16))
         assert rel_l2(y, expect) <= 3 * REL_L2          # few outputs: single final-ulp flips weigh more
+
+
+@pytest.mark.parametrize("rows,cols,bpp", [(512, 2048, 4.0), (96, 256, 3.0), (300, 1032, 8.0), (64, 4104, 2.0), (1024, 3072, 5.0)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_fused_rows_never_materialise_the_weight_and_match(rows, cols, bpp, m):
+    """One to four activation rows go through the multiply-on-the-fly decode kernel (every table kind that has one);
+    the result must equal x @ bf16(W_dec).T + b to accumulation-order noise. Shapes cover row ends inside a group
+    (cols / 8 not a multiple of 32), rows shorter and longer than a tile, and prob_bits 12."""
+    from entropack_amd.backends import hip as hip_backend
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    print("case", rows, cols, bpp, m, flush=True)
+    layer, _, bias = _c3_layer("fused", rows=rows, cols=cols, bpp=bpp)
+    torch.manual_seed(13)
+    x = torch.randn(m, cols).to(torch.bfloat16).cuda()
+    decoded = layer.dequantize("cuda")
+    expect = F.linear(x.float(), decoded.float(), bias.cuda().float())
+    seen = []
+    for kind in (None, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_LDS_WIDE):
+        hip_lane.FORCE_TABLE_KIND = kind
+        try:
+            y = layer(x)
+        except hip_backend.HipError as error:
+            if error.status != hip_backend.EUNSUPPORTED:
+                raise
+            continue
+        finally:
+            hip_lane.FORCE_TABLE_KIND = None
+        torch.cuda.synchronize()
+        seen.append(kind)
+        assert y.shape == (m, rows) and y.dtype == torch.bfloat16
+        assert within_one_ulp(y, expect.to(torch.bfloat16)), kind
+        assert rel_l2(y, expect) <= 3 * REL_L2, kind                 # few outputs: single final-ulp flips weigh more
+    assert None in seen and hip_backend.TABLE_LDS_RANK in seen
+
+
+def test_fused_rows_direct_call_checks_and_f32_accuracy():
+    """linear_rows itself: float32-level agreement of the accumulator path (bias-free, so the only rounding left is the
+    final cast), batch-shaped activations, and the argument checks."""
+    from entropack_amd.schemes.base import packed_buffers
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
+    layer, _, _ = _c3_layer("fused", rows=384, cols=1024, bpp=4.0)
+    container = layer.weight
+    buffers = packed_buffers(container.buffers, LatticeBuffers)
+    decoded = layer.dequantize("cuda").float()
+    torch.manual_seed(14)
+    x = torch.randn(2, 2, 1024).to(torch.bfloat16).cuda()
+    y = hip_lane.linear_rows(buffers, shape=(384, 1024), x=x, bias=None)
+    assert y.shape == (2, 2, 384)
+    assert within_one_ulp(y, (x.float() @ decoded.T).to(torch.bfloat16))
+    hip_lane.check_errors(buffers)
+    with pytest.raises(ValueError):
+        hip_lane.linear_rows(buffers, shape=(384, 1024), x=torch.randn(5, 1024).to(torch.bfloat16).cuda(), bias=None)
+    with pytest.raises(ValueError):
+        hip_lane.linear_rows(buffers, shape=(384, 1024), x=x.float(), bias=None)
 
 
 @pytest.mark.parametrize("mode", ["decode_then_gemm", "fused"])
