@@ -13,6 +13,8 @@
 // 8 bf16 / 16 int8 consecutive in K of one row), so tiles go global -> LDS -> fragment with 16-byte accesses only.
 // Block tile 128 x 128 x 64 (bf16) or 128 x 128 x 128 (int8), 4 waves in a 2 x 2 arrangement, each wave 64 x 64 as
 // 2 x 2 MFMA tiles; the next K tile is fetched into registers while the current one is multiplied.
+#include <type_traits>
+
 #include "ep_common.hpp"
 
 namespace ep {
@@ -235,6 +237,151 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const void* __restri
 }
 
 
+// ---- large products: 256 x 256 block tiles ----------------------------------------------------------------------------------
+//
+// With 64 x 64 per wave (above) every matrix-core instruction needs one 16-byte LDS read per lane and the LDS port, not
+// the matrix cores, sets the pace. Here eight waves share a 256 x 256 block tile, 64 x 128 each: 8 matrix-core
+// instructions per 6 fragment reads, accumulators in 128 registers, two waves per SIMD so that one wave's reads hide
+// behind the other's multiplies. Two LDS stages alternate, so a K step costs one barrier: the tile for step k + 1 is
+// written while step k is multiplied, and the global loads for step k + 2 are already in flight in registers.
+constexpr int kBigM = 256, kBigN = 256, kBigThreads = 512;
+constexpr int kBigStageBytes = (kBigM + kBigN) * kRowStride;
+constexpr int kBigLdsBytes = 2 * kBigStageBytes;
+
+template <bool INT8>
+__global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                          const float* __restrict__ scale_a, const float* __restrict__ scale_b,
+                                                          const void* __restrict__ bias, void* __restrict__ y, int M, int N,
+                                                          int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy,
+                                                          int out_kind) {
+  extern __shared__ __align__(16) uint8_t big_smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 1, wave_n = wave & 1;          // 4 x 2 waves of 64 x 128
+  const int m0 = blockIdx.y * kBigM, n0 = blockIdx.x * kBigN;
+  const int frag_row = lane & 31;
+  const int frag_k = (lane >> 5) * 16;
+
+  // Per operand tile: 256 rows of 8 chunks of 16 bytes; thread t moves chunks t, t + 512, ..., 4 per operand.
+  uint4 reg_a[4], reg_b[4];
+  auto fetch = [&](int64_t kb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = tid + kBigThreads * i;
+      const int r = chunk >> 3;
+      const int64_t at = kb + 16 * (chunk & 7);
+      reg_a[i] = make_uint4(0, 0, 0, 0);
+      reg_b[i] = make_uint4(0, 0, 0, 0);
+      if (m0 + r < M && at < k_bytes) reg_a[i] = *reinterpret_cast<const uint4*>(a + (m0 + r) * lda_bytes + at);
+      if (n0 + r < N && at < k_bytes) reg_b[i] = *reinterpret_cast<const uint4*>(b + (n0 + r) * ldb_bytes + at);
+    }
+  };
+  auto stash = [&](int stage) {
+    uint8_t* tile_a = big_smem + stage * kBigStageBytes;
+    uint8_t* tile_b = tile_a + kBigM * kRowStride;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = tid + kBigThreads * i;
+      *reinterpret_cast<uint4*>(tile_a + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = reg_a[i];
+      *reinterpret_cast<uint4*>(tile_b + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = reg_b[i];
+    }
+  };
+
+  using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
+  Acc acc[2][4] = {};
+  const int64_t steps = (k_bytes + kTileBytesK - 1) / kTileBytesK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  if (steps > 1) fetch(kTileBytesK);
+  for (int64_t step = 0; step < steps; ++step) {
+    const int stage = static_cast<int>(step & 1);
+    if (step + 1 < steps) stash(stage ^ 1);
+    if (step + 2 < steps) fetch((step + 2) * kTileBytesK);
+    const uint8_t* tile_a = big_smem + stage * kBigStageBytes + (wave_m * 64 + frag_row) * kRowStride + frag_k;
+    const uint8_t* tile_b = big_smem + stage * kBigStageBytes + (kBigM + wave_n * 128 + frag_row) * kRowStride + frag_k;
+#pragma unroll
+    for (int kk = 0; kk < kTileBytesK / 32; ++kk) {
+      if constexpr (INT8) {
+        i32x4 fa[2], fb[4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) fa[t] = *reinterpret_cast<const i32x4*>(tile_a + t * 32 * kRowStride + kk * 32);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) fb[t] = *reinterpret_cast<const i32x4*>(tile_b + t * 32 * kRowStride + kk * 32);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      } else {
+        bf16x8 fa[2], fb[4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) fa[t] = *reinterpret_cast<const bf16x8*>(tile_a + t * 32 * kRowStride + kk * 32);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) fb[t] = *reinterpret_cast<const bf16x8*>(tile_b + t * 32 * kRowStride + kk * 32);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+
+  // Accumulator layout of a 32 x 32 tile: register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + wave_n * 128 + j * 32 + (lane & 31);
+      if (n >= N) continue;
+      const bool has_bias = bias != nullptr;
+      const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
+      float sb = 1.0f;
+      if constexpr (INT8) sb = scale_b[n];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wave_m * 64 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+        if (m >= M) continue;
+        float v;
+        if constexpr (INT8) {
+          // int32 -> f32, times the activation row scale, times the weight row scale, plus bias: each one rounded operation.
+          v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[m]), sb);
+          if (has_bias) v = __fadd_rn(v, bv);
+        } else {
+          v = acc[i][j][r] + bv;
+        }
+        store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, v);
+      }
+    }
+  }
+}
+
+template <bool INT8>
+static int launch_big(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
+                      int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
+  static thread_local int configured_for = -1;
+  int device = 0;
+  EP_HIP_TRY(hipGetDevice(&device));
+  if (configured_for != device) {
+    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_big_kernel<INT8>), hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
+    configured_for = device;
+  }
+  const dim3 grid(static_cast<unsigned>((N + kBigN - 1) / kBigN), static_cast<unsigned>((M + kBigM - 1) / kBigM));
+  if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
+  hipLaunchKernelGGL(gemm_big_kernel<INT8>, grid, dim3(kBigThreads), kBigLdsBytes, stream, static_cast<const uint8_t*>(a),
+                     static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                     lda_bytes, ldb_bytes, ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+// The big tiles pay once a product has enough of them to occupy the device; below that the 128 x 128 kernel spreads
+// the work over more CUs.
+static bool big_tiles_pay(int64_t M, int64_t N) {
+  return M >= kBigM && N >= kBigN && ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN) >= 96;
+}
+
 // ---- few activation rows (M <= 128): the weight stream bounds the product ---------------------------------------------------
 //
 // y = x W^T reads every weight exactly once, so the kernel is built around that stream: a block owns 128 weight rows
@@ -364,6 +511,10 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  if (big_tiles_pay(M, N)) {
+    return launch_big<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind,
+                             static_cast<hipStream_t>(stream));
+  }
   const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
   hipLaunchKernelGGL(gemm_bf16_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
@@ -421,6 +572,10 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
   if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  if (big_tiles_pay(M, N)) {
+    return launch_big<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind,
+                            static_cast<hipStream_t>(stream));
+  }
   const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
   hipLaunchKernelGGL(gemm_i8_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a_dev, b_dev, scale_a_dev,
