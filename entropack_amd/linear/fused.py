@@ -18,7 +18,7 @@ def linear_forward(layer, x: torch.Tensor) -> torch.Tensor:
     if container.compress_method == "lattice_rans" and container.encoded_dtype == torch.bfloat16:
         on_device = container.to(device=x.device)
         buffers = packed_buffers(on_device.buffers, LatticeBuffers)
-        if hip_lane.fused_linear_usable(buffers, tuple(container.shape), x):
+        if hip_lane.fused_linear_pays(buffers, tuple(container.shape), x):
             return hip_lane.linear_rows(buffers, shape=tuple(container.shape), x=x, bias=layer._bias_on(x.device))
     weight = layer.dequantize(x.device)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:

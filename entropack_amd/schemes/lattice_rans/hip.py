@@ -130,6 +130,23 @@ def fused_linear_usable(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool
             and x.shape[-1] == shape[1] and buffers.payload.device.type == "cuda")
 
 
+def fused_linear_pays(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
+    """Usable, and measured faster than decoding and multiplying separately.
+
+    With rank/select tables the four-row kernel needs more registers than two resident blocks per CU allow and loses
+    to decode + the split-K product; one row still wins there.
+    """
+    if not fused_linear_usable(buffers, shape, x):
+        return False
+    info, _, _ = _checked_geometry(buffers, shape, torch.bfloat16)
+    with torch.cuda.device(buffers.payload.device):
+        plan = _plan_for(buffers, info)
+    if plan.desc.table_kind == _hip.TABLE_GLOBAL64:
+        return False
+    rows = x.numel() // x.shape[-1]
+    return rows == 1 or plan.desc.table_kind != _hip.TABLE_LDS_RANK
+
+
 def linear_rows(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
     """x[..., K] @ W.T (+ bias) for up to four activation rows, W = this bf16 container, without ever writing W.
 

@@ -164,11 +164,16 @@ def test_fused_rows_never_materialise_the_weight_and_match(rows, cols, bpp, m):
     x = torch.randn(m, cols).to(torch.bfloat16).cuda()
     decoded = layer.dequantize("cuda")
     expect = F.linear(x.float(), decoded.float(), bias.cuda().float())
+    from entropack_amd.schemes.base import packed_buffers
+    from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
+    buffers = packed_buffers(layer.weight.buffers, LatticeBuffers)
     seen = []
     for kind in (None, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_LDS_WIDE):
         hip_lane.FORCE_TABLE_KIND = kind
         try:
-            y = layer(x)
+            # The kernel itself for every table kind; the layer's own choice (which may prefer decode + GEMM) once.
+            y = hip_lane.linear_rows(buffers, shape=(rows, cols), x=x, bias=bias.cuda())
+            y_layer = layer(x) if kind is None else y
         except hip_backend.HipError as error:
             if error.status != hip_backend.EUNSUPPORTED:
                 raise
@@ -176,10 +181,12 @@ def test_fused_rows_never_materialise_the_weight_and_match(rows, cols, bpp, m):
         finally:
             hip_lane.FORCE_TABLE_KIND = None
         torch.cuda.synchronize()
+        hip_lane.check_errors(buffers)
         seen.append(kind)
-        assert y.shape == (m, rows) and y.dtype == torch.bfloat16
-        assert within_one_ulp(y, expect.to(torch.bfloat16)), kind
-        assert rel_l2(y, expect) <= 3 * REL_L2, kind                 # few outputs: single final-ulp flips weigh more
+        for got in (y, y_layer):
+            assert got.shape == (m, rows) and got.dtype == torch.bfloat16
+            assert within_one_ulp(got, expect.to(torch.bfloat16)), kind
+            assert rel_l2(got, expect) <= 3 * REL_L2, kind                 # few outputs: single final-ulp flips weigh more
     assert None in seen and hip_backend.TABLE_LDS_RANK in seen
 
 
