@@ -30,7 +30,8 @@ def within_one_ulp(got, rounded):
 
 
 @pytest.mark.parametrize("shape", [(4096, 3072, 3072), (1, 256, 512), (17, 100, 72), (130, 129, 264), (128, 8192, 1024),
-                                   (5, 300, 1000), (64, 257, 4104), (100, 128, 128), (33, 1000, 28672), (96, 640, 8)])
+                                   (5, 300, 1000), (64, 257, 4104), (100, 128, 128), (33, 1000, 28672), (96, 640, 8),
+                                   (4100, 4200, 520)])          # the last one: 17 x 17 ragged 256 x 256 block tiles
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
     print("case", shape, with_bias, flush=True)
@@ -86,7 +87,7 @@ def test_quantize_rows_is_exact(rows, inner, dtype):
     assert codes[0].abs().max() == 0
 
 
-@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040)])
+@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040), (4100, 4200, 528)])
 def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
     print("case", shape, flush=True)
     m, n, k = shape
