@@ -5,11 +5,12 @@
 // CU stages the 16 field tables once (u32 per slot: frequency | slot - cdf | symbol) and then walks its pairs.
 //
 // Payload. Renormalisation words are consumed from the tile's end downwards, at most 32 per step. Each half keeps
-// a 128-word LDS window holding payload[W, W + 128), W a multiple of 64, with the read position p = ptr - W in
-// [64, 128) before every step. The 64 words below W are already in flight in a register (one dword per lane);
-// when p drops below 64 the window slides down by 64 words: its lower chunk moves up, the prefetched words become
-// the lower chunk and the next 64 are requested, so no renormalisation ever waits on HBM. Both halves' p live in
-// one scalar register (pA | pB << 16); they never leave [32, 128), whatever the stream holds.
+// a 128-word LDS window holding payload[W, W + 128), W a multiple of 64, with the read position p = ptr - W. The 64
+// words below W are already in flight in a register (one dword per lane). After every second step the window is
+// checked: when p has dropped below 64 it slides down by 64 words (its lower chunk moves up, the prefetched words
+// become the lower chunk and the next 64 are requested), so p is in [64, 128) before a pair of steps, at least 32
+// between them and at least 0 after them, whatever the stream holds, and no renormalisation ever waits on HBM.
+// Both halves' p live in one scalar register, biased by 64 so that the packed arithmetic never borrows.
 //
 // The nine dependent symbol steps of a group are written in inline assembly: the compiler's version of the same
 // C++ spent more scalar than vector instructions on mask bookkeeping. Per step and pair: 12 VALU, 9 SALU, one
@@ -28,6 +29,7 @@
 namespace ep {
 
 constexpr int kModeByte = 0, kModeWide = 1, kModeRank = 2;
+constexpr uint32_t kPosBias = 64;
 // KIND template values besides an ep_hip_store_kind: any container through the generic store, or no store at all:
 // the decoded weights are multiplied with a few activation rows on the fly (a.x, a.y32).
 constexpr int kKindAny = -1, kKindDot1 = -2, kKindDot4 = -3;    // one activation row, or up to four
@@ -55,7 +57,8 @@ struct Pair {
   uint32_t ring_lane;    // ring + 4 * (lane & 31): where this lane's dword of a 64-word chunk goes
   uint32_t vector0;      // first vector of this lane's tile
   int count;             // vectors in this lane's tile (0 = no tile)
-  uint32_t pos;          // pA | pB << 16: read positions inside the windows, always in [32, 128)
+  uint32_t pos;          // (pA + 64) | (pB + 64) << 16: read positions inside the windows, biased by kPosBias so that the
+                         // scalar arithmetic of a step never borrows across the fields while pA, pB fall to 0
   int windowA, windowB;  // window starts, relative to a 64-aligned base below each tile (may go negative)
   int beginA, beginB;    // position of each tile's first word, relative to that base
   uint32_t coset_base;   // LDS byte offset of this lane's coset inside a field's table pair (0 or one table)
@@ -108,11 +111,11 @@ struct Pair {
 #define EP_ASM_TAKE_SAVED(S)                                    \
   "v_lshl_or_b32 %[t" S "], %[x" S "], 16, %[d" S "]\n"          \
   "v_cndmask_b32_e64 %[x" S "], %[x" S "], %[t" S "], %[m0]\n"
-// The same with the vote as execution mask (one vector instruction less); the caller restores exec from %[sv].
+// The same with the vote as execution mask (one vector instruction less). Only the unmasked steps use it: they run
+// with every lane active, so the mask is restored to all ones without having been saved.
 #define EP_ASM_TAKE_EXEC_VCC(S) "s_mov_b64 exec, vcc\n v_lshl_or_b32 %[x" S "], %[x" S "], 16, %[d" S "]\n"
 #define EP_ASM_TAKE_EXEC_SAVED(S) "s_mov_b64 exec, %[m0]\n v_lshl_or_b32 %[x" S "], %[x" S "], 16, %[d" S "]\n"
-#define EP_ASM_SAVE_EXEC "s_mov_b64 %[sv], exec\n"
-#define EP_ASM_RESTORE_EXEC "s_mov_b64 exec, %[sv]\n"
+#define EP_ASM_RESTORE_FULL "s_mov_b64 exec, -1\n"
 
 // Coset symbol in closed form: c = slot >= f0; freq = c ? T - f0 : f0; begin = c ? f0 : 0.
 #define EP_ASM_COSET(S)                                         \
@@ -158,8 +161,8 @@ __device__ __forceinline__ void field_step_single(Pair& p, int field, uint32_t o
   EP_ASM_LOOKUP("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_ADVANCE("0") EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" \
       EP_ASM_TAKE_VCC("0")
 #define EP_FIELD_SINGLE_FAST                                                                                   \
-  EP_ASM_SAVE_EXEC EP_ASM_LOOKUP("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_ADVANCE("0") EP_ASM_VOTE("0")              \
-      "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_EXEC
+  EP_ASM_LOOKUP("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_ADVANCE("0") EP_ASM_VOTE("0")              \
+      "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_FULL
 #define EP_FIELD_SINGLE_OPERANDS(OFF)                                                                           \
   : [x0] "+v"(p.x), [pos0] "+s"(pos), [e0] "=&v"(e), [t0] "=&v"(t), [h0] "=&v"(h), [d0] "=&v"(d), [na] "=&s"(na),   \
     [nb] "=&s"(nb), [sv] "=&s"(sv)                                                                               \
@@ -196,10 +199,10 @@ __device__ __forceinline__ void field_step_dual(Pair& p0, Pair& p1, int field, u
       "s_mov_b64 %[m0], vcc\n s_waitcnt lgkmcnt(1)\n" EP_ASM_ADVANCE("1") EP_ASM_VOTE("1") "s_waitcnt lgkmcnt(1)\n" \
           EP_ASM_TAKE_SAVED("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("1")
 #define EP_FIELD_DUAL_FAST                                                                                     \
-  EP_ASM_SAVE_EXEC EP_ASM_LOOKUP("0") EP_ASM_LOOKUP("1") "s_waitcnt lgkmcnt(1)\n" EP_ASM_ADVANCE("0")            \
+  EP_ASM_LOOKUP("0") EP_ASM_LOOKUP("1") "s_waitcnt lgkmcnt(1)\n" EP_ASM_ADVANCE("0")            \
       EP_ASM_VOTE("0") "s_mov_b64 %[m0], vcc\n s_waitcnt lgkmcnt(1)\n" EP_ASM_ADVANCE("1") EP_ASM_VOTE("1")      \
           "s_waitcnt lgkmcnt(1)\n" EP_ASM_TAKE_EXEC_SAVED("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("1") \
-              EP_ASM_RESTORE_EXEC
+              EP_ASM_RESTORE_FULL
 #define EP_FIELD_DUAL_OPERANDS(OFF)                                                                             \
   : [x0] "+v"(p0.x), [x1] "+v"(p1.x), [pos0] "+s"(pos0), [pos1] "+s"(pos1), [e0] "=&v"(e0), [e1] "=&v"(e1),       \
     [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(h0), [h1] "=&v"(h1), [d0] "=&v"(d0), [d1] "=&v"(d1), [na] "=&s"(na), \
@@ -233,7 +236,7 @@ __device__ __forceinline__ void coset_step_single(Pair& p, const StepConsts& k, 
   valid = uniform(valid);
 #define EP_COSET_SINGLE_BODY EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("0")
 #define EP_COSET_SINGLE_FAST \
-  EP_ASM_SAVE_EXEC EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_EXEC
+  EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_FULL
 #define EP_COSET_SINGLE_OPERANDS                                                                                \
   : [x0] "+v"(p.x), [pos0] "+s"(pos), [cb0] "=&v"(cb), [t0] "=&v"(t), [h0] "=&v"(h), [d0] "=&v"(d), [na] "=&s"(na),  \
     [nb] "=&s"(nb), [sv] "=&s"(sv)                                                                               \
@@ -258,9 +261,9 @@ __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepCo
   EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_mov_b64 %[m0], vcc\n" EP_ASM_COSET("1") EP_ASM_VOTE("1")          \
       "s_waitcnt lgkmcnt(1)\n" EP_ASM_TAKE_SAVED("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("1")
 #define EP_COSET_DUAL_FAST                                                                               \
-  EP_ASM_SAVE_EXEC EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_mov_b64 %[m0], vcc\n" EP_ASM_COSET("1") EP_ASM_VOTE("1") \
+  EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_mov_b64 %[m0], vcc\n" EP_ASM_COSET("1") EP_ASM_VOTE("1") \
       "s_waitcnt lgkmcnt(1)\n" EP_ASM_TAKE_EXEC_SAVED("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("1")     \
-          EP_ASM_RESTORE_EXEC
+          EP_ASM_RESTORE_FULL
 #define EP_COSET_DUAL_OPERANDS                                                                                    \
   : [x0] "+v"(p0.x), [x1] "+v"(p1.x), [pos0] "+s"(pos0), [pos1] "+s"(pos1), [cb0] "=&v"(cb0), [cb1] "=&v"(cb1),     \
     [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(h0), [h1] "=&v"(h1), [d0] "=&v"(d0), [d1] "=&v"(d1), [na] "=&s"(na),   \
@@ -370,7 +373,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
     for (int j = 0; j < ILP; ++j) {
       Pair& s = st[j];
       const int64_t tile = 2 * static_cast<int64_t>(first_pair + j) + half;
-      s.ring = rings0 + static_cast<uint32_t>((wave * ILP + j) * 2 + half) * kRingBytes;
+      const uint32_t window_at = rings0 + static_cast<uint32_t>((wave * ILP + j) * 2 + half) * kRingBytes;
+      s.ring = window_at - 2u * kPosBias;                   // positions are kept biased, see Pair::pos
       uint32_t word_begin = 0, word_end = 0;
       s.count = 0;
       s.x = kStateMin;
@@ -399,7 +403,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       const int begin = static_cast<int>(word_begin - base);
       const int ptr = static_cast<int>(word_end - base);
       const int low = (ptr & ~63) - 64;                       // the window holds relative [low, low + 128)
-      s.ring_lane = s.ring + 4u * static_cast<uint32_t>(l32);
+      s.ring_lane = window_at + 4u * static_cast<uint32_t>(l32);
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const int64_t at = static_cast<int64_t>(base) + low + 64 * c + 2 * l32;
@@ -410,7 +414,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       }
       s.fetch_dword = static_cast<int32_t>((static_cast<int64_t>(base) + low - 64) >> 1) + l32;
       s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
-      const int p = ptr - low;                                // in [64, 128)
+      const int p = ptr - low + static_cast<int>(kPosBias);  // position in [64, 128), stored biased
       s.pos = static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 0)) | (static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 32)) << 16);
       s.windowA = __builtin_amdgcn_readlane(low, 0);
       s.windowB = __builtin_amdgcn_readlane(low, 32);
@@ -423,19 +427,19 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
     // (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
     // the next 64 words down.
     auto top_up = [&](Pair& s) {
-      const uint32_t low_bits = ~s.pos & 0x00400040u;        // bit 6 of a field clear <=> that position < 64
+      const uint32_t low_bits = ~s.pos & 0x00800080u;        // bit 7 of a biased field clear <=> that position < 64
       if (__builtin_expect(low_bits != 0, 0)) {
         asm volatile("" ::: "memory");     // keep this a scalar branch: the common case must cost no vector work
-        if ((low_bits >> (half ? 22 : 6)) & 1u) {
+        if ((low_bits >> (half ? 23 : 7)) & 1u) {
           const uint32_t kept = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(s.ring_lane));
           lds_write32(s.ring_lane + 128u, kept);
           lds_write32(s.ring_lane, s.prefetch);
           s.fetch_dword -= 32;
           s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
         }
-        s.pos += low_bits;                  // + 64 in the fields that slid
-        s.windowA -= static_cast<int>(low_bits & 0x40u);
-        s.windowB -= static_cast<int>((low_bits >> 16) & 0x40u);
+        s.pos += low_bits >> 1;             // + 64 in the fields that slid
+        s.windowA -= static_cast<int>((low_bits >> 1) & 0x40u);
+        s.windowB -= static_cast<int>((low_bits >> 17) & 0x40u);
       }
     };
 
@@ -589,10 +593,10 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         scale[j] = valid_lane ? a.scales[row] : 0.0f;
         if constexpr (DOT_ROWS > 0) dot_prefetch(vector[j], row, valid_lane, dot_in[j]);
       }
+      // A window is checked (and slid) after every second step: a step consumes at most 32 words per half and a check
+      // leaves at least 64 in the window. The checks sit after fields 0, 2, 4, 6 and after the group's last step.
       if constexpr (ILP == 2) coset_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], k, valid);
       else coset_step_single<PB, MODE, MASKED>(st[0], k, valid);
-#pragma unroll
-      for (int j = 0; j < ILP; ++j) top_up(st[j]);
       uint32_t high[ILP];
 #pragma unroll
       for (int j = 0; j < ILP; ++j) high[j] = st[j].coset_base + L::kHighBase;
@@ -607,8 +611,10 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         } else {
           field_step_single<PB, MODE, MASKED>(st[0], f, f & 3, f < 4 ? st[0].coset_base : high[0], k, valid);
         }
+        if ((f & 1) == 0 || f == kFields - 1) {
 #pragma unroll
-        for (int j = 0; j < ILP; ++j) top_up(st[j]);
+          for (int j = 0; j < ILP; ++j) top_up(st[j]);
+        }
       }
       if constexpr (DOT_ROWS > 0) {
 #pragma unroll
@@ -628,7 +634,6 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       DotInput dot_in;
       if constexpr (DOT_ROWS > 0) dot_prefetch(vector, row, valid_lane, dot_in);
       coset_step_single<PB, MODE, true>(s, k, valid);
-      top_up(s);
       const uint32_t high = s.coset_base + L::kHighBase;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
@@ -638,7 +643,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         } else {
           field_step_single<PB, MODE, true>(s, f, f & 3, f < 4 ? s.coset_base : high, k, valid);
         }
-        top_up(s);
+        if ((f & 1) == 0 || f == kFields - 1) top_up(s);
       }
       if constexpr (DOT_ROWS > 0) dot_emit(s, scale, valid_lane, dot_in);
       else if (valid_lane) emit(s, vector, scale);
@@ -693,7 +698,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       const uint64_t stale = __builtin_amdgcn_ballot_w64(s.count > 0 && s.x != kStateMin);
       const uint64_t live = __builtin_amdgcn_ballot_w64(s.count > 0);
       const bool liveA = (live & 1u) != 0, liveB = ((live >> 32) & 1u) != 0;
-      const int ptrA = s.windowA + static_cast<int>(s.pos & 0xFFFFu), ptrB = s.windowB + static_cast<int>(s.pos >> 16);
+      const int ptrA = s.windowA + static_cast<int>(s.pos & 0xFFFFu) - static_cast<int>(kPosBias);
+      const int ptrB = s.windowB + static_cast<int>(s.pos >> 16) - static_cast<int>(kPosBias);
       const bool badA = liveA && (ptrA != s.beginA || static_cast<uint32_t>(stale) != 0);
       const bool badB = liveB && (ptrB != s.beginB || static_cast<uint32_t>(stale >> 32) != 0);
       if ((badA || badB) && lane == 0) {
