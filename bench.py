@@ -349,7 +349,7 @@ def main():
                         f"{' +0.1% x20 outliers' if outliers else ''} @ {bpp} bpp target",
             "actual_bpp": round(container.actual_bpp, 4), "tiles": int(lattice.states.shape[0]),
             "prob_bits": int(container.buffers["layout"][1]), "tile_elements": int(container.buffers["layout"][2]),
-            "table_kind": hip_lane.plan_of(lattice).table_kind, "algorithmic_bytes": alg_bytes,
+            "table_kind": hip_lane.launch_table_kind(lattice, shape=(rows, cols), dtype=torch.bfloat16), "algorithmic_bytes": alg_bytes,
             "params_per_s": round(rows * cols / (wall / args.steps), 1), "encode_seconds_cpu": round(encode_seconds, 2),
         },
         "roofline": {

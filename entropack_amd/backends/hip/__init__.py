@@ -16,8 +16,9 @@ LIBRARY_PATH = os.path.join(_PACKAGE_DIR, "libentropack_hip.so")
 ABI_VERSION = 1
 
 OK, EINVAL, EUNSUPPORTED, ERUNTIME, ENODEVICE = range(5)
-TABLE_GLOBAL64, TABLE_LDS_BYTE, TABLE_LDS_WIDE, TABLE_LDS_RANK = range(4)
-TABLE_KIND_NAMES = {TABLE_GLOBAL64: "global64", TABLE_LDS_BYTE: "lds_byte", TABLE_LDS_WIDE: "lds_wide", TABLE_LDS_RANK: "lds_rank"}
+TABLE_GLOBAL64, TABLE_LDS_BYTE, TABLE_LDS_WIDE, TABLE_LDS_RANK, TABLE_LDS_SYM = range(5)
+TABLE_KIND_NAMES = {TABLE_GLOBAL64: "global64", TABLE_LDS_BYTE: "lds_byte", TABLE_LDS_WIDE: "lds_wide", TABLE_LDS_RANK: "lds_rank",
+                    TABLE_LDS_SYM: "lds_sym"}
 DECODE_ERRORS = {
     2: "a renormalisation read passed the start of a tile's payload (truncated or corrupt payload)",
     3: "a tile ended with unread payload words or a lane state other than 2**15 (corrupt payload, states or tables)",
@@ -43,7 +44,7 @@ class PlanDesc(ctypes.Structure):
     _fields_ = [
         ("table_kind", ctypes.c_int), ("prob_bits", ctypes.c_int), ("table_bytes", ctypes.c_size_t),
         ("lds_bytes", ctypes.c_int), ("max_alphabet", ctypes.c_int), ("alphabet_sum", ctypes.c_int),
-        ("present_offset", ctypes.c_int * 18),
+        ("sym_offset", ctypes.c_int), ("present_offset", ctypes.c_int * 18),
     ]
 
 
@@ -79,6 +80,8 @@ _SIGNATURES = {
         ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
         ctypes.POINTER(PlanDesc), ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_void_p]),
+    "ep_hip_decode_table_kind": (ctypes.c_int, [
+        ctypes.POINTER(PlanDesc), ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int]),
     "ep_hip_batch_plan": (ctypes.c_int, [
         ctypes.POINTER(DecodeJob), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_size_t)]),
     "ep_hip_decode_lattice_batch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),

@@ -59,6 +59,13 @@ inline size_t rank_table_bytes(int present, int prob_bits) {
   return rank_rs_offset(present, prob_bits) + kFieldStreams * rank_rs_stream_bytes(prob_bits);
 }
 
+// LDS_SYM section: FB u64[16][256] = {freq | (value + 128) << 24, cdf + LDS address of the stream's slot table}, then
+// SLOT u8[16][2^pb] = value + 128. The kernel stages it at LDS offset 0.
+constexpr int kSymFbStreamBytes = 256 * 8;
+constexpr int kSymFbBytes = kFieldStreams * kSymFbStreamBytes;
+inline int sym_table_bytes(int prob_bits) { return kSymFbBytes + (kFieldStreams << prob_bits); }
+inline int lds_sym_decode_bytes(int prob_bits, int waves) { return sym_table_bytes(prob_bits) + waves * 2 * kRingBytes + 256; }
+
 // LDS bytes the LDS-table decode kernel needs for `waves` wavefronts each carrying `ilp` tile pairs.
 inline int lds_decode_bytes(int prob_bits, int waves, int ilp) {
   return (kFieldStreams << prob_bits) * 4 + waves * ilp * 2 * kRingBytes + 256;

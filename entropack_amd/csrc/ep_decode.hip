@@ -145,6 +145,7 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
   args.num_tiles = static_cast<int>(tiles);
   args.error = error_dev;
   args.lut_bytes = args.rank_val_offset = args.rank_rs_offset = 0;
+  args.sym_tables = nullptr;
   args.m_rows = 0;
   args.x = nullptr;
   args.y32 = nullptr;
@@ -174,9 +175,14 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
       args.rank_rs_offset = static_cast<uint32_t>(rank_rs_offset(present, desc->prob_bits));
       return EP_HIP_OK;
     }
+    case EP_TABLE_LDS_SYM:
+      if (desc->sym_offset == 0) return EP_HIP_EINVAL;
+      [[fallthrough]];
     case EP_TABLE_LDS_BYTE:
     case EP_TABLE_LDS_WIDE:
-      return desc->prob_bits <= 11 ? EP_HIP_OK : EP_HIP_EINVAL;
+      if (desc->prob_bits > 11 || desc->sym_offset < 0) return EP_HIP_EINVAL;
+      if (desc->sym_offset != 0) args.sym_tables = static_cast<const uint8_t*>(tables_dev) + desc->sym_offset;
+      return EP_HIP_OK;
     default:
       return EP_HIP_EINVAL;
   }
@@ -232,6 +238,16 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   return launch_lds_decode(args, *desc, store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, pairs, s);
 }
 
+extern "C" int ep_hip_decode_table_kind(const ep_hip_plan_desc* desc, int store_kind, int64_t rows, int64_t cols_padded, int tile_elements,
+                                        int compute_units) {
+  using namespace ep;
+  if (desc == nullptr || rows <= 0 || cols_padded <= 0 || tile_elements <= 0 || compute_units <= 0) return -1;
+  const int64_t vectors = rows * (cols_padded / 8);
+  const int tv = tile_vectors_of(tile_elements);
+  const int64_t pairs = ((vectors + tv - 1) / tv + 1) / 2;
+  return effective_table_kind(*desc, store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, pairs, compute_units);
+}
+
 extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int compute_units, void* blob_host, size_t* blob_bytes) {
   using namespace ep;
   if (jobs == nullptr || n_jobs <= 0 || blob_bytes == nullptr || compute_units <= 0) return EP_HIP_EINVAL;
@@ -241,8 +257,9 @@ extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int 
   int n_groups = 0;
   auto group_of = [&](const ep_hip_plan_desc& d, int store_kind) {
     const int kind = store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1;
+    const int tables = effective_table_kind(d, kind, int64_t{1} << 40, compute_units);     // a batch is always a large launch
     for (int g = 0; g < n_groups; ++g) {
-      if (groups[g].table_kind == d.table_kind && groups[g].prob_bits == d.prob_bits && groups[g].kind == kind) return g;
+      if (groups[g].table_kind == tables && groups[g].prob_bits == d.prob_bits && groups[g].kind == kind) return g;
     }
     return -1;
   };
@@ -265,7 +282,8 @@ extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int 
     if (g < 0) {
       if (n_groups == kBatchMaxLaunches) return EP_HIP_EUNSUPPORTED;
       g = n_groups++;
-      groups[g] = {j.desc->table_kind, j.desc->prob_bits, j.store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, 0, 0};
+      const int kind = j.store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1;
+      groups[g] = {effective_table_kind(*j.desc, kind, int64_t{1} << 40, compute_units), j.desc->prob_bits, kind, 0, 0};
     }
     groups[g].pairs += pairs;
     if (j.desc->lds_bytes > groups[g].lut_bytes) groups[g].lut_bytes = j.desc->lds_bytes;

@@ -22,9 +22,21 @@ static int launch_pb(EP_LAUNCH_PARAMS) {
   return bf16 ? launch_one<PB, MODE, 1, EP_STORE_BF16>(EP_LAUNCH_ARGS) : launch_one<PB, MODE, 1, kKindAny>(EP_LAUNCH_ARGS);
 }
 
+static int lds_bytes_for(int table_kind, int prob_bits, int lut_bytes, int waves, int ilp) {
+  if (table_kind == EP_TABLE_LDS_RANK) return lds_rank_decode_bytes_of(lut_bytes, waves);
+  if (table_kind == EP_TABLE_LDS_SYM) return lds_sym_decode_bytes(prob_bits, waves);
+  return lds_decode_bytes(prob_bits, waves, ilp);
+}
+
 int lds_resident_blocks(int table_kind, int prob_bits, int lut_bytes) {
-  const int one = table_kind == EP_TABLE_LDS_RANK ? lds_rank_decode_bytes_of(lut_bytes, 16) : lds_decode_bytes(prob_bits, 16, 1);
-  return 2 * one <= 160 * 1024 ? 2 : 1;
+  return 2 * lds_bytes_for(table_kind, prob_bits, lut_bytes, 16, 1) <= 160 * 1024 ? 2 : 1;
+}
+
+int effective_table_kind(const ep_hip_plan_desc& desc, int kind, int64_t pairs, int cus) {
+  const bool has_kernel = kind == EP_STORE_BF16 || kind == kKindAny || kind == kKindDot1;
+  if (desc.table_kind == EP_TABLE_LDS_SYM) return has_kernel ? EP_TABLE_LDS_SYM : EP_TABLE_LDS_BYTE;     // the byte tables are there too
+  if (desc.table_kind == EP_TABLE_LDS_BYTE && desc.sym_offset != 0 && has_kernel && pairs > static_cast<int64_t>(cus) * 16) return EP_TABLE_LDS_SYM;
+  return desc.table_kind;
 }
 
 LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, int kind, int pairs, int cus) {
@@ -35,18 +47,20 @@ LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, int ki
   // Tables that leave room for two blocks per CU run one pair per wave on twice the waves, which hides latency best.
   // Otherwise one block per CU, and two interleaved pairs per wave once 16 waves on every CU cannot hold all pairs.
   const int resident = lds_resident_blocks(table_kind, prob_bits, lut_bytes);
-  cfg.ilp = table_kind != EP_TABLE_LDS_RANK && resident == 1 && pairs > cus * 16 ? 2 : 1;
+  const bool single_pair_only = table_kind == EP_TABLE_LDS_RANK || table_kind == EP_TABLE_LDS_SYM;
+  cfg.ilp = !single_pair_only && resident == 1 && pairs > cus * 16 ? 2 : 1;
   int waves = (pairs + cus * resident * cfg.ilp - 1) / (cus * resident * cfg.ilp);
   waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
   int blocks = (pairs + waves * cfg.ilp - 1) / (waves * cfg.ilp);
   cfg.blocks = blocks > cus * resident ? cus * resident : blocks;
   cfg.threads = waves * 64;
-  cfg.lds_bytes = table_kind == EP_TABLE_LDS_RANK ? lds_rank_decode_bytes_of(lut_bytes, waves) : lds_decode_bytes(prob_bits, waves, cfg.ilp);
+  cfg.lds_bytes = lds_bytes_for(table_kind, prob_bits, lut_bytes, waves, cfg.ilp);
   return cfg;
 }
 
 int launch_lds(EP_LAUNCH_PARAMS) {
   if (cfg.table_kind == EP_TABLE_LDS_RANK) return launch_rank(EP_LAUNCH_ARGS);
+  if (cfg.table_kind == EP_TABLE_LDS_SYM) return launch_sym(EP_LAUNCH_ARGS);
   if (cfg.kind == kKindDot1 || cfg.kind == kKindDot4) return block_jobs == nullptr ? launch_dot(cfg, args, num_pairs, stream) : EP_HIP_EINVAL;
   const bool wide = cfg.table_kind == EP_TABLE_LDS_WIDE;
   switch (cfg.prob_bits) {
@@ -62,7 +76,7 @@ int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int 
   EP_HIP_TRY(hipGetDevice(&device));
   EP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
   if (cus <= 0) cus = 256;
-  const LdsLaunch cfg = choose_lds_launch(desc.table_kind, desc.prob_bits, desc.lds_bytes, kind, pairs, cus);
+  const LdsLaunch cfg = choose_lds_launch(effective_table_kind(desc, kind, pairs, cus), desc.prob_bits, desc.lds_bytes, kind, pairs, cus);
   return launch_lds(cfg, args, pairs, nullptr, nullptr, nullptr, stream);
 }
 

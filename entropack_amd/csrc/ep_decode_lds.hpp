@@ -28,7 +28,7 @@
 
 namespace ep {
 
-constexpr int kModeByte = 0, kModeWide = 1, kModeRank = 2;
+constexpr int kModeByte = 0, kModeWide = 1, kModeRank = 2, kModeSym = 3;
 constexpr uint32_t kPosBias = 64;
 // KIND template values besides an ep_hip_store_kind: any container through the generic store, or no store at all:
 // the decoded weights are multiplied with a few activation rows on the fly (a.x, a.y32).
@@ -314,15 +314,51 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, 
   p.pos = pos;
 }
 
+// ---- two-level tables (byte values, prob_bits <= 11) --------------------------------------------------------------------
+//
+// slot -> value + 128 (one byte) -> {freq | (value + 128) << 24, cdf}. A quarter of the slot table of the byte form,
+// so two workgroups share a CU; one more dependent LDS read per step, one vector instruction less. The stored cdf
+// already contains the LDS address bits that `slot | table address` carries, and the first word has the layout of
+// a byte-form entry, so reconstruction is shared with it.
+template <int PB, bool MASKED>
+__device__ __forceinline__ void sym_step(Pair& p, int field, uint32_t slot_cb, const StepConsts& k, bool valid_lane) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(3))) const u32x2* lds_u2;
+  typedef __attribute__((address_space(3))) const uint8_t* lds_u8;
+  constexpr uint32_t kTable = 1u << PB;
+  const uint32_t x = p.x;
+  const uint32_t at = (x & (kTable - 1u)) | slot_cb;
+  const uint32_t value = *reinterpret_cast<lds_u8>(static_cast<uintptr_t>(at + static_cast<uint32_t>(field) * 2u * kTable));
+  const u32x2 entry = *reinterpret_cast<lds_u2>(static_cast<uintptr_t>((value << 3) + p.coset_base + static_cast<uint32_t>(field) * 2u * kSymFbStreamBytes));
+  const uint32_t next = __umul24(entry.x, x >> PB) + at - entry.y;
+  p.e[field] = entry.x;
+  p.x = (!MASKED || valid_lane) ? next : x;
+  uint32_t t, d, na, nb;
+  uint32_t pos = uniform(p.pos);
+  if constexpr (MASKED) {
+    asm volatile(EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("0")
+                 : [x0] "+v"(p.x), [pos0] "+s"(pos), [t0] "=&v"(t), [d0] "=&v"(d), [na] "=&s"(na), [nb] "=&s"(nb)
+                 : [ring0] "v"(p.ring), [shv] "v"(k.shv)
+                 : "vcc", "scc", "memory");
+  } else {
+    asm volatile(EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_FULL
+                 : [x0] "+v"(p.x), [pos0] "+s"(pos), [t0] "=&v"(t), [d0] "=&v"(d), [na] "=&s"(na), [nb] "=&s"(nb)
+                 : [ring0] "v"(p.ring), [shv] "v"(k.shv)
+                 : "vcc", "scc", "memory");
+  }
+  p.pos = pos;
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
 template <int PB, int MODE, int ILP, int KIND>
 __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_begin, int pair_end, int pair_stride) {
   extern __shared__ __align__(16) uint8_t smem[];
   using L = Layout<PB, MODE>;
-  constexpr bool WIDE = MODE != kModeByte;      // symbols as integers (plus minima or already as values), not biased bytes
-  static_assert(MODE != kModeRank || ILP == 1, "the rank/select steps are single-pair");
-  const uint32_t lut_bytes = MODE == kModeRank ? (a.lut_bytes + 255u) / 256u * 256u : L::kLutBytes;
+  constexpr bool WIDE = MODE == kModeWide || MODE == kModeRank;    // symbols as integers, not as biased bytes in bits 24..31
+  static_assert((MODE != kModeRank && MODE != kModeSym) || ILP == 1, "the rank/select and two-level steps are single-pair");
+  const uint32_t lut_bytes = MODE == kModeRank ? (a.lut_bytes + 255u) / 256u * 256u
+                                               : (MODE == kModeSym ? static_cast<uint32_t>(kSymFbBytes + (kFieldStreams << PB)) : L::kLutBytes);
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
 
   const int waves = blockDim.x >> 6;
@@ -337,9 +373,9 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   auto lds_write32 = [](uint32_t at, uint32_t value) { *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(at)) = value; };
 
   {
-    const uint4* src = reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.plan) + kHeaderBytes);
+    const uint4* src = reinterpret_cast<const uint4*>(MODE == kModeSym ? a.sym_tables : reinterpret_cast<const uint8_t*>(a.plan) + kHeaderBytes);
     uint4* dst = reinterpret_cast<uint4*>(smem);
-    const uint32_t quads = (MODE == kModeRank ? a.lut_bytes : L::kLutBytes) / 16;
+    const uint32_t quads = (MODE == kModeRank ? a.lut_bytes : lut_bytes) / 16;
     for (uint32_t i = threadIdx.x; i < quads; i += blockDim.x) dst[i] = src[i];
     if (threadIdx.x < kStreams) {
       reinterpret_cast<int32_t*>(smem + lut_bytes + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes)[threadIdx.x] =
@@ -356,7 +392,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   k.f0s = uniform(a.plan[kHdrCosetFreq0]);
   k.f0v = k.f0s;
   k.f1v = L::kTable - k.f0s;
-  k.ktab = MODE == kModeRank ? (L::kTable / 32u) * 8u : L::kTableBytes;    // byte distance between a field's two cosets
+  // Byte distance between a field's two cosets, in the table the coset offset is added to.
+  k.ktab = MODE == kModeRank ? (L::kTable / 32u) * 8u : (MODE == kModeSym ? static_cast<uint32_t>(kSymFbStreamBytes) : L::kTableBytes);
   const uint32_t rank_val0 = uniform(a.rank_val_offset), rank_rs0 = uniform(a.rank_rs_offset);
   k.shv = half ? 16u : 0u;
   // Keep the per-lane constants in vector registers (the steps name them as VGPR operands).
@@ -580,6 +617,11 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       s.dot_row = any ? low : -1;
     };
 
+    // Two-level tables: LDS address of the lane's coset's slot table of field 0 (coset_base is 0 or one FB stream).
+    auto sym_slot_base = [](uint32_t coset_base) {
+      return static_cast<uint32_t>(kSymFbBytes) + (coset_base != 0 ? L::kTable : 0u);
+    };
+
     // One group of 32 vectors per half, both interleaved pairs in lock step. `valid` is the wave's lane mask.
     auto group_dual = [&](auto masked_tag, int offset, bool valid_lane, uint64_t valid) {
       constexpr bool MASKED = decltype(masked_tag)::value;
@@ -605,6 +647,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         if constexpr (MODE == kModeRank) {
           rank_step<PB, MASKED>(st[0], f, st[0].coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)),
                                 rank_val0, k, valid_lane);
+        } else if constexpr (MODE == kModeSym) {
+          sym_step<PB, MASKED>(st[0], f, sym_slot_base(st[0].coset_base), k, valid_lane);
         } else if constexpr (ILP == 2) {
           field_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], f, f & 3, f < 4 ? st[0].coset_base : high[0],
                                             f < 4 ? st[ILP - 1].coset_base : high[ILP - 1], k, valid);
@@ -640,6 +684,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         if constexpr (MODE == kModeRank) {
           rank_step<PB, true>(s, f, s.coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)), rank_val0, k,
                               valid_lane);
+        } else if constexpr (MODE == kModeSym) {
+          sym_step<PB, true>(s, f, sym_slot_base(s.coset_base), k, valid_lane);
         } else {
           field_step_single<PB, MODE, true>(s, f, f & 3, f < 4 ? s.coset_base : high, k, valid);
         }
@@ -724,6 +770,13 @@ __global__ __launch_bounds__(1024, 8) void decode_rank_kernel(DecodeArgs a, int 
   decode_lds_body<PB, kModeRank, 1, KIND>(a, static_cast<int>(blockIdx.x) * per_block, num_pairs, static_cast<int>(gridDim.x) * per_block);
 }
 
+// The two-level tables are a quarter of the byte form's: two workgroups per CU, at most 64 registers.
+template <int PB, int KIND>
+__global__ __launch_bounds__(1024, 8) void decode_sym_kernel(DecodeArgs a, int num_pairs) {
+  const int per_block = static_cast<int>(blockDim.x >> 6);
+  decode_lds_body<PB, kModeSym, 1, KIND>(a, static_cast<int>(blockIdx.x) * per_block, num_pairs, static_cast<int>(gridDim.x) * per_block);
+}
+
 // Batch: each block decodes its slice of one of many containers. The argument block is read with every word made
 // wave-uniform, so that it lives in scalar registers exactly as kernel arguments do.
 __device__ __forceinline__ DecodeArgs load_job(const DecodeArgs* __restrict__ jobs, const BlockJob& mine, uint8_t* arena) {
@@ -746,6 +799,16 @@ __global__ __launch_bounds__(1024) void decode_lds_batch_kernel(const DecodeArgs
   const int first = static_cast<int>(uniform(static_cast<uint32_t>(mine.first_pair)));
   const int count = static_cast<int>(uniform(static_cast<uint32_t>(mine.n_pairs)));
   decode_lds_body<PB, MODE, ILP, KIND>(a, first, first + count, static_cast<int>(blockDim.x >> 6) * ILP);
+}
+
+template <int PB, int KIND>
+__global__ __launch_bounds__(1024, 8) void decode_sym_batch_kernel(const DecodeArgs* __restrict__ jobs,
+                                                                   const BlockJob* __restrict__ block_jobs, uint8_t* arena) {
+  const BlockJob mine = block_jobs[blockIdx.x];
+  const DecodeArgs a = load_job(jobs, mine, arena);
+  const int first = static_cast<int>(uniform(static_cast<uint32_t>(mine.first_pair)));
+  const int count = static_cast<int>(uniform(static_cast<uint32_t>(mine.n_pairs)));
+  decode_lds_body<PB, kModeSym, 1, KIND>(a, first, first + count, static_cast<int>(blockDim.x >> 6));
 }
 
 template <int PB, int KIND>

@@ -16,6 +16,51 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint4* __restrict__ p, s
   for (size_t i = blockIdx.x * size_t{256} + threadIdx.x; i < quads; i += gridDim.x * size_t{256}) p[i] = make_uint4(0, 0, 0, 0);
 }
 
+// LDS_SYM section of a byte-valued plan: one block per field stream, same chunked scan as below.
+__global__ __launch_bounds__(256) void build_sym_tables_kernel(const int32_t* __restrict__ meta, const uint16_t* __restrict__ freq_tables,
+                                                               int prob_bits, uint8_t* __restrict__ section) {
+  __shared__ uint32_t chunk_sum[256];
+  const int stream = blockIdx.x + 1;
+  const int tid = threadIdx.x;
+  const uint32_t size = 1u << prob_bits;
+  const int sym_min = meta[stream * kMetaWidth + 1];
+  const int freq_off = meta[stream * kMetaWidth + 2];
+  const int alphabet = meta[stream * kMetaWidth + 3];
+  if (alphabet <= 0) return;
+  const uint16_t* freq = freq_tables + freq_off;
+  const int per = (alphabet + 255) / 256;
+  const int first = tid * per;
+  const int last = first + per < alphabet ? first + per : alphabet;
+  uint32_t local = 0;
+  for (int s = first; s < last; ++s) local += freq[s];
+  chunk_sum[tid] = local;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t running = 0;
+    for (int i = 0; i < 256; ++i) {
+      const uint32_t v = chunk_sum[i];
+      chunk_sum[i] = running;
+      running += v;
+    }
+  }
+  __syncthreads();
+  uint32_t running = chunk_sum[tid];
+  // The decode step forms slot | (LDS address of this stream's slot table) and subtracts the second word from
+  // freq * (x >> pb) + that, so the address is folded into the stored cdf.
+  const uint32_t slot_table_at = static_cast<uint32_t>(kSymFbBytes) + (static_cast<uint32_t>(stream - 1) << prob_bits);
+  const uint32_t folded = static_cast<uint32_t>(kSymFbBytes) + ((static_cast<uint32_t>(stream - 1) & 1u) << prob_bits);
+  uint2* fb = reinterpret_cast<uint2*>(section) + (stream - 1) * 256;
+  uint8_t* slots = section + slot_table_at;
+  for (int s = first; s < last; ++s) {
+    const uint32_t f = freq[s];
+    if (f == 0) continue;
+    const uint32_t value = static_cast<uint32_t>(s + sym_min + 128);
+    fb[value] = make_uint2(f | (value << 24), running + folded);
+    for (uint32_t d = 0; d < f && running + d < size; ++d) slots[running + d] = static_cast<uint8_t>(value);
+    running += f;
+  }
+}
+
 struct RankLayout {
   int present_offset[18];
   uint32_t val_offset;     // byte offsets inside the table area
@@ -197,6 +242,7 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   if (meta[0 * 4 + 3] == 0) return EP_HIP_EINVAL;
 
   const bool lds_fits = prob_bits <= 11 && ep::lds_decode_bytes(prob_bits, 1, 1) <= lds_limit_bytes;
+  const bool sym_ok = byte_ok && lds_fits;
   rank_ok = rank_ok && present <= 65535 && ep::lds_rank_decode_bytes(static_cast<int>(present), prob_bits, 4) <= lds_limit_bytes;
   int kind = EP_TABLE_GLOBAL64;
   if (lds_fits && byte_ok) kind = EP_TABLE_LDS_BYTE;
@@ -204,7 +250,8 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   else if (rank_ok) kind = EP_TABLE_LDS_RANK;
   if (force_kind >= 0) {
     const bool allowed = force_kind == EP_TABLE_GLOBAL64 || (force_kind == EP_TABLE_LDS_BYTE && lds_fits && byte_ok) ||
-                         (force_kind == EP_TABLE_LDS_WIDE && lds_fits && wide_ok) || (force_kind == EP_TABLE_LDS_RANK && rank_ok);
+                         (force_kind == EP_TABLE_LDS_WIDE && lds_fits && wide_ok) || (force_kind == EP_TABLE_LDS_RANK && rank_ok) ||
+                         (force_kind == EP_TABLE_LDS_SYM && sym_ok);
     if (!allowed) return EP_HIP_EUNSUPPORTED;
     kind = force_kind;
   }
@@ -222,6 +269,13 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   } else {
     desc->table_bytes = ep::kHeaderBytes + (static_cast<size_t>(ep::kFieldStreams) << prob_bits) * 4;
     desc->lds_bytes = (ep::kFieldStreams << prob_bits) * 4;
+    // Byte-valued plans whose slot tables leave room for only one workgroup per CU also carry the two-level form,
+    // which fits twice: launches with more tile pairs than one pass of resident waves use it.
+    const bool crowded = 2 * ep::lds_decode_bytes(prob_bits, 16, 1) > 160 * 1024;
+    if (kind == EP_TABLE_LDS_SYM || (kind == EP_TABLE_LDS_BYTE && crowded && 2 * ep::lds_sym_decode_bytes(prob_bits, 16) <= 160 * 1024)) {
+      desc->sym_offset = static_cast<int>((desc->table_bytes + 255) / 256 * 256);
+      desc->table_bytes = static_cast<size_t>(desc->sym_offset) + static_cast<size_t>(ep::sym_table_bytes(prob_bits));
+    }
   }
   return EP_HIP_OK;
 }
@@ -231,7 +285,10 @@ int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_table
   if (stream_meta_dev == nullptr || desc == nullptr || tables_dev == nullptr) return EP_HIP_EINVAL;
   if (freq_tables_dev == nullptr && desc->alphabet_sum != 0) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(tables_dev) % 256 != 0) return EP_HIP_EINVAL;
-  if (desc->prob_bits < 9 || desc->prob_bits > 15 || desc->table_kind < 0 || desc->table_kind > EP_TABLE_LDS_RANK) return EP_HIP_EINVAL;
+  if (desc->prob_bits < 9 || desc->prob_bits > 15 || desc->table_kind < 0 || desc->table_kind > EP_TABLE_LDS_SYM) return EP_HIP_EINVAL;
+  if (desc->sym_offset != 0 && (desc->sym_offset % 256 != 0 || desc->prob_bits > 11 ||
+                                static_cast<size_t>(desc->sym_offset) + ep::sym_table_bytes(desc->prob_bits) > desc->table_bytes)) return EP_HIP_EINVAL;
+  if (desc->table_kind == EP_TABLE_LDS_SYM && desc->sym_offset == 0) return EP_HIP_EINVAL;
   if (desc->table_bytes < ep::kHeaderBytes || desc->table_bytes % 16 != 0) return EP_HIP_EINVAL;
   ep::RankLayout rank = {};
   if (desc->table_kind == EP_TABLE_LDS_RANK) {
@@ -251,9 +308,16 @@ int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_table
   hipLaunchKernelGGL(ep::zero_fill_kernel, dim3(static_cast<unsigned>((quads + 255) / 256 < 1024 ? (quads + 255) / 256 : 1024)),
                      dim3(256), 0, s, static_cast<uint4*>(tables_dev), quads);
   EP_HIP_TRY(hipGetLastError());
+  // A plan of kind LDS_SYM holds the byte tables too (the kernels without a two-level form read those).
+  const int built_kind = desc->table_kind == EP_TABLE_LDS_SYM ? EP_TABLE_LDS_BYTE : desc->table_kind;
   hipLaunchKernelGGL(ep::build_tables_kernel, dim3(ep::kStreams), dim3(256), 0, s, stream_meta_dev, freq_tables_dev,
-                     desc->table_kind, desc->prob_bits, static_cast<uint32_t*>(tables_dev), rank);
+                     built_kind, desc->prob_bits, static_cast<uint32_t*>(tables_dev), rank);
   EP_HIP_TRY(hipGetLastError());
+  if (desc->sym_offset != 0) {
+    hipLaunchKernelGGL(ep::build_sym_tables_kernel, dim3(ep::kFieldStreams), dim3(256), 0, s, stream_meta_dev, freq_tables_dev,
+                       desc->prob_bits, static_cast<uint8_t*>(tables_dev) + desc->sym_offset);
+    EP_HIP_TRY(hipGetLastError());
+  }
   return EP_HIP_OK;
 }
 

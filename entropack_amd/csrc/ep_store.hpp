@@ -25,6 +25,7 @@ struct DecodeArgs {
   uint32_t lut_bytes;       // LDS_RANK: bytes of tables to stage, and where the value and rank/select parts start
   uint32_t rank_val_offset;
   uint32_t rank_rs_offset;
+  const uint8_t* sym_tables;   // the plan's two-level (LDS_SYM) section, or null
   // Multiply-on-the-fly kernels only: activations x[m_rows][ldx] (bf16) and the f32 accumulator y32[m_rows][ldy32].
   int m_rows;
   const uint16_t* x;
@@ -188,6 +189,11 @@ int launch_lds(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, cons
 int launch_rank(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs, const BlockJob* block_jobs,
                 uint8_t* arena, hipStream_t stream);
 int launch_dot(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, hipStream_t stream);
+int launch_sym(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, const DecodeArgs* jobs, const BlockJob* block_jobs,
+               uint8_t* arena, hipStream_t stream);
+// The table form a launch of `pairs` tile pairs really uses: byte plans with a two-level section switch to it once
+// the launch is larger than one pass of resident waves (where occupancy, not the length of a step, sets the pace).
+int effective_table_kind(const ep_hip_plan_desc& desc, int kind, int64_t pairs, int cus);
 int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int kind, int num_pairs, hipStream_t stream);
 
 }  // namespace ep

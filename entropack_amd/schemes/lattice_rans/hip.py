@@ -238,6 +238,19 @@ class BatchDecoder:
             check_errors(buffers)
 
 
+def launch_table_kind(buffers: LatticeBuffers, *, shape, dtype) -> str:
+    """Name of the table form a decode of this container to `dtype` runs with (after at least one decode)."""
+    plan = plan_of(buffers)
+    if plan is None:
+        raise RuntimeError("the container has not been decoded yet")
+    info, out_dtype, _ = _checked_geometry(buffers, shape, dtype)
+    device = buffers.payload.device
+    caps = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device())
+    kind = _hip.library().ep_hip_decode_table_kind(ctypes.byref(plan.desc), _hip.STORE_KINDS[out_dtype], info["rows"], info["cols"],
+                                                   info["tile_elements"], caps.compute_units)
+    return _hip.TABLE_KIND_NAMES[kind]
+
+
 def plan_of(buffers: LatticeBuffers) -> DecodePlan | None:
     """The cached plan of a container that has been decoded at least once."""
     return getattr(buffers.layout, "_lattice_rans_hip_plan", None)

@@ -45,8 +45,12 @@ enum ep_hip_table_kind {
   EP_TABLE_GLOBAL64 = 0,    /* u64 per slot in HBM/L2, any prob_bits 9..15, any alphabet */
   EP_TABLE_LDS_BYTE = 1,    /* u32 per slot, LDS-resident; prob_bits <= 11, every field value in [-128, 127] */
   EP_TABLE_LDS_WIDE = 2,    /* u32 per slot, LDS-resident; prob_bits <= 11, alphabets <= 1024, frequencies < 2048 */
-  EP_TABLE_LDS_RANK = 3     /* LDS-resident rank/select form: per 32 slots a bitmap of symbol ends + running symbol count,
+  EP_TABLE_LDS_RANK = 3,    /* LDS-resident rank/select form: per 32 slots a bitmap of symbol ends + running symbol count,
                                per present symbol freq | cdf << 16 and an int16 value; any prob_bits whose tables fit LDS */
+  EP_TABLE_LDS_SYM = 4      /* two-level, LDS-resident: u8 per slot (the value + 128) and, per value, freq | (value+128) << 24
+                               and cdf; a quarter of LDS_BYTE's size, so two workgroups share a CU. Same conditions as
+                               LDS_BYTE. LDS_BYTE plans at prob_bits 11 carry it as a second section (sym_offset) that
+                               large launches use; as a plan's own kind (force_kind only) every launch uses it */
 };
 
 /* Device-side error flag values written (first one wins) to *error_dev by the decode kernels; same meaning as the
@@ -74,6 +78,7 @@ typedef struct ep_hip_plan_desc {
   int lds_bytes;              /* dynamic LDS the decode kernel will request (0 for GLOBAL64) */
   int max_alphabet;
   int alphabet_sum;
+  int sym_offset;             /* byte offset of the LDS_SYM section inside the plan buffer, 0 = none */
   int present_offset[18];     /* LDS_RANK: symbols with non-zero frequency in field streams before stream s (index s),
                                  [17] = their total; zero for the other kinds */
 } ep_hip_plan_desc;
@@ -119,6 +124,12 @@ int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, c
                           const uint32_t* states_dev, const float* scales_dev, const void* tables_dev,
                           const ep_hip_plan_desc* desc, void* out_dev, int store_kind, int64_t rows,
                           int64_t cols_padded, int tile_elements, int32_t* error_dev, void* stream);
+
+/* The table form ep_hip_decode_lattice uses for a container of this geometry: desc->table_kind, except that
+ * LDS_BYTE plans with a two-level section (sym_offset != 0) take EP_TABLE_LDS_SYM once the launch has more tile pairs
+ * than 16 waves on every one of `compute_units` CUs can hold. Host only; -1 on bad arguments. */
+int ep_hip_decode_table_kind(const ep_hip_plan_desc* desc, int store_kind, int64_t rows, int64_t cols_padded,
+                             int tile_elements, int compute_units);
 
 /* Batched decode --------------------------------------------------------------------------------------------- */
 

@@ -49,6 +49,18 @@ def _host_jobs(names, compute_units=256, force=None):
     return jobs, descs, pairs
 
 
+def _qualifies(name, force):
+    """Does this golden container have the forced table form?"""
+    golden = Golden(name)
+    meta = np.ascontiguousarray(golden.buffers["stream_meta"], dtype=np.int32)
+    freq = np.ascontiguousarray(golden.buffers["freq_tables"], dtype=np.uint16)
+    _, prob_bits, tile_elements = (int(v) for v in golden.buffers["layout"])
+    desc = hip_backend.PlanDesc()
+    return hip_backend.library().ep_hip_plan_describe(
+        meta.ctypes.data, freq.ctypes.data if freq.size else None, freq.size, prob_bits, tile_elements, 160 * 1024,
+        -1 if force is None else force, ctypes.byref(desc)) == hip_backend.OK
+
+
 def _plan(jobs, compute_units=256):
     lib = hip_backend.library()
     size = ctypes.c_size_t(0)
@@ -80,7 +92,10 @@ def test_batch_plan_covers_every_pair_exactly_once(compute_units):
         for job, first, count, _ in blocks[launch.first_block:launch.first_block + launch.blocks]:
             desc = descs[job]
             bf16 = jobs[job].store_kind == hip_backend.STORE_KINDS[torch.bfloat16]
-            assert (desc.table_kind, desc.prob_bits, 13 if bf16 else -1) == (launch.table_kind, launch.prob_bits, launch.kind)
+            tables = desc.table_kind                                   # a batch always takes the two-level form where a plan has it
+            if tables == hip_backend.TABLE_LDS_BYTE and desc.sym_offset:
+                tables = hip_backend.TABLE_LDS_SYM
+            assert (tables, desc.prob_bits, 13 if bf16 else -1) == (launch.table_kind, launch.prob_bits, launch.kind)
             assert count > 0 and count % 1 == 0
             covered[job][first:first + count] += 1
         seen_blocks += launch.blocks
@@ -127,10 +142,12 @@ def _bits(tensor):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("force", [None, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_GLOBAL64], ids=["auto", "lds_rank", "global64"])
+@pytest.mark.parametrize("force", [None, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_LDS_SYM, hip_backend.TABLE_GLOBAL64],
+                         ids=["auto", "lds_rank", "lds_sym", "global64"])
 def test_batch_of_golden_containers_matches_reference_bits(force):
     from entropack_amd.schemes.lattice_rans import hip as hip_lane
-    names = golden_names()
+    names = [name for name in golden_names() if _qualifies(name, force)]
+    assert len(names) >= 5
     print("batch of", names, "force", force, flush=True)
     hip_lane.FORCE_TABLE_KIND = force
     try:

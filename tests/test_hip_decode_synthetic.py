@@ -68,7 +68,8 @@ def decode_and_check(weight, kinds=(None,), dtype=torch.bfloat16, **options):
     return container, used
 
 
-ALL_KINDS = (None, hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE, hip_backend.TABLE_LDS_RANK)
+ALL_KINDS = (None, hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_WIDE, hip_backend.TABLE_LDS_RANK,
+             hip_backend.TABLE_LDS_SYM)
 
 
 def test_config_2_outliers_4096x4096():
@@ -135,5 +136,10 @@ def test_full_size_target_8192x28672():
         first = ep.decompress(on_gpu, ep.EntroPackLossyConfig(execution_backend="hip"))
         second = ep.decompress(on_gpu, ep.EntroPackLossyConfig())          # "auto" resolves to hip on this box
         assert torch.equal(first, second)
+        lattice = LatticeBuffers(**{k: on_gpu.buffers[k] for k in LatticeBuffers._fields})
+        # Byte plans at prob_bits 11 switch to their two-level section when the launch has more tile pairs than 16 waves
+        # per CU hold (8066 at 4 bpp; the 4033 pairs at 2 bpp are one pass and stay); prob_bits 12 uses rank/select.
+        expected = {2.0: "lds_byte", 4.0: "lds_sym", 8.0: "lds_rank"}[bpp]
+        assert hip_lane.launch_table_kind(lattice, shape=(8192, 28672), dtype=torch.bfloat16) == expected
         del first, second, on_gpu, container
         torch.cuda.empty_cache()

@@ -169,7 +169,7 @@ def test_fused_rows_never_materialise_the_weight_and_match(rows, cols, bpp, m):
     from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
     buffers = packed_buffers(layer.weight.buffers, LatticeBuffers)
     seen = []
-    for kind in (None, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_LDS_WIDE):
+    for kind in (None, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_LDS_WIDE, hip_backend.TABLE_LDS_SYM):
         hip_lane.FORCE_TABLE_KIND = kind
         try:
             # The kernel itself for every table kind; the layer's own choice (which may prefer decode + GEMM) once.
