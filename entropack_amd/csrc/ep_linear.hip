@@ -248,7 +248,7 @@ constexpr int kBigM = 256, kBigN = 256, kBigThreads = 512;
 constexpr int kBigStageBytes = (kBigM + kBigN) * kRowStride;
 constexpr int kBigLdsBytes = 2 * kBigStageBytes;
 
-template <bool INT8>
+template <bool INT8, bool GUARD>      // GUARD = false: M, N multiples of 256 and K of one tile step, no bounds checks on loads
 __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                           const float* __restrict__ scale_a, const float* __restrict__ scale_b,
                                                           const void* __restrict__ bias, void* __restrict__ y, int M, int N,
@@ -273,8 +273,8 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
       const int64_t at = kb + 16 * (chunk & 7);
       reg_a[i] = make_uint4(0, 0, 0, 0);
       reg_b[i] = make_uint4(0, 0, 0, 0);
-      if (m0 + r < M && at < k_bytes) reg_a[i] = *reinterpret_cast<const uint4*>(a + (m0 + r) * lda_bytes + at);
-      if (n0 + r < N && at < k_bytes) reg_b[i] = *reinterpret_cast<const uint4*>(b + (n0 + r) * ldb_bytes + at);
+      if (!GUARD || (m0 + r < M && at < k_bytes)) reg_a[i] = *reinterpret_cast<const uint4*>(a + (m0 + r) * lda_bytes + at);
+      if (!GUARD || (n0 + r < N && at < k_bytes)) reg_b[i] = *reinterpret_cast<const uint4*>(b + (n0 + r) * ldb_bytes + at);
     }
   };
   auto stash = [&](int stage) {
@@ -357,23 +357,31 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
   }
 }
 
-template <bool INT8>
-static int launch_big(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
+template <bool INT8, bool GUARD>
+static int launch_big_variant(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                       int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
   static thread_local int configured_for = -1;
   int device = 0;
   EP_HIP_TRY(hipGetDevice(&device));
   if (configured_for != device) {
-    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_big_kernel<INT8>), hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
+    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_big_kernel<INT8, GUARD>), hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
     configured_for = device;
   }
   const dim3 grid(static_cast<unsigned>((N + kBigN - 1) / kBigN), static_cast<unsigned>((M + kBigM - 1) / kBigM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
-  hipLaunchKernelGGL(gemm_big_kernel<INT8>, grid, dim3(kBigThreads), kBigLdsBytes, stream, static_cast<const uint8_t*>(a),
+  hipLaunchKernelGGL((gemm_big_kernel<INT8, GUARD>), grid, dim3(kBigThreads), kBigLdsBytes, stream, static_cast<const uint8_t*>(a),
                      static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
                      lda_bytes, ldb_bytes, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
+}
+
+template <bool INT8>
+static int launch_big(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
+                      int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
+  const bool interior = M % kBigM == 0 && N % kBigN == 0 && k_bytes % kTileBytesK == 0;
+  return interior ? launch_big_variant<INT8, false>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream)
+                  : launch_big_variant<INT8, true>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream);
 }
 
 // The big tiles pay once a product has one of them for every CU of the device (256 on MI355X); below that the
