@@ -235,7 +235,7 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   if (status != EP_HIP_OK) return status;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (desc->table_kind == EP_TABLE_GLOBAL64) return launch_global64(args, pairs, s);
-  return launch_lds_decode(args, *desc, store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, pairs, s);
+  return launch_lds_decode(args, *desc, kernel_kind_of(store_kind), pairs, s);
 }
 
 extern "C" int ep_hip_decode_table_kind(const ep_hip_plan_desc* desc, int store_kind, int64_t rows, int64_t cols_padded, int tile_elements,
@@ -245,7 +245,7 @@ extern "C" int ep_hip_decode_table_kind(const ep_hip_plan_desc* desc, int store_
   const int64_t vectors = rows * (cols_padded / 8);
   const int tv = tile_vectors_of(tile_elements);
   const int64_t pairs = ((vectors + tv - 1) / tv + 1) / 2;
-  return effective_table_kind(*desc, store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1, pairs, compute_units);
+  return effective_table_kind(*desc, kernel_kind_of(store_kind), pairs, compute_units);
 }
 
 extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int compute_units, void* blob_host, size_t* blob_bytes) {
@@ -256,7 +256,7 @@ extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int 
   Group groups[kBatchMaxLaunches];
   int n_groups = 0;
   auto group_of = [&](const ep_hip_plan_desc& d, int store_kind) {
-    const int kind = store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1;
+    const int kind = kernel_kind_of(store_kind);
     const int tables = effective_table_kind(d, kind, int64_t{1} << 40, compute_units);     // a batch is always a large launch
     for (int g = 0; g < n_groups; ++g) {
       if (groups[g].table_kind == tables && groups[g].prob_bits == d.prob_bits && groups[g].kind == kind) return g;
@@ -282,7 +282,7 @@ extern "C" int ep_hip_batch_plan(const ep_hip_decode_job* jobs, int n_jobs, int 
     if (g < 0) {
       if (n_groups == kBatchMaxLaunches) return EP_HIP_EUNSUPPORTED;
       g = n_groups++;
-      const int kind = j.store_kind == EP_STORE_BF16 ? EP_STORE_BF16 : -1;
+      const int kind = kernel_kind_of(j.store_kind);
       groups[g] = {effective_table_kind(*j.desc, kind, int64_t{1} << 40, compute_units), j.desc->prob_bits, kind, 0, 0};
     }
     groups[g].pairs += pairs;

@@ -17,9 +17,14 @@ static int launch_one(EP_LAUNCH_PARAMS) {
 
 template <int PB, int MODE>
 static int launch_pb(EP_LAUNCH_PARAMS) {
-  const bool bf16 = cfg.kind == EP_STORE_BF16;
-  if (cfg.ilp == 2) return bf16 ? launch_one<PB, MODE, 2, EP_STORE_BF16>(EP_LAUNCH_ARGS) : launch_one<PB, MODE, 2, kKindAny>(EP_LAUNCH_ARGS);
-  return bf16 ? launch_one<PB, MODE, 1, EP_STORE_BF16>(EP_LAUNCH_ARGS) : launch_one<PB, MODE, 1, kKindAny>(EP_LAUNCH_ARGS);
+  if (cfg.ilp == 2) {
+    if (cfg.kind == EP_STORE_BF16) return launch_one<PB, MODE, 2, EP_STORE_BF16>(EP_LAUNCH_ARGS);
+    if (cfg.kind == EP_STORE_I8) return launch_one<PB, MODE, 2, EP_STORE_I8>(EP_LAUNCH_ARGS);
+    return launch_one<PB, MODE, 2, kKindAny>(EP_LAUNCH_ARGS);
+  }
+  if (cfg.kind == EP_STORE_BF16) return launch_one<PB, MODE, 1, EP_STORE_BF16>(EP_LAUNCH_ARGS);
+  if (cfg.kind == EP_STORE_I8) return launch_one<PB, MODE, 1, EP_STORE_I8>(EP_LAUNCH_ARGS);
+  return launch_one<PB, MODE, 1, kKindAny>(EP_LAUNCH_ARGS);
 }
 
 static int lds_bytes_for(int table_kind, int prob_bits, int lut_bytes, int waves, int ilp) {
@@ -33,7 +38,7 @@ int lds_resident_blocks(int table_kind, int prob_bits, int lut_bytes) {
 }
 
 int effective_table_kind(const ep_hip_plan_desc& desc, int kind, int64_t pairs, int cus) {
-  const bool has_kernel = kind == EP_STORE_BF16 || kind == kKindAny || kind == kKindDot1;
+  const bool has_kernel = kind == EP_STORE_BF16 || kind == EP_STORE_I8 || kind == kKindAny || kind == kKindDot1;
   if (desc.table_kind == EP_TABLE_LDS_SYM) return has_kernel ? EP_TABLE_LDS_SYM : EP_TABLE_LDS_BYTE;     // the byte tables are there too
   if (desc.table_kind == EP_TABLE_LDS_BYTE && desc.sym_offset != 0 && has_kernel && pairs > static_cast<int64_t>(cus) * 16) return EP_TABLE_LDS_SYM;
   return desc.table_kind;

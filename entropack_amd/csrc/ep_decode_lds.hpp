@@ -537,6 +537,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
         const u32x4 quad = {packed[0], packed[1], packed[2], packed[3]};
         __builtin_nontemporal_store(quad, reinterpret_cast<u32x4*>(a.out) + vector);
+      } else if constexpr (KIND == EP_STORE_I8) {
+        store_vector_i8(a.out, vector, w);
       } else {
         store_vector(a.out, a.store_kind, vector, w);
       }

@@ -20,6 +20,7 @@ template <int PB>
 static int launch_rank_pb(EP_LAUNCH_PARAMS) {
   switch (cfg.kind) {
     case EP_STORE_BF16: return launch_rank_one<PB, EP_STORE_BF16>(EP_LAUNCH_ARGS);
+    case EP_STORE_I8: return launch_rank_one<PB, EP_STORE_I8>(EP_LAUNCH_ARGS);
     case kKindDot1: return launch_rank_one<PB, kKindDot1>(EP_LAUNCH_ARGS);
     case kKindDot4: return launch_rank_one<PB, kKindDot4>(EP_LAUNCH_ARGS);
     default: return launch_rank_one<PB, kKindAny>(EP_LAUNCH_ARGS);

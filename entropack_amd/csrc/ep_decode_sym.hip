@@ -25,6 +25,7 @@ template <int PB>
 static int launch_sym_pb(EP_LAUNCH_PARAMS) {
   switch (cfg.kind) {
     case EP_STORE_BF16: return launch_sym_one<PB, EP_STORE_BF16>(EP_LAUNCH_ARGS);
+    case EP_STORE_I8: return launch_sym_one<PB, EP_STORE_I8>(EP_LAUNCH_ARGS);
     case kKindDot1: return launch_sym_dot<PB, kKindDot1>(EP_LAUNCH_ARGS);
     case kKindDot4: return EP_HIP_EINVAL;       // four activation rows do not fit this kernel's 64 registers
     default: return launch_sym_one<PB, kKindAny>(EP_LAUNCH_ARGS);

@@ -95,7 +95,8 @@ def test_batch_plan_covers_every_pair_exactly_once(compute_units):
             tables = desc.table_kind                                   # a batch always takes the two-level form where a plan has it
             if tables == hip_backend.TABLE_LDS_BYTE and desc.sym_offset:
                 tables = hip_backend.TABLE_LDS_SYM
-            assert (tables, desc.prob_bits, 13 if bf16 else -1) == (launch.table_kind, launch.prob_bits, launch.kind)
+            int8 = jobs[job].store_kind == hip_backend.STORE_KINDS[torch.int8]
+            assert (tables, desc.prob_bits, 13 if bf16 else 4 if int8 else -1) == (launch.table_kind, launch.prob_bits, launch.kind)
             assert count > 0 and count % 1 == 0
             covered[job][first:first + count] += 1
         seen_blocks += launch.blocks
