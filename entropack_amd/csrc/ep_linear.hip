@@ -399,43 +399,46 @@ static bool big_tiles_pay(int64_t M, int64_t N) {
 // resident per CU, which is what keeps enough bytes in flight; K is split across blocks so that every CU streams.
 // The partial sums land in f32 slabs [slice][M][N] and a second kernel adds them, the bias, and rounds once.
 constexpr int kSkinnyBlockN = 128;
-constexpr int kSkinnyChunk = 64;                              // K elements per step (128 bytes per row)
+constexpr int kSkinnyChunkBytes = 128;                        // bytes of K per row and step: 64 bf16 or 128 int8
 
-template <int MT>     // number of 32-row activation tiles, 1..4
-__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                                                               float* __restrict__ partial, int M, int N, int K, int64_t ldx,
-                                                               int64_t ldw, int chunks_per_slice) {
+template <int MT, bool INT8>     // MT = number of 32-row activation tiles, 1..4
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
+                                                          void* __restrict__ partial, int M, int N, int64_t k_bytes,
+                                                          int64_t ldx_bytes, int64_t ldw_bytes, int chunks_per_slice) {
   __shared__ __align__(16) uint8_t tile_w[kSkinnyBlockN * kRowStride];
   __shared__ __align__(16) uint8_t tile_x[MT * 32 * kRowStride];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int frag_row = lane & 31;
-  const int frag_k = (lane >> 5) * 16;             // byte offset of this lane's 8 bf16 inside a 16-element K step
+  const int frag_k = (lane >> 5) * 16;             // byte offset of this lane's 16 bytes inside a 32-byte K step
   const int n0 = blockIdx.x * kSkinnyBlockN;
-  const int k_begin = blockIdx.y * chunks_per_slice * kSkinnyChunk;
-  const int k_end = min(K, k_begin + chunks_per_slice * kSkinnyChunk);
+  const int64_t k_begin = static_cast<int64_t>(blockIdx.y) * chunks_per_slice * kSkinnyChunkBytes;
+  const int64_t k_stop = k_begin + static_cast<int64_t>(chunks_per_slice) * kSkinnyChunkBytes;
+  const int64_t k_end = k_stop < k_bytes ? k_stop : k_bytes;
 
   // Tiles are rows of 8 chunks of 16 bytes; thread t moves chunks t, t + 256, ... (chunk c: row c / 8, bytes 16 (c % 8)).
   uint4 w_next[4], x_next[MT];
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int64_t k0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int chunk = tid + 256 * i;
-      const int n = n0 + (chunk >> 3), k = k0 + 8 * (chunk & 7);
+      const int n = n0 + (chunk >> 3);
+      const int64_t k = k0 + 16 * (chunk & 7);
       w_next[i] = make_uint4(0, 0, 0, 0);
       if (n < N && k < k_end) {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w + static_cast<int64_t>(n) * ldw + k));   // read once
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w + n * ldw_bytes + k));   // read once
         w_next[i] = make_uint4(v.x, v.y, v.z, v.w);
       }
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
       const int chunk = tid + 256 * i;
-      const int m = chunk >> 3, k = k0 + 8 * (chunk & 7);
+      const int m = chunk >> 3;
+      const int64_t k = k0 + 16 * (chunk & 7);
       x_next[i] = make_uint4(0, 0, 0, 0);
-      if (m < M && k < k_end) x_next[i] = *reinterpret_cast<const uint4*>(x + static_cast<int64_t>(m) * ldx + k);
+      if (m < M && k < k_end) x_next[i] = *reinterpret_cast<const uint4*>(x + m * ldx_bytes + k);
     }
   };
   auto stash = [&]() {
@@ -451,20 +454,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const uint16_t* _
     }
   };
 
-  f32x16 acc[MT] = {};
+  using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
+  Acc acc[MT] = {};
   fetch(k_begin);
-  for (int k0 = k_begin; k0 < k_end; k0 += kSkinnyChunk) {
+  for (int64_t k0 = k_begin; k0 < k_end; k0 += kSkinnyChunkBytes) {
     __syncthreads();                                 // every wave is done with the previous tiles
     stash();
     __syncthreads();
-    if (k0 + kSkinnyChunk < k_end) fetch(k0 + kSkinnyChunk);
+    if (k0 + kSkinnyChunkBytes < k_end) fetch(k0 + kSkinnyChunkBytes);
 #pragma unroll
-    for (int kk = 0; kk < kSkinnyChunk / 16; ++kk) {
-      const bf16x8 fb = *reinterpret_cast<const bf16x8*>(tile_w + (wave * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
+    for (int kk = 0; kk < kSkinnyChunkBytes / 32; ++kk) {
+      const uint8_t* at_w = tile_w + (wave * 32 + frag_row) * kRowStride + kk * 32 + frag_k;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const bf16x8 fa = *reinterpret_cast<const bf16x8*>(tile_x + (t * 32 + frag_row) * kRowStride + kk * 32 + frag_k);
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[t], 0, 0, 0);
+        const uint8_t* at_x = tile_x + (t * 32 + frag_row) * kRowStride + kk * 32 + frag_k;
+        if constexpr (INT8) {
+          acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const i32x4*>(at_x), *reinterpret_cast<const i32x4*>(at_w), acc[t], 0, 0, 0);
+        } else {
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(at_x), *reinterpret_cast<const bf16x8*>(at_w), acc[t], 0, 0, 0);
+        }
       }
     }
   }
@@ -472,7 +480,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const uint16_t* _
   // Register r of lane l holds activation row 8 (r / 4) + 4 (l / 32) + r % 4 of its tile, weight row l % 32.
   const int n = n0 + wave * 32 + frag_row;
   if (n >= N) return;
-  float* slab = partial + static_cast<int64_t>(blockIdx.y) * M * N;
+  using Cell = typename std::conditional<INT8, int32_t, float>::type;
+  Cell* slab = static_cast<Cell*>(partial) + static_cast<int64_t>(blockIdx.y) * M * N;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
 #pragma unroll
@@ -483,26 +492,63 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const uint16_t* _
   }
 }
 
-__global__ __launch_bounds__(256) void gemm_skinny_finish_kernel(const float* __restrict__ partial, int slices, const void* __restrict__ bias,
+// Adds the K slices. bf16 product: f32 sums + bias, one rounding. int8 product: int32 sums are exact, then
+// f32(sum) * sa[m] * sb[n] + bias as single rounded operations (the same epilogue as the tiled kernels).
+template <bool INT8>
+__global__ __launch_bounds__(256) void gemm_skinny_finish_kernel(const void* __restrict__ partial, int slices, const float* __restrict__ scale_a,
+                                                                 const float* __restrict__ scale_b, const void* __restrict__ bias,
                                                                  void* __restrict__ y, int M, int N, int64_t ldy, int out_kind) {
   const int64_t cell = blockIdx.x * int64_t{256} + threadIdx.x;
   if (cell >= static_cast<int64_t>(M) * N) return;
   const int m = static_cast<int>(cell / N), n = static_cast<int>(cell % N);
-  float sum = 0.0f;
-  for (int s = 0; s < slices; ++s) sum += partial[static_cast<int64_t>(s) * M * N + cell];
-  if (bias != nullptr) sum += load_bias(bias, out_kind, n);
-  store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, sum);
+  float v;
+  if constexpr (INT8) {
+    int32_t sum = 0;
+    for (int s = 0; s < slices; ++s) sum += static_cast<const int32_t*>(partial)[static_cast<int64_t>(s) * M * N + cell];
+    v = __fmul_rn(__fmul_rn(static_cast<float>(sum), scale_a[m]), scale_b[n]);
+    if (bias != nullptr) v = __fadd_rn(v, load_bias(bias, out_kind, n));
+  } else {
+    v = 0.0f;
+    for (int s = 0; s < slices; ++s) v += static_cast<const float*>(partial)[static_cast<int64_t>(s) * M * N + cell];
+    if (bias != nullptr) v += load_bias(bias, out_kind, n);
+  }
+  store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, v);
 }
 
-// K slices for M x N x K on `cus` compute units: enough blocks for about four per CU, at least one chunk each.
-static int skinny_slices(int64_t N, int64_t K, int cus) {
+// K slices for an M x N product with `k_bytes` bytes per row on `cus` compute units: enough blocks for about four
+// per CU, at least one chunk each.
+static int skinny_slices(int64_t N, int64_t k_bytes, int cus) {
   const int64_t n_blocks = (N + kSkinnyBlockN - 1) / kSkinnyBlockN;
-  const int64_t chunks = (K + kSkinnyChunk - 1) / kSkinnyChunk;
+  const int64_t chunks = (k_bytes + kSkinnyChunkBytes - 1) / kSkinnyChunkBytes;
   int64_t slices = (4 * static_cast<int64_t>(cus) + n_blocks - 1) / n_blocks;
   slices = slices < 1 ? 1 : (slices > chunks ? chunks : slices);
   slices = slices > 64 ? 64 : slices;
   const int64_t per = (chunks + slices - 1) / slices;
   return static_cast<int>((chunks + per - 1) / per);
+}
+
+template <bool INT8>
+static int launch_skinny(const void* x, const void* w, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
+                         int64_t N, int64_t k_bytes, int64_t ldx_bytes, int64_t ldw_bytes, int64_t ldy, int out_kind, int cus,
+                         void* workspace, size_t workspace_bytes, hipStream_t s) {
+  const int slices = skinny_slices(N, k_bytes, cus);
+  if (workspace_bytes < static_cast<size_t>(slices) * static_cast<size_t>(M) * static_cast<size_t>(N) * 4) return EP_HIP_EINVAL;
+  const int chunks = static_cast<int>((k_bytes + kSkinnyChunkBytes - 1) / kSkinnyChunkBytes);
+  const int per = (chunks + slices - 1) / slices;
+  const dim3 grid(static_cast<unsigned>((N + kSkinnyBlockN - 1) / kSkinnyBlockN), static_cast<unsigned>(slices));
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  const uint8_t* wb = static_cast<const uint8_t*>(w);
+  const int m = static_cast<int>(M), n = static_cast<int>(N);
+  if (M <= 32) hipLaunchKernelGGL((gemm_skinny_kernel<1, INT8>), grid, dim3(256), 0, s, xb, wb, workspace, m, n, k_bytes, ldx_bytes, ldw_bytes, per);
+  else if (M <= 64) hipLaunchKernelGGL((gemm_skinny_kernel<2, INT8>), grid, dim3(256), 0, s, xb, wb, workspace, m, n, k_bytes, ldx_bytes, ldw_bytes, per);
+  else if (M <= 96) hipLaunchKernelGGL((gemm_skinny_kernel<3, INT8>), grid, dim3(256), 0, s, xb, wb, workspace, m, n, k_bytes, ldx_bytes, ldw_bytes, per);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<4, INT8>), grid, dim3(256), 0, s, xb, wb, workspace, m, n, k_bytes, ldx_bytes, ldw_bytes, per);
+  EP_HIP_TRY(hipGetLastError());
+  const int64_t cells = M * N;
+  hipLaunchKernelGGL(gemm_skinny_finish_kernel<INT8>, dim3(static_cast<unsigned>((cells + 255) / 256)), dim3(256), 0, s, workspace, slices,
+                     scale_a, scale_b, bias, y, m, n, ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
 }
 
 static int out_kind_valid(int kind) { return kind == kOutBF16 || kind == kOutF16 || kind == kOutF32; }
@@ -532,10 +578,10 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   return EP_HIP_OK;
 }
 
-size_t ep_hip_gemm_bf16_skinny_workspace(int64_t M, int64_t N, int64_t K, int compute_units) {
+size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units) {
   using namespace ep;
-  if (M <= 0 || N <= 0 || K <= 0 || compute_units <= 0) return 0;
-  return static_cast<size_t>(skinny_slices(N, K, compute_units)) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+  if (M <= 0 || N <= 0 || k_bytes <= 0 || compute_units <= 0) return 0;
+  return static_cast<size_t>(skinny_slices(N, k_bytes, compute_units)) * static_cast<size_t>(M) * static_cast<size_t>(N) * 4;
 }
 
 int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
@@ -543,32 +589,30 @@ int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bi
                             void* workspace_dev, size_t workspace_bytes, void* stream) {
   using namespace ep;
   if (x_dev == nullptr || w_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
-  if (M <= 0 || N <= 0 || K <= 0 || N > 0x7FFFFFFF || K > 0x7FFFFFFF - kSkinnyChunk || compute_units <= 0) return EP_HIP_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0 || N > 0x7FFFFFFF || K > 0x3FFFFFFF || compute_units <= 0) return EP_HIP_EINVAL;
   if (M > 128) return EP_HIP_EUNSUPPORTED;
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  const int slices = skinny_slices(N, K, compute_units);
-  if (workspace_bytes < static_cast<size_t>(slices) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float)) return EP_HIP_EINVAL;
-  const int chunks = static_cast<int>((K + kSkinnyChunk - 1) / kSkinnyChunk);
-  const int per = (chunks + slices - 1) / slices;
-  const dim3 grid(static_cast<unsigned>((N + kSkinnyBlockN - 1) / kSkinnyBlockN), static_cast<unsigned>(slices));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const uint16_t* x = static_cast<const uint16_t*>(x_dev);
-  const uint16_t* w = static_cast<const uint16_t*>(w_dev);
-  float* partial = static_cast<float*>(workspace_dev);
-  const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-  if (M <= 32) hipLaunchKernelGGL(gemm_bf16_skinny_kernel<1>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
-  else if (M <= 64) hipLaunchKernelGGL(gemm_bf16_skinny_kernel<2>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
-  else if (M <= 96) hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
-  else hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, dim3(256), 0, s, x, w, partial, m, n, k, ldx, ldw, per);
-  EP_HIP_TRY(hipGetLastError());
-  const int64_t cells = M * N;
-  hipLaunchKernelGGL(gemm_skinny_finish_kernel, dim3(static_cast<unsigned>((cells + 255) / 256)), dim3(256), 0, s, partial, slices, bias_dev,
-                     y_dev, m, n, ldy, out_kind);
-  EP_HIP_TRY(hipGetLastError());
-  return EP_HIP_OK;
+  return launch_skinny<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, compute_units,
+                              workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int ep_hip_gemm_i8_skinny(const int8_t* a_dev, const int8_t* b_dev, const float* scale_a_dev, const float* scale_b_dev,
+                          const void* bias_dev, void* y_dev, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                          int64_t ldy, int out_kind, int compute_units, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  using namespace ep;
+  if (a_dev == nullptr || b_dev == nullptr || scale_a_dev == nullptr || scale_b_dev == nullptr || y_dev == nullptr ||
+      workspace_dev == nullptr) return EP_HIP_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0 || N > 0x7FFFFFFF || K > 0x7FFFFFFF || compute_units <= 0) return EP_HIP_EINVAL;
+  if (M > 128) return EP_HIP_EUNSUPPORTED;
+  if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0) return EP_HIP_EINVAL;
+  if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  return launch_skinny<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, compute_units,
+                             workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_a_dev, const float* scale_b_dev,

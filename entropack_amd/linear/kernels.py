@@ -46,7 +46,7 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
         with torch.cuda.device(device):
             lib = _hip.library()
             cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
-            workspace = torch.empty(lib.ep_hip_gemm_bf16_skinny_workspace(rows, outer, inner, cus), dtype=torch.uint8, device=device)
+            workspace = torch.empty(lib.ep_hip_gemm_skinny_workspace(rows, outer, inner * 2, cus), dtype=torch.uint8, device=device)
             _hip.check("ep_hip_gemm_bf16_skinny", lib.ep_hip_gemm_bf16_skinny(
                 flat.data_ptr(), w.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(),
                 rows, outer, inner, flat.stride(0), w.stride(0), out.stride(0), _hip.FLOAT_KINDS[out_dtype], cus,
@@ -99,10 +99,20 @@ def int8_gemm(activation: torch.Tensor, codes: torch.Tensor, activation_scale: t
     if rows == 0:
         return out
     bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
+    scale_a, scale_b = activation_scale.float().contiguous(), weight_scale.float().contiguous()
+    if rows <= SKINNY_MAX_ROWS:
+        with torch.cuda.device(device):
+            lib = _hip.library()
+            cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
+            workspace = torch.empty(lib.ep_hip_gemm_skinny_workspace(rows, outer, a.shape[1], cus), dtype=torch.uint8, device=device)
+            _hip.check("ep_hip_gemm_i8_skinny", lib.ep_hip_gemm_i8_skinny(
+                a.data_ptr(), b.data_ptr(), scale_a.data_ptr(), scale_b.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(),
+                out.data_ptr(), rows, outer, a.shape[1], a.stride(0), b.stride(0), out.stride(0), _hip.FLOAT_KINDS[out_dtype], cus,
+                workspace.data_ptr(), workspace.numel(), _hip.current_stream(device)))
+        return out
     with torch.cuda.device(device):
         _hip.check("ep_hip_gemm_i8", _hip.library().ep_hip_gemm_i8(
-            a.data_ptr(), b.data_ptr(), activation_scale.float().contiguous().data_ptr(),
-            weight_scale.float().contiguous().data_ptr(), None if bias_ready is None else bias_ready.data_ptr(),
+            a.data_ptr(), b.data_ptr(), scale_a.data_ptr(), scale_b.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(),
             out.data_ptr(), rows, outer, a.shape[1], a.stride(0), b.stride(0), out.stride(0),
             _hip.FLOAT_KINDS[out_dtype], _hip.current_stream(device)))
     return out

@@ -176,16 +176,21 @@ enum ep_hip_float_kind { EP_FLOAT_BF16 = 0, EP_FLOAT_F16 = 1, EP_FLOAT_F32 = 2 }
 int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
                      int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, void* stream);
 
-/* The same product for at most 128 activation rows, where reading W once bounds the time: K is split over blocks so
- * that every CU streams weights, partial sums go to `workspace_dev` (f32, 16-byte aligned, at least
- * ep_hip_gemm_bf16_skinny_workspace(M, N, K, compute_units) bytes, contents irrelevant on entry) and a second kernel
- * adds them and the bias and rounds once. Same operand rules as ep_hip_gemm_bf16; M > 128 returns
- * EP_HIP_EUNSUPPORTED. Reference: the F.linear call of CompressedLinear.forward at small batch,
- * entropack/linear/linear.py:163-165. */
-size_t ep_hip_gemm_bf16_skinny_workspace(int64_t M, int64_t N, int64_t K, int compute_units);
+/* The same products for at most 128 activation rows, where reading W once bounds the time: K is split over blocks so
+ * that every CU streams weights, partial sums (f32, or exact int32 for the int8 product) go to `workspace_dev`
+ * (16-byte aligned, at least ep_hip_gemm_skinny_workspace(M, N, bytes of one row of K, compute_units) bytes, contents
+ * irrelevant on entry) and a second kernel adds them, applies the same epilogue as ep_hip_gemm_bf16 / ep_hip_gemm_i8
+ * and rounds once. Same operand rules as those; M > 128 returns EP_HIP_EUNSUPPORTED. Reference: the F.linear call of
+ * CompressedLinear.forward and the int8 GEMM of CompressedINT8Linear at small batch, entropack/linear/linear.py:163-165,
+ * 485-490. */
+size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units);
 int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
                             int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, int compute_units,
                             void* workspace_dev, size_t workspace_bytes, void* stream);
+int ep_hip_gemm_i8_skinny(const int8_t* a_dev, const int8_t* b_dev, const float* scale_a_dev, const float* scale_b_dev,
+                          const void* bias_dev, void* y_dev, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                          int64_t ldy, int out_kind, int compute_units, void* workspace_dev, size_t workspace_bytes,
+                          void* stream);
 
 /* y[M][N] = (a[M][K] . b[N][K]^T)_int32 -> f32 * scale_a[m] * scale_b[n] (+ bias[n]) -> out_kind. K a multiple of 16.
  * Reference: int8_gemm / _int8_gemm_kernel, entropack/linear/quant_kernels.py:15-54,81-93. */

@@ -87,7 +87,8 @@ def test_quantize_rows_is_exact(rows, inner, dtype):
     assert codes[0].abs().max() == 0
 
 
-@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040), (4100, 4200, 528)])
+@pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040), (4100, 4200, 528), (1, 300, 4112), (128, 1000, 28672),
+                                   (33, 257, 16)])
 def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
     print("case", shape, flush=True)
     m, n, k = shape
