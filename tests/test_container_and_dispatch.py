@@ -234,3 +234,37 @@ def test_plan_describe_rejects_inconsistent_tables():
     wide_only = Golden("huge_alpha_16x1024_bf16_7p0")
     assert _describe(wide_only.buffers["stream_meta"], wide_only.buffers["freq_tables"], 11,
                      force=hip_backend.TABLE_LDS_BYTE)[0] == hip_backend.EUNSUPPORTED
+
+
+def test_launch_table_form_depends_on_the_launch_size():
+    """A byte-valued prob_bits-11 plan decodes small containers with its slot tables and large ones (more tile pairs
+    than 16 waves on every CU hold) with its two-level section; other plans never switch. Pure host logic."""
+    lib = hip_backend.library()
+    golden = Golden("c1_256x256_bf16_3p5")
+    _, desc = _describe(golden.buffers["stream_meta"], golden.buffers["freq_tables"], 11, tile_elements=16384)
+    assert desc.table_kind == hip_backend.TABLE_LDS_BYTE and desc.sym_offset != 0
+    bf16, int8, f32 = (hip_backend.STORE_KINDS[t] for t in (torch.bfloat16, torch.int8, torch.float32))
+    kind = lambda d, store, rows, cols, cus=256: lib.ep_hip_decode_table_kind(ctypes.byref(d), store, rows, cols, 16384, cus)
+    assert kind(desc, bf16, 256, 256) == hip_backend.TABLE_LDS_BYTE
+    assert kind(desc, bf16, 8192, 28672) == hip_backend.TABLE_LDS_SYM          # 8066 pairs > 256 * 16
+    assert kind(desc, int8, 8192, 28672) == hip_backend.TABLE_LDS_SYM
+    assert kind(desc, f32, 8192, 28672) == hip_backend.TABLE_LDS_SYM
+    assert kind(desc, bf16, 4096, 28672) == hip_backend.TABLE_LDS_BYTE         # 4033 pairs: one pass of resident waves
+    assert kind(desc, bf16, 4096, 28672, 64) == hip_backend.TABLE_LDS_SYM      # ... on a quarter of the CUs it is not
+    assert kind(desc, bf16, 0, 256) == -1
+    _, forced = _describe(golden.buffers["stream_meta"], golden.buffers["freq_tables"], 11, force=hip_backend.TABLE_LDS_SYM)
+    assert forced.table_kind == hip_backend.TABLE_LDS_SYM and kind(forced, bf16, 256, 256) == hip_backend.TABLE_LDS_SYM
+    wide = Golden("huge_alpha_16x1024_bf16_7p0")
+    _, wide_desc = _describe(wide.buffers["stream_meta"], wide.buffers["freq_tables"], 11)
+    assert wide_desc.sym_offset == 0 and kind(wide_desc, bf16, 8192, 28672) == hip_backend.TABLE_LDS_WIDE
+    assert _describe(wide.buffers["stream_meta"], wide.buffers["freq_tables"], 11, force=hip_backend.TABLE_LDS_SYM)[0] == hip_backend.EUNSUPPORTED
+
+
+def test_skinny_gemm_workspace_matches_its_split():
+    """Workspace = K slices x M x N x 4 bytes; slices aim at four blocks per CU and never exceed the 128-byte chunks of a row."""
+    lib = hip_backend.library()
+    size = lib.ep_hip_gemm_skinny_workspace
+    assert size(16, 8192, 28672 * 2, 256) == 16 * 16 * 8192 * 4                # 64 row blocks -> 16 slices
+    assert size(1, 128, 256, 256) == 2 * 1 * 128 * 4                           # only two chunks to split
+    assert size(128, 100000, 4096, 256) == 2 * 128 * 100000 * 4                # already enough row blocks: (1024 + 781) / 782 = 2
+    assert size(0, 10, 10, 256) == 0 and size(4, 10, 10, 0) == 0
