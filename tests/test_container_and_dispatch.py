@@ -261,10 +261,19 @@ def test_launch_table_form_depends_on_the_launch_size():
 
 
 def test_skinny_gemm_workspace_matches_its_split():
-    """Workspace = K slices x M x N x 4 bytes; slices aim at four blocks per CU and never exceed the 128-byte chunks of a row."""
-    lib = hip_backend.library()
-    size = lib.ep_hip_gemm_skinny_workspace
+    """Workspace = K slices x M x N x 4 bytes. A block owns 128 weight rows; slices aim at four blocks per CU, never exceed
+    the 128-byte chunks of a row or 64, and are evened out."""
+    size = hip_backend.library().ep_hip_gemm_skinny_workspace
+
+    def expect(m, n, k_bytes, cus):
+        rows = 128
+        blocks, chunks = -(-n // rows), -(-k_bytes // 128)
+        slices = max(1, min(-(-4 * cus // blocks), chunks, 64))
+        per = -(-chunks // slices)
+        return -(-chunks // per) * m * n * 4
+
     assert size(16, 8192, 28672 * 2, 256) == 16 * 16 * 8192 * 4                # 64 row blocks -> 16 slices
     assert size(1, 128, 256, 256) == 2 * 1 * 128 * 4                           # only two chunks to split
-    assert size(128, 100000, 4096, 256) == 2 * 128 * 100000 * 4                # already enough row blocks: (1024 + 781) / 782 = 2
+    for case in [(16, 8192, 57344, 256), (128, 8192, 57344, 256), (128, 100000, 4096, 256), (65, 300, 1 << 20, 256), (3, 77, 16, 8)]:
+        assert size(*case) == expect(*case), case
     assert size(0, 10, 10, 256) == 0 and size(4, 10, 10, 0) == 0
