@@ -7,6 +7,7 @@
  *   hc_quantize      entropack/schemes/lattice_rans/eager.py:18-51  (nearest E8 point, point -> coset + fields)
  *   hc_levels        entropack/schemes/lattice_rans/eager.py:54-58  (fields -> point)
  *   hc_rans_encode   entropack/schemes/lattice_rans/rans.py:133-186 (tiled 32-way interleaved rANS encode)
+ *   hc_tile_ans_encode  entropack/schemes/tile_ans/eager.py:145-228 (byte-lane streams: raw words or 32-way rANS)
  * Built with -ffp-contract=off: every float operation below is a single IEEE operation, as in the reference.
  */
 #include <math.h>
@@ -222,6 +223,79 @@ int hc_rans_encode(const int8_t* coset, const int32_t* fields, int64_t vectors, 
   }
   for (int64_t tile = 0; tile < tiles; ++tile) free(lists[tile].words);
   free(lists);
+  *payload = joined;
+  return failed == 0 ? 0 : (failed == 2 ? -2 : -1);
+}
+
+/* Lossless byte-lane coder. `bytes` is the tensor's storage, num_elements x num_lanes bytes; stream (lane, tile)
+ * covers byte `lane` of elements [tile * tile_elements, ...). A raw lane stores its bytes two per word (even element in
+ * the low byte); a coded lane runs 32 interleaved rANS states over its symbols in order, group after group of 32.
+ * freq / cdf: u16[num_lanes][256]. states: u32[tiles * coded lanes][32], coded lanes in lane order; offsets:
+ * u32[num_lanes * tiles + 1]; *payload: malloc'd (hc_free). Returns 0, -1 out of memory, -2 payload beyond 32-bit offsets. */
+int hc_tile_ans_encode(const uint8_t* bytes, int64_t num_elements, int num_lanes, int64_t tile_elements, int prob_bits,
+                       const uint16_t* freq, const uint16_t* cdf, const uint8_t* lane_raw, uint32_t* states,
+                       uint32_t* offsets, uint16_t** payload, int threads) {
+  const int64_t tiles = (num_elements + tile_elements - 1) / tile_elements;
+  const int64_t streams = tiles * num_lanes;
+  word_list* lists = (word_list*)calloc((size_t)streams, sizeof(word_list));
+  int* coded_before = (int*)calloc((size_t)num_lanes + 1, sizeof(int));
+  if (!lists || !coded_before) { free(lists); free(coded_before); return -1; }
+  for (int lane = 0; lane < num_lanes; ++lane) coded_before[lane + 1] = coded_before[lane] + (lane_raw[lane] ? 0 : 1);
+  int failed = 0;
+#pragma omp parallel for schedule(dynamic, 8) num_threads(threads > 0 ? threads : 1)
+  for (int64_t stream = 0; stream < streams; ++stream) {
+    const int lane = (int)(stream / tiles);
+    const int64_t tile = stream % tiles;
+    const int64_t begin = tile * tile_elements;
+    const int64_t end = begin + tile_elements < num_elements ? begin + tile_elements : num_elements;
+    word_list* out = &lists[stream];
+    int bad = 0;
+    if (lane_raw[lane]) {
+      for (int64_t e = begin; e < end && !bad; e += 2) {
+        uint16_t word = bytes[e * num_lanes + lane];
+        if (e + 1 < end) word |= (uint16_t)(bytes[(e + 1) * num_lanes + lane] << 8);
+        if (push_word(out, word)) bad = 1;
+      }
+    } else {
+      uint32_t x[HC_STATES];
+      for (int l = 0; l < HC_STATES; ++l) x[l] = HC_STATE_MIN;
+      const uint16_t* f = freq + lane * 256;
+      const uint16_t* c = cdf + lane * 256;
+      for (int64_t base = begin; base < end && !bad; base += HC_STATES) {
+        const int lanes = (int)(end - base < HC_STATES ? end - base : HC_STATES);
+        for (int l = 0; l < lanes; ++l) {
+          const uint8_t symbol = bytes[(base + l) * num_lanes + lane];
+          if (put(&x[l], f[symbol], c[symbol], prob_bits, out)) { bad = 1; break; }
+        }
+      }
+      memcpy(states + ((int64_t)coded_before[lane] * tiles + tile) * HC_STATES, x, sizeof(x));
+    }
+    if (bad) {
+#pragma omp atomic write
+      failed = 1;
+    }
+  }
+  uint64_t total = 0;
+  offsets[0] = 0;
+  for (int64_t stream = 0; stream < streams; ++stream) {
+    total += lists[stream].size;
+    if (total > 0xFFFFFFFFull) failed = 2;
+    offsets[stream + 1] = (uint32_t)total;
+  }
+  uint16_t* joined = NULL;
+  if (!failed) {
+    joined = (uint16_t*)malloc((total ? total : 1) * sizeof(uint16_t));
+    if (!joined) failed = 1;
+  }
+  if (!failed) {
+#pragma omp parallel for schedule(static) num_threads(threads > 0 ? threads : 1)
+    for (int64_t stream = 0; stream < streams; ++stream) {
+      if (lists[stream].size) memcpy(joined + offsets[stream], lists[stream].words, lists[stream].size * sizeof(uint16_t));
+    }
+  }
+  for (int64_t stream = 0; stream < streams; ++stream) free(lists[stream].words);
+  free(lists);
+  free(coded_before);
   *payload = joined;
   return failed == 0 ? 0 : (failed == 2 ? -2 : -1);
 }

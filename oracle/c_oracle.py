@@ -21,7 +21,7 @@ ERRORS = {1: "bad argument", 2: "payload truncated", 3: "tile not fully consumed
 
 
 def build() -> str:
-    subprocess.run(["make", "-C", _HERE, "-B", "liblattice_oracle.so"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE, "-B", "all"], check=True, capture_output=True)
     return _LIB_PATH
 
 
@@ -89,4 +89,42 @@ def decode(buffers: dict, shape, dtype: str, threads: int = 1) -> np.ndarray:
     _check(load().orc_decode(
         _ptr(b["payload"]), _ptr(b["offsets"]), _ptr(b["states"]), _ptr(b["stream_meta"]), _ptr(b["freq_tables"]),
         _ptr(b["scales"]), rows, cols, prob_bits, tile_elements, kind, _ptr(out), int(threads)))
+    return out
+
+
+# ---- tile_ans (lossless) ---------------------------------------------------------------------------------------------
+
+_TILE_LIB_PATH = os.path.join(_HERE, "libtile_ans_oracle.so")
+_tile_lib = None
+TILE_ERRORS = {1: "bad argument", 2: "payload truncated", 3: "payload contains unread words", 4: "raw lane payload length is invalid"}
+
+
+def load_tile_ans():
+    global _tile_lib
+    if _tile_lib is None:
+        if not os.path.exists(_TILE_LIB_PATH):
+            build()
+        lib = ctypes.CDLL(_TILE_LIB_PATH)
+        p = ctypes.c_void_p
+        lib.tao_decode.argtypes = [p, p, p, p, p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64, p, ctypes.c_int]
+        lib.tao_decode.restype = ctypes.c_int
+        _tile_lib = lib
+    return _tile_lib
+
+
+def tile_ans_decode(buffers: dict, element_bytes: int, threads: int = 1) -> np.ndarray:
+    """Storage bytes (uint8[elements * element_bytes]) of a tile_ans container given as numpy buffers."""
+    payload = np.ascontiguousarray(buffers["payload"]).view(np.uint16) if np.asarray(buffers["payload"]).size else np.zeros(1, np.uint16)
+    offsets = np.ascontiguousarray(buffers["offsets"]).astype(np.uint32)
+    states = np.ascontiguousarray(buffers["states"]).astype(np.uint32).reshape(-1) if np.asarray(buffers["states"]).size else np.zeros(32, np.uint32)
+    tables = np.ascontiguousarray(buffers["decode_tables"]).astype(np.uint32)
+    modes = np.ascontiguousarray(buffers["lane_modes"]).astype(np.uint8)
+    tile_elements, prob_bits, lanes, elements = (int(v) for v in np.asarray(buffers["layout"]))
+    if lanes != element_bytes:
+        raise ValueError("layout does not match the element size")
+    out = np.empty(elements * lanes, dtype=np.uint8)
+    rc = load_tile_ans().tao_decode(_ptr(payload), _ptr(offsets), _ptr(states), _ptr(tables), _ptr(modes), tile_elements, prob_bits, lanes,
+                                    elements, _ptr(out), int(threads))
+    if rc:
+        raise ValueError(f"tile_ans oracle: {TILE_ERRORS.get(rc, rc)}")
     return out
