@@ -82,6 +82,9 @@ _SIGNATURES = {
         ctypes.c_void_p, ctypes.c_void_p]),
     "ep_hip_decode_table_kind": (ctypes.c_int, [
         ctypes.POINTER(PlanDesc), ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int]),
+    "ep_hip_decode_tile_ans": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "ep_hip_batch_plan": (ctypes.c_int, [
         ctypes.POINTER(DecodeJob), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_size_t)]),
     "ep_hip_decode_lattice_batch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),

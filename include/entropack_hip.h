@@ -131,6 +131,20 @@ int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, c
 int ep_hip_decode_table_kind(const ep_hip_plan_desc* desc, int store_kind, int64_t rows, int64_t cols_padded,
                              int tile_elements, int compute_units);
 
+/* Lossless decode ----------------------------------------------------------------------------------------------- */
+
+/* Decodes a tile_ans container (payload u16[W], offsets u32[lanes * tiles + 1], states u32[tiles * coded lanes][32],
+ * decode_tables u32[lanes][2^prob_bits], layout = tile_elements, prob_bits, lanes, elements) into `out_dev`, the
+ * tensor's storage (elements * lanes bytes, element-aligned). `lane_modes_host` is a host copy of the container's
+ * lane_modes (0 = coded, 1 = raw); lanes is 1, 2, 4 or 8. `error_dev` as for ep_hip_decode_lattice (a stream that
+ * ends with unread words reports 3, one that runs out 2, bad offsets / raw lengths 4).
+ * Reference: decode() and the tile_ans_decode_* kernels it launches, entropack/schemes/tile_ans/cuda.py:117-170,
+ * tile_ans.cu:175-470. */
+int ep_hip_decode_tile_ans(const uint16_t* payload_dev, uint64_t payload_words, const uint32_t* offsets_dev,
+                           const uint32_t* states_dev, const uint32_t* decode_tables_dev,
+                           const uint8_t* lane_modes_host, int64_t tile_elements, int prob_bits, int num_lanes,
+                           int64_t num_elements, void* out_dev, int32_t* error_dev, void* stream);
+
 /* Batched decode --------------------------------------------------------------------------------------------- */
 
 /* One container of a batch: the arguments of ep_hip_decode_lattice, with the output given as a byte offset

@@ -1,0 +1,119 @@
+"""GPU parity for the lossless `tile_ans` decode: the HIP lane against the reference-written fixtures and, on containers
+this package's encoder wrote (byte-identical to the reference's on the fixtures), against the input itself and the
+CPU oracle, from one element to 8192 x 28672."""
+import numpy as np
+import pytest
+import torch
+
+import entropack_amd as ep
+from entropack_amd.schemes.base import packed_buffers
+from entropack_amd.schemes.tile_ans import hip as tile_lane
+from entropack_amd.schemes.tile_ans.format import TileBuffers
+from oracle import c_oracle
+from test_tile_ans_golden import TileGolden, tile_names
+
+pytestmark = pytest.mark.gpu
+
+_BITS = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+
+
+def bits_of(tensor):
+    tensor = tensor.detach().contiguous()
+    if tensor.dtype == torch.bool:
+        return tensor.to(torch.uint8).cpu().numpy()
+    return tensor.view(_BITS[tensor.element_size()]).cpu().numpy()
+
+
+@pytest.mark.parametrize("name", tile_names())
+def test_decompress_matches_reference_bits(name):
+    print("case", name, flush=True)
+    golden = TileGolden(name)
+    container = ep.CompressedTensor.unpack(torch.from_numpy(golden.quant_state.copy()).cuda())
+    restored = ep.decompress(container, ep.TileANSConfig(execution_backend="hip"))
+    torch.cuda.synchronize()
+    tile_lane.check_errors(packed_buffers(container.buffers, TileBuffers))
+    assert restored.shape == golden.shape and restored.dtype == golden.dtype and restored.device.type == "cuda"
+    want = golden.weight_bits if golden.dtype != torch.bool else golden.weight_bits.astype(np.uint8)
+    assert np.array_equal(bits_of(restored), want.reshape(golden.shape))
+
+
+def round_trip(tensor, **options):
+    container = ep.compress(tensor, ep.TileANSConfig(execution_backend="eager", **options))
+    assert container.compress_method == "tile_ans"
+    on_gpu = container.to("cuda")
+    restored = ep.decompress(on_gpu, ep.TileANSConfig())            # "auto" resolves to hip on this box
+    torch.cuda.synchronize()
+    tile_lane.check_errors(packed_buffers(on_gpu.buffers, TileBuffers))
+    assert restored.shape == tensor.shape and restored.dtype == tensor.dtype
+    assert np.array_equal(bits_of(restored), bits_of(tensor))
+    return container
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.int8, torch.uint8, torch.int16, torch.int32,
+                                   torch.int64, torch.bool, torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("shape", [(1,), (31,), (33, 3), (257, 129), (5, 4096), (3, 8192 + 17)])
+def test_round_trip_every_dtype_and_ragged_sizes(dtype, shape):
+    print("case", dtype, shape, flush=True)
+    torch.manual_seed(hash((str(dtype), shape)) % 1000)
+    if dtype == torch.bool:
+        tensor = torch.rand(*shape) < 0.3
+    elif dtype.is_floating_point:
+        tensor = (torch.randn(*shape) * 0.05).to(dtype)
+    else:
+        tensor = (torch.randn(*shape) * 40).round().clamp(-120, 120).to(dtype) if dtype != torch.uint8 else torch.randint(0, 40, shape, dtype=dtype)
+    round_trip(tensor)
+
+
+@pytest.mark.parametrize("options", [dict(tile_elements=400), dict(tile_elements=4096, probability_bits=12), dict(probability_bits=9),
+                                     dict(raw_lane_threshold=0.0), dict(raw_lane_threshold=8.0, tile_elements=2048)])
+def test_round_trip_across_options(options):
+    print("case", options, flush=True)
+    torch.manual_seed(77)
+    container = round_trip((torch.randn(300, 517) * 0.02).to(torch.bfloat16), **options)
+    if options.get("raw_lane_threshold") == 0.0:
+        assert container.buffers["lane_modes"].tolist() == [1, 1]          # nothing coded: a plain unpacking of the words
+    steps = torch.randint(-300, 300, (123, 77), dtype=torch.int16) * 16        # both byte lanes coded
+    container = round_trip(steps, **options)
+    if options.get("raw_lane_threshold", 7.9) > 0.0:
+        assert container.buffers["lane_modes"].tolist() == [0, 0]
+
+
+def test_model_weight_sizes_match_the_oracle_and_the_input():
+    """A 4096 x 4096 bf16 weight (8192-element tiles, raw low byte + coded high byte) and a float32 one, against the oracle."""
+    for dtype, shape in ((torch.bfloat16, (4096, 4096)), (torch.float32, (1024, 3072)), (torch.int8, (2048, 4096))):
+        print("case", dtype, shape, flush=True)
+        torch.manual_seed(5)
+        tensor = (torch.randn(*shape) * 0.02).to(dtype) if dtype.is_floating_point else (torch.randn(*shape) * 30).round().clamp(-127, 127).to(dtype)
+        container = round_trip(tensor)
+        host = {}
+        for key, value in container.buffers.items():
+            if value.dtype in (torch.uint16, torch.uint32):
+                signed = value.view(torch.int16 if value.dtype == torch.uint16 else torch.int32).numpy()
+                host[key] = signed.view(np.uint16 if value.dtype == torch.uint16 else np.uint32)
+            else:
+                host[key] = value.numpy()
+        expect = c_oracle.tile_ans_decode(host, tensor.element_size(), threads=8)
+        assert np.array_equal(expect, tensor.contiguous().view(torch.uint8).numpy().reshape(-1))
+        ratio = container.storage_nbytes() / (tensor.numel() * tensor.element_size())
+        assert ratio < 0.9                                                    # gaussian weights do compress (float32: 0.84)
+
+
+def test_full_size_8192x28672_bf16_is_lossless():
+    torch.manual_seed(4)
+    tensor = (torch.randn(8192, 28672) * 0.015).to(torch.bfloat16)
+    container = round_trip(tensor)
+    assert container.buffers["lane_modes"].tolist() == [1, 0] and int(container.buffers["layout"][0]) == 8192
+
+
+def test_corrupt_stream_sets_the_error_flag_and_stays_in_bounds():
+    golden = TileGolden("int8_128x100_auto")
+    container = ep.CompressedTensor.unpack(torch.from_numpy(golden.quant_state.copy()).cuda())
+    buffers = dict(container.buffers)
+    states = buffers["states"].clone()
+    states.view(torch.int32)[0, 3] += 12345                                   # a wrong initial state derails that lane
+    buffers["states"] = states
+    lattice = TileBuffers(**buffers)
+    tile_lane.decode(lattice, dtype=torch.int8)
+    with pytest.raises(ValueError, match="decode error"):
+        tile_lane.check_errors(lattice)
+    tile_lane.check_errors(lattice)                                           # the flag was cleared by the read
