@@ -45,6 +45,7 @@ struct Layout {
   static constexpr uint32_t kHighBase = 8u * kTableBytes;       // fields 4..7 are addressed from base + this
   static constexpr int kFreqMask = WIDE ? 0x7FF : 0xFFF;
   static constexpr int kDeltaShift = WIDE ? 11 : 12;
+  static constexpr int kDeltaWidth = WIDE ? 11 : 12;            // byte form: bits 12..23 (lattice containers use 11 of them)
   static constexpr int kSymShift = WIDE ? 22 : 24;
 };
 
@@ -85,7 +86,7 @@ struct Pair {
 // x = freq * (x >> PB) + (slot - cdf)
 #define EP_ASM_ADVANCE(S)                                       \
   "v_and_b32 %[t" S "], %[fmask], %[e" S "]\n"                   \
-  "v_bfe_u32 %[d" S "], %[e" S "], %[dshift], 11\n"              \
+  "v_bfe_u32 %[d" S "], %[e" S "], %[dshift], %[dwidth]\n"       \
   "v_mad_u32_u24 %[x" S "], %[t" S "], %[h" S "], %[d" S "]\n"
 
 // Vote, per-half counts, new positions, window address, issue the window read. Leaves the vote in vcc.
@@ -167,7 +168,7 @@ __device__ __forceinline__ void field_step_single(Pair& p, int field, uint32_t o
   : [x0] "+v"(p.x), [pos0] "+s"(pos), [e0] "=&v"(e), [t0] "=&v"(t), [h0] "=&v"(h), [d0] "=&v"(d), [na] "=&s"(na),   \
     [nb] "=&s"(nb), [sv] "=&s"(sv)                                                                               \
   : [cb0] "v"(cb), [ring0] "v"(p.ring), [shv] "v"(k.shv), [kslot] "s"(kslot), [kring] "s"(kring), [valid] "s"(valid), \
-    [off] "n"(OFF), [pb] "n"(PB), [fmask] "n"(L::kFreqMask), [dshift] "n"(L::kDeltaShift)                           \
+    [off] "n"(OFF), [pb] "n"(PB), [fmask] "n"(L::kFreqMask), [dshift] "n"(L::kDeltaShift), [dwidth] "n"(L::kDeltaWidth)                           \
   : "vcc", "scc", "memory"
   // The LDS offset must be an immediate, so the four field positions inside a group are spelled out.
 #define EP_FIELD_SINGLE_CASE(OFF)                                                                              \
@@ -209,7 +210,7 @@ __device__ __forceinline__ void field_step_dual(Pair& p0, Pair& p1, int field, u
     [nb] "=&s"(nb), [sv] "=&s"(sv), [m0] "=&s"(m0)                                                               \
   : [cb0] "v"(cb0), [cb1] "v"(cb1), [ring0] "v"(p0.ring), [ring1] "v"(p1.ring), [shv] "v"(k.shv),                \
     [kslot] "s"(kslot), [kring] "s"(kring), [valid] "s"(valid), [off] "n"(OFF), [pb] "n"(PB),                    \
-    [fmask] "n"(L::kFreqMask), [dshift] "n"(L::kDeltaShift)                                                      \
+    [fmask] "n"(L::kFreqMask), [dshift] "n"(L::kDeltaShift), [dwidth] "n"(L::kDeltaWidth)                                                      \
   : "vcc", "scc", "memory"
 #define EP_FIELD_DUAL_CASE(OFF)                                                                            \
   if constexpr (MASKED) asm volatile(EP_ASM_MASK_ON EP_FIELD_DUAL_BODY EP_ASM_MASK_OFF EP_FIELD_DUAL_OPERANDS(OFF)); \
@@ -349,6 +350,66 @@ __device__ __forceinline__ void sym_step(Pair& p, int field, uint32_t slot_cb, c
   p.pos = pos;
 }
 
+// ---- payload windows ---------------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ void lds_store32(uint32_t at, uint32_t value) {
+  *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(at)) = value;
+}
+
+// Opens the window of each half's stream, words [word_begin, word_end) of `payload` (per-half values; lanes of a
+// half agree): fills the 128 LDS words at `window_at` with the stream's last one or two 64-word chunks, requests the
+// 64 words below them, and sets the biased positions and the bookkeeping the end-of-stream check needs.
+__device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_t word_begin, uint32_t word_end,
+                                            const uint16_t* __restrict__ payload, uint64_t payload_words, int l32) {
+  const uint32_t* payload32 = reinterpret_cast<const uint32_t*>(payload);
+  s.ring = window_at - 2u * kPosBias;                   // positions are kept biased, see Pair::pos
+  const uint32_t base = word_begin & ~63u;               // absolute index of relative position 0
+  const int begin = static_cast<int>(word_begin - base);
+  const int ptr = static_cast<int>(word_end - base);
+  const int low = (ptr & ~63) - 64;                       // the window holds relative [low, low + 128)
+  s.ring_lane = window_at + 4u * static_cast<uint32_t>(l32);
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int64_t at = static_cast<int64_t>(base) + low + 64 * c + 2 * l32;
+    uint32_t lo = 0, hi = 0;
+    if (at >= 0 && static_cast<uint64_t>(at) < payload_words) lo = payload[at];
+    if (at + 1 >= 0 && static_cast<uint64_t>(at + 1) < payload_words) hi = payload[at + 1];
+    lds_store32(s.ring_lane + 128u * c, lo | (hi << 16));
+  }
+  s.fetch_dword = static_cast<int32_t>((static_cast<int64_t>(base) + low - 64) >> 1) + l32;
+  s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
+  const int p = ptr - low + static_cast<int>(kPosBias);  // position in [64, 128), stored biased
+  s.pos = static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 0)) | (static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 32)) << 16);
+  s.windowA = __builtin_amdgcn_readlane(low, 0);
+  s.windowB = __builtin_amdgcn_readlane(low, 32);
+  s.beginA = __builtin_amdgcn_readlane(begin, 0);
+  s.beginB = __builtin_amdgcn_readlane(begin, 32);
+}
+
+// After a step (or two): a half whose position fell below 64 slides its window down by 64 words. All 32 lanes of the
+// half (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
+// the next 64 words down.
+__device__ __forceinline__ void slide_window(Pair& s, int half, const uint32_t* __restrict__ payload32) {
+  const uint32_t low_bits = ~s.pos & 0x00800080u;        // bit 7 of a biased field clear <=> that position < 64
+  if (__builtin_expect(low_bits != 0, 0)) {
+    asm volatile("" ::: "memory");     // keep this a scalar branch: the common case must cost no vector work
+    if ((low_bits >> (half ? 23 : 7)) & 1u) {
+      const uint32_t kept = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(s.ring_lane));
+      lds_store32(s.ring_lane + 128u, kept);
+      lds_store32(s.ring_lane, s.prefetch);
+      s.fetch_dword -= 32;
+      s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
+    }
+    s.pos += low_bits >> 1;             // + 64 in the fields that slid
+    s.windowA -= static_cast<int>((low_bits >> 1) & 0x40u);
+    s.windowB -= static_cast<int>((low_bits >> 17) & 0x40u);
+  }
+}
+
+// Where each half's stream stands, relative to the same base as Pair::beginA / beginB.
+__device__ __forceinline__ int window_pointer_a(const Pair& s) { return s.windowA + static_cast<int>(s.pos & 0xFFFFu) - static_cast<int>(kPosBias); }
+__device__ __forceinline__ int window_pointer_b(const Pair& s) { return s.windowB + static_cast<int>(s.pos >> 16) - static_cast<int>(kPosBias); }
+
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
 template <int PB, int MODE, int ILP, int KIND>
@@ -370,7 +431,6 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr)smem));
   const uint32_t rings0 = lds0 + lut_bytes;
   const uint32_t minima0 = rings0 + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes;
-  auto lds_write32 = [](uint32_t at, uint32_t value) { *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(at)) = value; };
 
   {
     const uint4* src = reinterpret_cast<const uint4*>(MODE == kModeSym ? a.sym_tables : reinterpret_cast<const uint8_t*>(a.plan) + kHeaderBytes);
@@ -411,7 +471,6 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       Pair& s = st[j];
       const int64_t tile = 2 * static_cast<int64_t>(first_pair + j) + half;
       const uint32_t window_at = rings0 + static_cast<uint32_t>((wave * ILP + j) * 2 + half) * kRingBytes;
-      s.ring = window_at - 2u * kPosBias;                   // positions are kept biased, see Pair::pos
       uint32_t word_begin = 0, word_end = 0;
       s.count = 0;
       s.x = kStateMin;
@@ -436,49 +495,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         }
       }
       full = full && s.count == a.tile_vectors;
-      const uint32_t base = word_begin & ~63u;               // absolute index of relative position 0
-      const int begin = static_cast<int>(word_begin - base);
-      const int ptr = static_cast<int>(word_end - base);
-      const int low = (ptr & ~63) - 64;                       // the window holds relative [low, low + 128)
-      s.ring_lane = window_at + 4u * static_cast<uint32_t>(l32);
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const int64_t at = static_cast<int64_t>(base) + low + 64 * c + 2 * l32;
-        uint32_t lo = 0, hi = 0;
-        if (at >= 0 && static_cast<uint64_t>(at) < a.payload_words) lo = a.payload[at];
-        if (at + 1 >= 0 && static_cast<uint64_t>(at + 1) < a.payload_words) hi = a.payload[at + 1];
-        lds_write32(s.ring_lane + 128u * c, lo | (hi << 16));
-      }
-      s.fetch_dword = static_cast<int32_t>((static_cast<int64_t>(base) + low - 64) >> 1) + l32;
-      s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
-      const int p = ptr - low + static_cast<int>(kPosBias);  // position in [64, 128), stored biased
-      s.pos = static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 0)) | (static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 32)) << 16);
-      s.windowA = __builtin_amdgcn_readlane(low, 0);
-      s.windowB = __builtin_amdgcn_readlane(low, 32);
-      s.beginA = __builtin_amdgcn_readlane(begin, 0);
-      s.beginB = __builtin_amdgcn_readlane(begin, 32);
+      open_window(s, window_at, word_begin, word_end, a.payload, a.payload_words, l32);
     }
     const bool all_full = __builtin_amdgcn_readfirstlane(__all(full) ? 1 : 0) != 0;
 
     // After a step: a half whose position fell below 64 slides its window down by 64 words. All 32 lanes of the half
     // (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
     // the next 64 words down.
-    auto top_up = [&](Pair& s) {
-      const uint32_t low_bits = ~s.pos & 0x00800080u;        // bit 7 of a biased field clear <=> that position < 64
-      if (__builtin_expect(low_bits != 0, 0)) {
-        asm volatile("" ::: "memory");     // keep this a scalar branch: the common case must cost no vector work
-        if ((low_bits >> (half ? 23 : 7)) & 1u) {
-          const uint32_t kept = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(s.ring_lane));
-          lds_write32(s.ring_lane + 128u, kept);
-          lds_write32(s.ring_lane, s.prefetch);
-          s.fetch_dword -= 32;
-          s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
-        }
-        s.pos += low_bits >> 1;             // + 64 in the fields that slid
-        s.windowA -= static_cast<int>((low_bits >> 1) & 0x40u);
-        s.windowB -= static_cast<int>((low_bits >> 17) & 0x40u);
-      }
-    };
+    auto top_up = [&](Pair& s) { slide_window(s, half, payload32); };
 
     // E8 point, row scale, container cast and store of the vector each valid lane just decoded.
     auto weights_of = [&](const Pair& s, float scale, float (&w)[8]) {
@@ -746,8 +770,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       const uint64_t stale = __builtin_amdgcn_ballot_w64(s.count > 0 && s.x != kStateMin);
       const uint64_t live = __builtin_amdgcn_ballot_w64(s.count > 0);
       const bool liveA = (live & 1u) != 0, liveB = ((live >> 32) & 1u) != 0;
-      const int ptrA = s.windowA + static_cast<int>(s.pos & 0xFFFFu) - static_cast<int>(kPosBias);
-      const int ptrB = s.windowB + static_cast<int>(s.pos >> 16) - static_cast<int>(kPosBias);
+      const int ptrA = window_pointer_a(s), ptrB = window_pointer_b(s);
       const bool badA = liveA && (ptrA != s.beginA || static_cast<uint32_t>(stale) != 0);
       const bool badB = liveB && (ptrB != s.beginB || static_cast<uint32_t>(stale >> 32) != 0);
       if ((badA || badB) && lane == 0) {

@@ -117,3 +117,54 @@ def test_corrupt_stream_sets_the_error_flag_and_stays_in_bounds():
     with pytest.raises(ValueError, match="decode error"):
         tile_lane.check_errors(lattice)
     tile_lane.check_errors(lattice)                                           # the flag was cleared by the read
+
+
+def test_one_symbol_lane_at_twelve_bits():
+    """A coded lane whose table holds a single symbol has frequency 4096, which the LDS entries of the one-coded-lane
+    kernel cannot hold; those workgroups decode stream by stream. Low byte random (raw), high byte constant (coded)."""
+    torch.manual_seed(11)
+    values = torch.randint(0, 256, (37, 1000), dtype=torch.int16) + 0x2A00
+    container = round_trip(values, probability_bits=12, tile_elements=4096)
+    assert container.buffers["lane_modes"].tolist() == [1, 0]
+    table = container.buffers["decode_tables"].view(torch.int32)[1]
+    assert int(((table >> 8) & 0xFFF).max()) == 0                       # 4096 is stored as 0
+    constant = torch.full((9000,), 7, dtype=torch.int8)
+    round_trip(constant, probability_bits=12, tile_elements=2048)
+
+
+@pytest.mark.parametrize("tile_elements", [256, 320, 1000, 4096])
+def test_one_coded_lane_tile_sizes(tile_elements):
+    """Whole 256-element chunks take the wide-store path, other tile sizes and the last short tile the group path."""
+    print("case", tile_elements, flush=True)
+    torch.manual_seed(tile_elements)
+    for dtype in (torch.bfloat16, torch.float32, torch.int8, torch.int64):
+        if dtype == torch.int64:       # seven random bytes under a peaked top byte: 7 raw lanes + 1 coded
+            tensor = torch.randint(0, 1 << 56, (70, 999), dtype=dtype) + ((torch.randn(70, 999) * 6).round().to(dtype).clamp(-100, 100) << 56)
+        else:
+            tensor = (torch.randn(70, 999) * 0.03).to(dtype) if dtype.is_floating_point else (torch.randn(70, 999) * 20).round().to(dtype)
+        container = round_trip(tensor, tile_elements=tile_elements)
+        assert sum(1 for mode in container.buffers["lane_modes"].tolist() if mode == 0) <= 1     # 0 where the states cost too much
+
+
+def test_output_address_need_not_be_aligned():
+    """Through the C ABI with an output 2 bytes off a 16-byte boundary: the same bytes."""
+    torch.manual_seed(3)
+    tensor = (torch.randn(64, 4096) * 0.02).to(torch.bfloat16)
+    container = ep.compress(tensor, ep.TileANSConfig(execution_backend="eager")).to("cuda")
+    buffers = packed_buffers(container.buffers, TileBuffers)
+    from entropack_amd.backends import hip as backend
+    modes = np.asarray(buffers.lane_modes.cpu().tolist(), dtype=np.uint8)
+    tile_elements, prob_bits, lanes, elements = (int(v) for v in buffers.layout.tolist())
+    room = torch.zeros(elements * lanes + 64, dtype=torch.uint8, device="cuda")
+    error = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for shift in (0, 2, 6):
+        room.zero_()
+        backend.check("ep_hip_decode_tile_ans", backend.library().ep_hip_decode_tile_ans(
+            backend.pointer(buffers.payload), buffers.payload.numel(), buffers.offsets.data_ptr(), backend.pointer(buffers.states),
+            buffers.decode_tables.data_ptr(), modes.ctypes.data, tile_elements, prob_bits, lanes, elements,
+            room.data_ptr() + shift, error.data_ptr(), backend.current_stream(room.device)))
+        torch.cuda.synchronize()
+        assert int(error.item()) == 0
+        got = room[shift:shift + elements * lanes].cpu().numpy()
+        assert np.array_equal(got, tensor.contiguous().view(torch.uint8).numpy().reshape(-1))
+        assert int(room[shift + elements * lanes:].max()) == 0 and int(room[:shift].sum()) == 0
