@@ -1,6 +1,6 @@
 """Headline benchmark: lossy (lattice_rans) decode throughput on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans]
 
 One "step" = one decode of the whole container (entropy decode + E8 reconstruction + BF16 store) from buffers
 already resident in HBM. Prints ONE JSON line. `value` = algorithmic bytes (container bytes read + dense bytes
@@ -274,12 +274,82 @@ def stack_workload(args, ep):
     return 0
 
 
+def lossless_workload(args, ep):
+    """The lossless neighbour of the target: tile_ans decode of 8192 x 28672 bf16 N(0, 0.015) seed 4 (the reference's
+    default options for bfloat16: 8192-element tiles, 10-bit tables; low byte raw, high byte coded)."""
+    from entropack_amd.schemes.base import packed_buffers
+    from entropack_amd.schemes.tile_ans import hip as tile_lane
+    from entropack_amd.schemes.tile_ans.format import TileBuffers
+    rows, cols, sigma, seed = 8192, 28672, 0.015, 4
+    started = time.perf_counter()
+    weight = make_weight(rows, cols, sigma, seed, False)
+    container = ep.compress(weight, ep.TileANSConfig(execution_backend="eager"))
+    encode_seconds = time.perf_counter() - started
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    on_gpu = container.to(device)
+    buffers = packed_buffers(on_gpu.buffers, TileBuffers)
+    alg_bytes = sum(t.numel() * t.element_size() for t in container.buffers.values()) + rows * cols * 2
+
+    def step():
+        return tile_lane.decode(buffers, dtype=torch.bfloat16)
+
+    for _ in range(max(args.warmup, 1)):
+        dense = step()
+    torch.cuda.synchronize()
+    tile_lane.check_errors(buffers)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    wall = time.perf_counter()
+    for begin, end in events:
+        begin.record()
+        dense = step()
+        end.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall) / args.steps
+    kernel_ms = sorted(begin.elapsed_time(end) for begin, end in events)
+    kernel_avg_ms = sum(kernel_ms) / len(kernel_ms)
+    tile_elements, prob_bits, lanes, elements = (int(v) for v in container.buffers["layout"].tolist())
+    result = {
+        "metric": "lossless decode GB/s (+% HBM roofline)", "value": round(alg_bytes / wall / 1e9, 3), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {
+            "workload": f"tile_ans decode to bf16, {rows}x{cols} N(0,{sigma}) seed {seed}, default options",
+            "tile_elements": tile_elements, "prob_bits": prob_bits, "lane_modes": container.buffers["lane_modes"].tolist(),
+            "stored_over_dense": round(container.storage_nbytes() / (rows * cols * 2), 4), "algorithmic_bytes": alg_bytes,
+            "elements_per_s": round(rows * cols / wall, 1), "encode_seconds_cpu": round(encode_seconds, 2),
+            "lossless": bool(torch.equal(dense.view(torch.int16).reshape(rows, cols).cpu(), weight.view(torch.int16))),
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9, 3), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": None,
+            "kernel_ms_avg": round(kernel_avg_ms, 5), "kernel_ms_median": round(kernel_ms[len(kernel_ms) // 2], 5),
+        },
+    }
+    if not args.no_cpu:
+        from oracle import c_oracle
+        c_oracle.load_tile_ans()
+        host = host_arrays(container.buffers)
+        threads = min(16, os.cpu_count() or 1)
+        best = float("inf")
+        for _ in range(2):
+            begin = time.perf_counter()
+            expect = c_oracle.tile_ans_decode(host, 2, threads=threads)
+            best = min(best, time.perf_counter() - begin)
+        result["cpu_baseline"] = {
+            "value": round(alg_bytes / best / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"whole container, C port of the reference CPU decoder, {threads} OpenMP threads, best of 2, {best:.3f} s"}
+        result["config"]["bit_exact_vs_oracle"] = bool(np.array_equal(dense.view(torch.uint8).cpu().numpy().reshape(-1), expect))
+    print(json.dumps(result))
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4"])
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans"])
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
@@ -298,6 +368,8 @@ def main():
 
     if args.workload == "c4":
         return stack_workload(args, ep)
+    if args.workload == "tile_ans":
+        return lossless_workload(args, ep)
     rows, cols, sigma, seed, bpp, outliers = WORKLOADS[args.workload]
     started = time.perf_counter()
     weight = make_weight(rows, cols, sigma, seed, outliers)
