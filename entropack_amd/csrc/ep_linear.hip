@@ -236,6 +236,135 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const void* __restri
   if (threadIdx.x == 0) scales[row] = scale;
 }
 
+// The same with an optional block rotation in front (entropack/linear/convrot.py:34-53 of the reference: activations
+// are multiplied, group by group, with the Kronecker power of the 4 x 4 matrix 1 - 2 * antidiagonal, divided by
+// sqrt(group), the product rounded to the activation dtype, and then quantised). The matrix is symmetric and every
+// radix-4 stage is y_a = (x_0 + x_1 + x_2 + x_3) - 2 * x_(3 - a), so a group of 4^stages elements takes `stages`
+// butterfly stages instead of a product. A lane holds 16 consecutive elements, so the first two stages stay in its
+// registers and a group of 256 is one 16-lane row: the third stage runs inside quads and the fourth across the four
+// quads of a row, both with data-parallel-primitive lane moves (no LDS traffic). The division is a power of two,
+// applied once at the end. One block of four waves per row; the rotated row stays in registers between the absmax
+// and the codes (CHUNKS x 4096 elements), so x is read once. stages = 0 is plain quantisation.
+template <int CTRL, int BANKS>
+__device__ __forceinline__ float dpp(float old, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), CTRL, 0xF, BANKS, false));
+}
+
+__device__ __forceinline__ void butterfly4(float& a, float& b, float& c, float& d) {
+  const float sum = (a + b) + (c + d);
+  const float ya = sum - 2.0f * d, yb = sum - 2.0f * c, yc = sum - 2.0f * b, yd = sum - 2.0f * a;
+  a = ya, b = yb, c = yc, d = yd;
+}
+
+template <int IN_KIND, int CHUNKS>
+__global__ __launch_bounds__(256) void rotate_quantize_rows_kernel(const void* __restrict__ x, int64_t ldx, int K, int stages,
+                                                                   int8_t* __restrict__ codes, float* __restrict__ scales) {
+  __shared__ float partial[4];
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  constexpr int kQuadSwap1 = 0xB1, kQuadSwap2 = 0x4E, kQuadReverse = 0x1B;      // quad_perm [1,0,3,2], [2,3,0,1], [3,2,1,0]
+  constexpr int kRowRor4 = 0x124, kRowRor8 = 0x128, kRowRor12 = 0x12C;          // lane l takes lane (l - n) mod 16 of its row
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const float shrink = __builtin_ldexpf(1.0f, -stages);
+
+  float v[CHUNKS][16];
+  float top = 0.0f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int k0 = (c * 4 + wave) * 1024 + lane * 16;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float* w = &v[c][4 * q];
+      w[0] = w[1] = w[2] = w[3] = 0.0f;
+      if (k0 + 4 * q < K) {
+        if constexpr (IN_KIND == kOutF32) {
+          const f32x4 in = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(x) + row * ldx + k0 + 4 * q);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w[i] = in[i];
+        } else {
+          const u32x2 in = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(x) + row * ldx + k0 + 4 * q);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t bits = (in[i >> 1] >> (16 * (i & 1))) & 0xFFFFu;
+            if constexpr (IN_KIND == kOutBF16) w[i] = __uint_as_float(bits << 16);
+            else w[i] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
+          }
+        }
+      }
+    }
+    if (stages >= 1) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) butterfly4(v[c][4 * q], v[c][4 * q + 1], v[c][4 * q + 2], v[c][4 * q + 3]);
+    }
+    if (stages >= 2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) butterfly4(v[c][r], v[c][4 + r], v[c][8 + r], v[c][12 + r]);
+    }
+    if (stages >= 3) {        // digit = lane & 3
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float value = v[c][i];
+        const float pair = value + dpp<kQuadSwap1, 0xF>(0.0f, value);
+        const float sum = pair + dpp<kQuadSwap2, 0xF>(0.0f, pair);
+        v[c][i] = sum - 2.0f * dpp<kQuadReverse, 0xF>(0.0f, value);
+      }
+    }
+    if (stages >= 4) {        // digit = (lane >> 2) & 3; its complement sits 4 lanes down for even digits, 4 up for odd ones
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float value = v[c][i];
+        const float pair = value + dpp<kRowRor8, 0xF>(0.0f, value);
+        const float sum = pair + dpp<kRowRor4, 0xF>(0.0f, pair);
+        float other = dpp<kRowRor4, 0x5>(0.0f, value);
+        other = dpp<kRowRor12, 0xA>(other, value);
+        v[c][i] = sum - 2.0f * other;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float scaled = v[c][i] * shrink;
+      if constexpr (IN_KIND == kOutBF16) v[c][i] = __uint_as_float(bf16_bits_of(scaled) << 16);
+      else if constexpr (IN_KIND == kOutF16) v[c][i] = static_cast<float>(static_cast<_Float16>(scaled));
+      else v[c][i] = scaled;
+      top = __builtin_fmaxf(top, __builtin_fabsf(v[c][i]));
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) top = __builtin_fmaxf(top, __shfl_xor(top, offset));
+  if (lane == 0) partial[wave] = top;
+  __syncthreads();
+  top = __builtin_fmaxf(__builtin_fmaxf(partial[0], partial[1]), __builtin_fmaxf(partial[2], partial[3]));
+  const float scale = __builtin_fmaxf(top / 127.0f, 1.1920928955078125e-07f);
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int k0 = (c * 4 + wave) * 1024 + lane * 16;
+    u32x4 packed;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float code = __builtin_fminf(__builtin_fmaxf(__builtin_rintf(v[c][4 * q + i] / scale), -127.0f), 127.0f);
+        word |= (static_cast<uint32_t>(static_cast<int>(code)) & 0xFFu) << (8 * i);
+      }
+      packed[q] = word;
+    }
+    int8_t* to = codes + row * K + k0;
+    if (k0 + 16 <= K && (K & 15) == 0) {
+      *reinterpret_cast<u32x4*>(to) = packed;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (k0 + 4 * q < K) *reinterpret_cast<uint32_t*>(to + 4 * q) = packed[q];
+      }
+    }
+  }
+  if (threadIdx.x == 0) scales[row] = scale;
+}
+
 
 // ---- large products: 256 x 256 block tiles ----------------------------------------------------------------------------------
 //
@@ -555,6 +684,39 @@ static int out_kind_valid(int kind) { return kind == kOutBF16 || kind == kOutF16
 
 }  // namespace ep
 
+namespace ep {
+
+// Four consecutive elements as one 8- or 16-byte load, four codes as one 4-byte store, a whole row in the registers of
+// one workgroup.
+constexpr int64_t kQuantiseRegisterColumns = 32768;
+static bool rows_take_wide_loads(const void* x, int in_kind, int64_t K, int64_t ldx, const void* codes) {
+  const uintptr_t element = in_kind == kOutF32 ? 4 : 2;
+  return K % 4 == 0 && K <= kQuantiseRegisterColumns && ldx % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * element) == 0 && reinterpret_cast<uintptr_t>(codes) % 4 == 0;
+}
+
+template <int IN_KIND>
+static void launch_rotate_quantize_of(const void* x, int64_t rows, int64_t K, int64_t ldx, int stages, int8_t* codes, float* scales,
+                                      hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>(rows)), block(256);
+  const int k = static_cast<int>(K);
+  if (K <= 4096) hipLaunchKernelGGL((rotate_quantize_rows_kernel<IN_KIND, 1>), grid, block, 0, s, x, ldx, k, stages, codes, scales);
+  else if (K <= 8192) hipLaunchKernelGGL((rotate_quantize_rows_kernel<IN_KIND, 2>), grid, block, 0, s, x, ldx, k, stages, codes, scales);
+  else if (K <= 16384) hipLaunchKernelGGL((rotate_quantize_rows_kernel<IN_KIND, 4>), grid, block, 0, s, x, ldx, k, stages, codes, scales);
+  else hipLaunchKernelGGL((rotate_quantize_rows_kernel<IN_KIND, 8>), grid, block, 0, s, x, ldx, k, stages, codes, scales);
+}
+
+static int launch_rotate_quantize(const void* x, int in_kind, int64_t rows, int64_t K, int64_t ldx, int stages, int8_t* codes,
+                                  float* scales, void* stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (in_kind == kOutBF16) launch_rotate_quantize_of<kOutBF16>(x, rows, K, ldx, stages, codes, scales, s);
+  else if (in_kind == kOutF16) launch_rotate_quantize_of<kOutF16>(x, rows, K, ldx, stages, codes, scales, s);
+  else launch_rotate_quantize_of<kOutF32>(x, rows, K, ldx, stages, codes, scales, s);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+}  // namespace ep
+
 extern "C" {
 
 int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
@@ -642,10 +804,24 @@ int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K
   using namespace ep;
   if (x_dev == nullptr || codes_dev == nullptr || scales_dev == nullptr) return EP_HIP_EINVAL;
   if (rows <= 0 || K <= 0 || rows > 0x7FFFFFFF || K > 0x7FFFFFFF || ldx < K || !out_kind_valid(in_kind)) return EP_HIP_EINVAL;
+  if (rows_take_wide_loads(x_dev, in_kind, K, ldx, codes_dev)) return launch_rotate_quantize(x_dev, in_kind, rows, K, ldx, 0, codes_dev, scales_dev, stream);
   hipLaunchKernelGGL(quantize_rows_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      x_dev, in_kind, ldx, static_cast<int>(K), codes_dev, scales_dev);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
+}
+
+int ep_hip_rotate_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K, int64_t ldx, int group,
+                                int8_t* codes_dev, float* scales_dev, void* stream) {
+  using namespace ep;
+  if (x_dev == nullptr || codes_dev == nullptr || scales_dev == nullptr) return EP_HIP_EINVAL;
+  if (rows <= 0 || K <= 0 || rows > 0x7FFFFFFF || K > 0x7FFFFFFF || ldx < K || !out_kind_valid(in_kind)) return EP_HIP_EINVAL;
+  int stages = 0;
+  while (stages < 16 && (1 << (2 * stages)) < group) ++stages;
+  if (group < 4 || (1 << (2 * stages)) != group || K % group != 0) return EP_HIP_EINVAL;       // a power of four dividing K
+  if (group > 256) return EP_HIP_EUNSUPPORTED;                                                   // a wave holds 256 elements
+  if (!rows_take_wide_loads(x_dev, in_kind, K, ldx, codes_dev)) return EP_HIP_EUNSUPPORTED;
+  return launch_rotate_quantize(x_dev, in_kind, rows, K, ldx, stages, codes_dev, scales_dev, stream);
 }
 
 }  // extern "C"

@@ -79,6 +79,37 @@ def quantize_rows(tensor: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return codes, scale
 
 
+def rotate_quantize_rows(tensor: torch.Tensor, group: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """`quantize_rows` of the block-rotated activation (groups of `group` features, see `linear.convrot`).
+
+    Groups up to 256 rotate inside the quantiser kernel; larger ones (and rows the kernel's 8/16-byte loads cannot take)
+    rotate through a library product on the same device first.
+    """
+    from . import convrot
+    device = _require_device(tensor)
+    if tensor.dtype not in _hip.FLOAT_KINDS:
+        raise TypeError(f"rotate_quantize_rows takes bf16/f16/f32 activations, got {tensor.dtype}")
+    flat = tensor.reshape(-1, tensor.shape[-1])
+    if flat.stride(-1) != 1:
+        flat = flat.contiguous()
+    rows, inner = flat.shape
+    if not convrot.is_convrot_group(group) or inner % group:
+        raise ValueError(f"convrot group {group} must be a power of four dividing in_features {inner}")
+    if rows and group <= convrot.FUSED_GROUP_LIMIT:
+        codes = torch.empty(rows, inner, dtype=torch.int8, device=device)
+        scale = torch.empty(rows, dtype=torch.float32, device=device)
+        with torch.cuda.device(device):
+            status = _hip.library().ep_hip_rotate_quantize_rows(
+                flat.data_ptr(), _hip.FLOAT_KINDS[tensor.dtype], rows, inner, flat.stride(0), group, codes.data_ptr(),
+                scale.data_ptr(), _hip.current_stream(device))
+        if status == _hip.OK:
+            return codes, scale
+        if status != _hip.EUNSUPPORTED:
+            _hip.check("ep_hip_rotate_quantize_rows", status)
+    matrix = convrot.build_convrot_matrix(group, device=device, dtype=flat.dtype)
+    return quantize_rows(convrot.rotate_activation(flat, matrix, group))
+
+
 def int8_gemm(activation: torch.Tensor, codes: torch.Tensor, activation_scale: torch.Tensor, weight_scale: torch.Tensor,
               bias: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
     """(activation[M, K] @ codes[N, K].T) in int32, times both row scales, plus bias, as `out_dtype`."""

@@ -25,6 +25,7 @@ from ..backends import hip as _hip
 from ..compression import CompressedTensor, compress, decompress
 from ..registry import default_config, get_scheme, name_for_config, require_dtype
 from ..schemes import EntroPackLossyConfig, RawConfig
+from . import convrot
 
 ENCODE_BACKEND = "eager"
 DECODE_BACKEND = "hip"
@@ -297,9 +298,16 @@ class QuantizedLinear(CompressedLinear):
 
     def compress_weight(self, weight: torch.Tensor) -> None:
         self._check_weight_shape(weight.shape)
-        codes, scale = self._quantize_rows(weight.detach())
+        codes, scale = self._quantize_rows(self._prepare_weight_source(weight.detach()))
         self.weight = torch.nn.Parameter(self._compress_tensor(codes), requires_grad=False)
         self.weight_quant_scale = scale
+
+    def _prepare_weight_source(self, weight: torch.Tensor) -> torch.Tensor:
+        """The basis the codes are taken in (the identity here)."""
+        return weight
+
+    def _restore_weight_basis(self, weight: torch.Tensor) -> torch.Tensor:
+        return weight
 
     def codes(self, device=None) -> torch.Tensor:
         """The weight codes in `code_dtype`, decoded on `device`."""
@@ -310,7 +318,7 @@ class QuantizedLinear(CompressedLinear):
 
     def dequantize(self, device=None) -> torch.Tensor:
         codes = self.codes(device)
-        return (codes.float() * self._scale(codes.device).unsqueeze(1)).to(self._init_dtype)
+        return self._restore_weight_basis(codes.float() * self._scale(codes.device).unsqueeze(1)).to(self._init_dtype)
 
     def _require_8bit_gemm(self, device: torch.device) -> None:
         reason = _hip.probe() if device.type == "cuda" else f"tensor is on {device}"
@@ -328,16 +336,48 @@ class QuantizedLinear(CompressedLinear):
 
 
 class CompressedINT8Linear(QuantizedLinear):
-    """Symmetric int8 weights and activations: y = (A_i8 . W_i8^T)_i32 * sa[m] * sw[n] + b[n], cast to x.dtype."""
+    """Symmetric int8 weights and activations: y = (A_i8 . W_i8^T)_i32 * sa[m] * sw[n] + b[n], cast to x.dtype.
+
+    `use_convrot=True` rotates groups of `convrot_groupsize` input features (a power of four, lowered by factors of four
+    until it divides `in_features`) of the weight before it is quantised and of the activations before they are: the
+    product is unchanged, outliers are spread. Like the reference (entropack/linear/linear.py:445-478) the flag is a
+    constructor argument, not part of the checkpoint.
+    """
 
     code_dtype = torch.int8
     code_max = 127.0
     rounds_to_integer = True
 
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, *, config=None, device=None,
+                 dtype: torch.dtype = torch.bfloat16, forward_mode: str = "decode_then_gemm", use_convrot: bool = False,
+                 convrot_groupsize: int = 256):
+        self.use_convrot = bool(use_convrot)
+        self._convrot_group = convrot.choose_convrot_group(in_features, convrot_groupsize) if self.use_convrot else None
+        if self.use_convrot and self._convrot_group is None:
+            raise ValueError(f"use_convrot requires in_features {in_features} to contain a power-of-four group; "
+                             f"got convrot_groupsize={convrot_groupsize}")
+        super().__init__(in_features, out_features, bias=bias, config=config, device=device, dtype=dtype, forward_mode=forward_mode)
+
+    def _rotation(self, like: torch.Tensor) -> torch.Tensor:
+        return convrot.build_convrot_matrix(self._convrot_group, device=like.device, dtype=like.dtype)
+
+    def _prepare_weight_source(self, weight: torch.Tensor) -> torch.Tensor:
+        if not self.use_convrot:
+            return weight
+        return convrot.rotate_weight(weight, self._rotation(weight), self._convrot_group)
+
+    def _restore_weight_basis(self, weight: torch.Tensor) -> torch.Tensor:
+        if not self.use_convrot:
+            return weight
+        return convrot.rotate_weight(weight, self._rotation(weight), self._convrot_group, inverse=True)
+
     def _forward8(self, x: torch.Tensor) -> torch.Tensor:
         from . import kernels
         flat = x.reshape(-1, x.shape[-1]).contiguous()
-        activation, activation_scale = kernels.quantize_rows(flat.detach())
+        if self.use_convrot:
+            activation, activation_scale = kernels.rotate_quantize_rows(flat.detach(), self._convrot_group)
+        else:
+            activation, activation_scale = kernels.quantize_rows(flat.detach())
         if self.forward_mode == "fused":
             from . import fused
             out = fused.int8_linear_forward(self, activation, activation_scale, x.dtype)

@@ -218,6 +218,18 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
 int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K, int64_t ldx, int8_t* codes_dev,
                          float* scales_dev, void* stream);
 
+/* The same on block-rotated activations: every `group` consecutive elements of a row (group = 4, 16, 64 or 256,
+ * dividing K) are multiplied with the symmetric orthogonal matrix kron^k([[1,1,1,-1],[1,1,-1,1],[1,-1,1,1],[-1,1,1,1]])
+ * / sqrt(group), the product is rounded to the activation dtype, and the rotated row is quantised as above. Sums are
+ * formed in float32 by radix-4 stages, not in the order of a matrix product, so a code can differ by one from a
+ * library product's where a value sits on a rounding boundary. Needs K and ldx multiples of 4 and x_dev aligned to
+ * four elements; EP_HIP_EUNSUPPORTED for groups above 256 or unaligned rows (rotate with a library product, then
+ * ep_hip_quantize_rows).
+ * Reference: rotate_activation followed by quantize_rows in CompressedINT8Linear._forward8,
+ * entropack/linear/convrot.py:34-53, entropack/linear/linear.py:463-466,338-341. */
+int ep_hip_rotate_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K, int64_t ldx, int group,
+                                int8_t* codes_dev, float* scales_dev, void* stream);
+
 /* y[m_rows][rows] = x[m_rows][cols_padded] * W^T (+ bias) for one to four activation rows, W given as a compressed
  * container (`weight`: the arguments of ep_hip_decode_lattice; out_offset is ignored, store_kind must be
  * EP_STORE_BF16): every decoded vector is rounded to bf16 as the store would, multiplied with the matching

@@ -236,6 +236,89 @@ def test_int8_linear_forward_matches_its_definition(mode):
     assert layer.weight_quant_scale.dtype == torch.float32        # Module.to must not cast the row scales
 
 
+def _rotation(order):
+    """Kronecker power of the 4 x 4 seed over sqrt(order), in float64 (entropack/linear/convrot.py:9-45 of the reference)."""
+    seed = torch.tensor([[1.0, 1, 1, -1], [1, 1, -1, 1], [1, -1, 1, 1], [-1, 1, 1, 1]], dtype=torch.float64)
+    matrix = seed
+    while matrix.shape[0] < order:
+        matrix = torch.kron(matrix, seed)
+    return matrix / matrix.shape[0] ** 0.5
+
+
+def _rotated_then_quantised(x, group):
+    """Exact rotation (float64), rounded once to x's dtype, then the IEEE float32 row quantiser, all on the CPU."""
+    flat = x.detach().cpu()
+    rows, inner = flat.shape
+    rotated = (flat.double().reshape(rows, inner // group, group) @ _rotation(group)).reshape(rows, inner).to(flat.dtype).float()
+    scale = (rotated.abs().amax(dim=1) / torch.tensor(127.0)).clamp(min=torch.finfo(torch.float32).eps)
+    return (rotated / scale.unsqueeze(1)).round().clamp(-127, 127).to(torch.int8), scale
+
+
+@pytest.mark.parametrize("group", [4, 16, 64, 256, 1024])
+@pytest.mark.parametrize("rows,inner,dtype", [(300, 3072, torch.bfloat16), (5, 1024, torch.float32), (1, 2048, torch.float16), (33, 5120, torch.bfloat16)])
+def test_rotate_quantize_rows_on_exactly_representable_sums(group, rows, inner, dtype):
+    """Small integers: every partial sum is exact in float32 whatever the order, so the codes must be THE codes."""
+    torch.manual_seed(group + rows)
+    x = torch.randint(-8, 9, (rows, inner)).to(dtype).cuda()
+    x[0, :] = 0
+    codes, scale = kernels.rotate_quantize_rows(x, group)
+    expect_codes, expect_scale = _rotated_then_quantised(x, group)
+    assert torch.equal(scale.cpu(), expect_scale)
+    assert torch.equal(codes.cpu(), expect_codes)
+
+
+@pytest.mark.parametrize("group,rows,inner,dtype", [(256, 4096, 3072, torch.bfloat16), (64, 17, 3136, torch.bfloat16), (16, 9, 1008, torch.float16),
+                                                    (4, 3, 4100, torch.float32), (256, 128, 28672, torch.bfloat16)])
+def test_rotate_quantize_rows_on_gaussian_rows_with_outliers(group, rows, inner, dtype):
+    """Float32 sums in butterfly order against the exact rotation: a value on a rounding boundary may move a code by one."""
+    torch.manual_seed(group)
+    x = torch.randn(rows, inner)
+    x[:, 5] *= 40.0
+    x = x.to(dtype).cuda()
+    codes, scale = kernels.rotate_quantize_rows(x, group)
+    expect_codes, expect_scale = _rotated_then_quantised(x, group)
+    assert torch.allclose(scale.cpu(), expect_scale, rtol=2.0 ** -7 if dtype != torch.float32 else 1e-6, atol=0)
+    same_scale = scale.cpu() == expect_scale
+    assert same_scale.float().mean() >= 0.98
+    delta = (codes.cpu().int() - expect_codes.int()).abs()[same_scale]
+    assert int(delta.max()) <= 1
+    assert float((delta != 0).float().mean()) <= 1e-3
+    # the rotation spread the outlier channel: no code row is dominated by one entry any more
+    plain_codes, _ = kernels.quantize_rows(x)
+    assert float(codes.float().abs().mean()) > (2.0 if group >= 64 else 1.1) * float(plain_codes.float().abs().mean())
+
+
+@pytest.mark.parametrize("mode", ["decode_then_gemm", "fused"])
+def test_int8_linear_with_rotation_matches_its_definition(mode):
+    """use_convrot: y = int8 product of the rotated-and-quantised activations with the codes of the rotated weight,
+    exact in float32; and against the dense layer it is closer than the unrotated W8A8 layer when x has outlier channels."""
+    torch.manual_seed(2)
+    rows, cols = 768, 1536
+    dense = torch.nn.Linear(cols, rows, dtype=torch.bfloat16)
+    dense.weight.data.copy_((torch.randn(rows, cols) * 0.02).to(torch.bfloat16))
+    dense.bias.data.copy_((torch.randn(rows) * 0.01).to(torch.bfloat16))
+    turned = ep.CompressedINT8Linear.from_linear(dense, forward_mode=mode, use_convrot=True).cuda()
+    plain = ep.CompressedINT8Linear.from_linear(dense, forward_mode=mode).cuda()
+    assert turned._convrot_group == 256
+    x = torch.randn(300, cols)
+    x[:, 11] *= 50.0
+    x[:, 700] *= 30.0
+    x = x.to(torch.bfloat16).cuda()
+    y = turned(x)
+    qa, sa = kernels.rotate_quantize_rows(x, 256)
+    codes = turned.codes("cuda")
+    expect = ((qa.double() @ codes.double().T).float() * sa.unsqueeze(1) * turned.weight_quant_scale.cuda().unsqueeze(0)
+              + dense.bias.data.cuda().float().unsqueeze(0)).to(torch.bfloat16)
+    assert torch.equal(y, expect)
+    exact = F.linear(x.float(), dense.weight.data.cuda().float(), dense.bias.data.cuda().float())
+    assert rel_l2(y, exact) < 0.5 * rel_l2(plain(x), exact)
+    assert rel_l2(y, exact) < 0.03
+    # the input gradient goes through the dequantised weight in the original basis
+    probe = x[:4].clone().requires_grad_(True)
+    turned(probe).float().sum().backward()
+    assert rel_l2(probe.grad.float(), dense.weight.data.cuda().float().sum(dim=0).expand(4, cols)) < 0.05
+
+
 def test_state_dict_round_trip_through_torch_save():
     """Usage/Linear-layers doc flow: save state_dict -> fresh layers -> torch.load(weights_only=True) -> same outputs."""
     layer, _, _ = _c3_layer("decode_then_gemm", rows=256, cols=512)
