@@ -139,6 +139,53 @@ def linear_section(ep, steps):
     return out
 
 
+def stack_linear_section(ep, steps, layers_total=48, distinct=4):
+    """Config 3's layer repeated as a stack (M = 4096, 3072 x 3072 @ 4 bpp + bias): a model's forward, where the weights of
+    `group` layers are decoded per pass on a second stream while the previous group multiplies (DecodeAhead). Per-layer
+    time over the whole stack; every pass decodes every layer (the stack has more than two groups)."""
+    import copy
+    torch.manual_seed(2)
+    protos = []
+    for _ in range(distinct):
+        dense = torch.nn.Linear(3072, 3072, dtype=torch.bfloat16)
+        dense.weight.data.copy_((torch.randn(3072, 3072) * 0.02).to(torch.bfloat16))
+        dense.bias.data.copy_((torch.randn(3072) * 0.01).to(torch.bfloat16))
+        protos.append(ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0)))
+    layers = [copy.deepcopy(protos[index % distinct]).cuda() for index in range(layers_total)]      # own device buffers each
+    x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
+    flops = 2.0 * 4096 * 3072 * 3072
+
+    def forward():
+        out = None
+        for layer in layers:
+            out = layer(x)
+        return out
+
+    def priced(ms_stack):
+        per_layer = ms_stack / layers_total
+        return {"ms_per_layer": round(per_layer, 5), "tflops": round(flops / per_layer / 1e9, 2),
+                "frac_of_mfma_peak": round(flops / per_layer / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5)}
+
+    out = {"workload": f"{layers_total} x CompressedLinear 3072x3072 @ 4.0 bpp + bias, X [4096, 3072] bf16, decode_then_gemm"}
+    reference = forward()
+    out["layer_by_layer"] = priced(_median_ms(forward, max(3, steps // 5), warmup=2))
+    weights = [layer.dequantize("cuda") for layer in layers[:distinct]]
+    out["dense_gemm_only"] = priced(_median_ms(lambda: [torch.nn.functional.linear(x, weights[i % distinct], layers[i].bias)
+                                                        for i in range(layers_total)], max(3, steps // 5), warmup=2))
+    del weights
+    for group in (8, 16):
+        if layers_total // group < 3:
+            continue
+        with ep.DecodeAhead(layers, group_size=group) as ahead:
+            same = bool(torch.equal(forward(), reference))
+            entry = priced(_median_ms(forward, max(3, steps // 5), warmup=2))
+            entry["identical_to_layer_by_layer"] = same
+            entry["dense_bytes_held"] = ahead.arena_bytes
+            ahead.check_errors()
+        out[f"decode_ahead_group_{group}"] = entry
+    return out
+
+
 def small_m_section(ep, on_gpu, rows, cols, bpp, steps):
     """BASELINE config 5, linear part: X [M, cols] bf16 N(0, 1), M in {1, 16, 128}, on the container just decoded.
 
@@ -439,6 +486,7 @@ def main():
 
     if not args.no_linear:
         result["linear"] = linear_section(ep, args.steps)
+        result["linear_stack"] = stack_linear_section(ep, args.steps)
         if rows * cols >= 1 << 27:
             result["linear_small_m"] = small_m_section(ep, on_gpu, rows, cols, bpp, args.steps)
 

@@ -20,12 +20,12 @@ def linear_forward(layer, x: torch.Tensor) -> torch.Tensor:
         buffers = packed_buffers(on_device.buffers, LatticeBuffers)
         if hip_lane.fused_linear_pays(buffers, tuple(container.shape), x):
             return hip_lane.linear_rows(buffers, shape=tuple(container.shape), x=x, bias=layer._bias_on(x.device))
-    weight = layer.dequantize(x.device)
+    weight = layer._decoded_for(x)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("the fused forward runs in bfloat16; use forward_mode='decode_then_gemm' for other dtypes")
     return kernels.gemm_bf16(x, weight, layer._bias_on(x.device), out_dtype=x.dtype)
 
 
 def int8_linear_forward(layer, activation: torch.Tensor, activation_scale: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    codes = layer.codes(activation.device)
+    codes = layer._decoded_for(activation)
     return kernels.int8_gemm(activation, codes, activation_scale, layer._scale(codes.device), layer._bias_on(activation.device), out_dtype)

@@ -55,6 +55,7 @@ class CompressedLinear(torch.nn.Linear):
         if forward_mode not in FORWARD_MODES:
             raise ValueError(f"forward_mode must be one of {FORWARD_MODES}, got {forward_mode!r}")
         self.forward_mode = forward_mode
+        self._decode_ahead = None          # a linear.ahead.DecodeAhead serving this layer's weight, if attached
         self.config = config
         self._init_dtype = require_dtype(dtype)
         if bias:
@@ -144,6 +145,16 @@ class CompressedLinear(torch.nn.Linear):
         """The dense weight, decoded on `device` (default: where the container lives)."""
         return self._reconstruct(device)
 
+    def _decoded_for(self, x: torch.Tensor) -> torch.Tensor:
+        """The container decoded in its own dtype for one product with `x`: from an attached DecodeAhead when autograd
+        will not keep the tensor (its memory is reused a few layers on), else decoded here."""
+        ahead = self._decode_ahead
+        if ahead is not None and x.device == ahead.device and not (torch.is_grad_enabled() and x.requires_grad):
+            weight = ahead.weight_of(self)
+            if weight is not None:
+                return weight
+        return decompress(self._container().to(device=x.device), self._decode_config)
+
     @classmethod
     def from_linear(cls, linear: torch.nn.Linear, **kwargs) -> "CompressedLinear":
         """A layer of this class holding `linear`'s weight compressed and a copy of its bias."""
@@ -170,7 +181,7 @@ class CompressedLinear(torch.nn.Linear):
         if self.forward_mode == "fused":
             from . import fused
             return fused.linear_forward(self, x)
-        return F.linear(x, self.dequantize(x.device).to(x.dtype), self._bias_on(x.device))
+        return F.linear(x, self._decoded_for(x).to(x.dtype), self._bias_on(x.device))
 
     def extra_repr(self) -> str:
         scheme = "auto" if self.config is None else name_for_config(self.config)
@@ -382,7 +393,7 @@ class CompressedINT8Linear(QuantizedLinear):
             from . import fused
             out = fused.int8_linear_forward(self, activation, activation_scale, x.dtype)
         else:
-            codes = self.codes(x.device)
+            codes = self._decoded_for(flat.detach())
             out = kernels.int8_gemm(activation, codes, activation_scale, self._scale(codes.device), self._bias_on(x.device), x.dtype)
         return out.reshape(*x.shape[:-1], self.out_features)
 
