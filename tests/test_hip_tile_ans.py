@@ -168,3 +168,25 @@ def test_output_address_need_not_be_aligned():
         got = room[shift:shift + elements * lanes].cpu().numpy()
         assert np.array_equal(got, tensor.contiguous().view(torch.uint8).numpy().reshape(-1))
         assert int(room[shift + elements * lanes:].max()) == 0 and int(room[:shift].sum()) == 0
+
+
+@pytest.mark.parametrize("mode", ["decode_then_gemm", "fused"])
+def test_compressed_linear_with_lossless_weights(mode):
+    """`CompressedLinear.from_linear(linear)` with no config stores the weight with tile_ans (the reference's default
+    for bfloat16): the layer's dense weight is the original one bit for bit, and its forward is the dense forward."""
+    torch.manual_seed(8)
+    dense = torch.nn.Linear(1024, 768, dtype=torch.bfloat16)
+    dense.weight.data.copy_((torch.randn(768, 1024) * 0.02).to(torch.bfloat16))
+    layer = ep.CompressedLinear.from_linear(dense, forward_mode=mode)
+    assert layer.weight.compress_method == "tile_ans" and layer.compressed_bits < 12.0
+    state = layer.state_dict()
+    fresh = ep.CompressedLinear(1024, 768, forward_mode=mode)
+    fresh.load_state_dict(state)
+    fresh = fresh.cuda()
+    assert torch.equal(fresh.dequantize("cuda").cpu().view(torch.int16), dense.weight.data.view(torch.int16))
+    for rows in (1, 7, 300):
+        x = torch.randn(rows, 1024).to(torch.bfloat16).cuda()
+        expect = torch.nn.functional.linear(x.float(), dense.weight.data.cuda().float(), dense.bias.data.cuda().float())
+        got = fresh(x)
+        error = ((got.float() - expect).norm() / expect.norm()).item()
+        assert got.dtype == torch.bfloat16 and error <= 4e-3, (rows, error)            # one bf16 rounding of the output
