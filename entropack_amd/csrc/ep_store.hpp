@@ -93,15 +93,29 @@ __device__ __forceinline__ void stream_store8(void* at, uint32_t a, uint32_t b) 
 }
 
 // int8 container, the kind the int8 linear layer decodes to: rint (half to even), clamp to [-128, 127], pack.
+// Clamping first gives the same result (the bounds are integers). Adding 1.5 * 2^23 to a value in [-128, 127] rounds it
+// to an integer, ties to even, in the sum's mantissa, whose low byte is then the two's-complement code; the add writes
+// that byte straight into its place in the packed word (sub-dword destination select), so a weight costs a clamp and an add.
 __device__ __forceinline__ void store_vector_i8(void* out, int64_t vector, const float (&w)[8]) {
-  uint32_t b[8];
+  float magic = 12582912.0f;
+  asm volatile("" : "+v"(magic));          // a vector register: the sub-dword form takes no literal
+  float c[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float r = __builtin_fminf(__builtin_fmaxf(__builtin_rintf(w[i]), -128.0f), 127.0f);
-    b[i] = static_cast<uint32_t>(static_cast<int>(r)) & 0xFFu;
-  }
-  stream_store8(reinterpret_cast<uint2*>(out) + vector, b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24),
-                b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
+  for (int i = 0; i < 8; ++i) c[i] = __builtin_fminf(__builtin_fmaxf(w[i], -128.0f), 127.0f);
+  uint32_t low, high;
+  // The two words alternate: an instruction that keeps the other bytes of its destination must not directly follow
+  // the one that wrote them (sub-dword writes need one instruction in between on this hardware).
+#define EP_I8_ADD(DST, SRC, BYTE, UNUSED) \
+  "v_add_f32_sdwa " DST ", " SRC ", %10 dst_sel:" BYTE " dst_unused:" UNUSED " src0_sel:DWORD src1_sel:DWORD\n"
+  asm(EP_I8_ADD("%0", "%2", "BYTE_0", "UNUSED_PAD") EP_I8_ADD("%1", "%6", "BYTE_0", "UNUSED_PAD")
+      EP_I8_ADD("%0", "%3", "BYTE_1", "UNUSED_PRESERVE") EP_I8_ADD("%1", "%7", "BYTE_1", "UNUSED_PRESERVE")
+      EP_I8_ADD("%0", "%4", "BYTE_2", "UNUSED_PRESERVE") EP_I8_ADD("%1", "%8", "BYTE_2", "UNUSED_PRESERVE")
+      EP_I8_ADD("%0", "%5", "BYTE_3", "UNUSED_PRESERVE") EP_I8_ADD("%1", "%9", "BYTE_3", "UNUSED_PRESERVE")
+      "s_nop 0\n"
+      : "=&v"(low), "=&v"(high)
+      : "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]), "v"(c[7]), "v"(magic));
+#undef EP_I8_ADD
+  stream_store8(reinterpret_cast<uint2*>(out) + vector, low, high);
 }
 
 // Writes the eight values of vector `vector` in any container kind.
