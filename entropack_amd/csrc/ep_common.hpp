@@ -21,7 +21,7 @@ constexpr int kHdrMagic = 0, kHdrKind = 1, kHdrProbBits = 2, kHdrCosetFreq0 = 3,
 constexpr int kHeaderWords = 64;
 constexpr size_t kHeaderBytes = kHeaderWords * 4;
 
-// LDS_BYTE entry: freq[0:12) | (slot - cdf)[12:23) | (value + 128)[24:32)
+// LDS_BYTE entry: freq[0:12) | (slot - cdf)[12:23) | value as a signed byte [24:32)
 // LDS_WIDE entry: freq[0:11) | (slot - cdf)[11:22) | symbol[22:32)
 // GLOBAL64 entry: symbol[0:16) | freq[16:32) | (slot - cdf)[32:64)
 
@@ -59,7 +59,7 @@ inline size_t rank_table_bytes(int present, int prob_bits) {
   return rank_rs_offset(present, prob_bits) + kFieldStreams * rank_rs_stream_bytes(prob_bits);
 }
 
-// LDS_SYM section: FB u64[16][256] = {freq | (value + 128) << 24, cdf + LDS address of the stream's slot table}, then
+// LDS_SYM section: FB u64[16][256] (indexed by value + 128) = {freq | (value & 0xFF) << 24, cdf + LDS address of the stream's slot table}, then
 // SLOT u8[16][2^pb] = value + 128. The kernel stages it at LDS offset 0.
 constexpr int kSymFbStreamBytes = 256 * 8;
 constexpr int kSymFbBytes = kFieldStreams * kSymFbStreamBytes;

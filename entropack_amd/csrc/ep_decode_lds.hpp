@@ -317,7 +317,7 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, 
 
 // ---- two-level tables (byte values, prob_bits <= 11) --------------------------------------------------------------------
 //
-// slot -> value + 128 (one byte) -> {freq | (value + 128) << 24, cdf}. A quarter of the slot table of the byte form,
+// slot -> value + 128 (one byte) -> {freq | (value & 0xFF) << 24, cdf}. A quarter of the slot table of the byte form,
 // so two workgroups share a CU; one more dependent LDS read per step, one vector instruction less. The stored cdf
 // already contains the LDS address bits that `slot | table address` carries, and the first word has the layout of
 // a byte-form entry, so reconstruction is shared with it.
@@ -504,34 +504,48 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
     // the next 64 words down.
     auto top_up = [&](Pair& s) { slide_window(s, half, payload32); };
 
-    // E8 point, row scale, container cast and store of the vector each valid lane just decoded.
-    auto weights_of = [&](const Pair& s, float scale, float (&w)[8]) {
-      const bool c = s.coset_base != 0;
-      float p[8];
+    // E8 point and row scale of the vector each valid lane just decoded. The reference forms (z + c / 2) * scale with
+    // one rounding. For an ordinary scale (positive, neither tiny nor huge) fma(z, scale, c * scale / 2) is the same
+    // number rounded once, c * scale / 2 being exact, and costs one instruction per weight less. Any other scale
+    // (zero, negative: the sign of a zero weight; subnormal; beyond 1e30: bf16 saturation) takes the literal form.
+    auto lattice_point = [&](const Pair& s, float (&z)[8]) {
       if constexpr (!WIDE) {
-        // Top byte = value + 128. 7 * 128 is even, so the parity of z0..z6 is the parity of the biased bytes.
+        // Top byte = the value as a signed byte; the parity of z0..z6 is the parity of those bytes.
         const uint32_t folded = xor3(xor3(s.e[0], s.e[1], s.e[2]), xor3(s.e[3], s.e[4], s.e[5]), s.e[6]);
         const float parity = static_cast<float>((folded >> 24) & 1u);
-        const float bias = c ? -127.5f : -128.0f;
 #pragma unroll
-        for (int f = 0; f < 7; ++f) p[f] = __fadd_rn(static_cast<float>(s.e[f] >> 24), bias);
-        p[7] = __fadd_rn(__fmaf_rn(static_cast<float>(s.e[7] >> 24), 2.0f, parity), c ? -255.5f : -256.0f);
+        for (int f = 0; f < 8; ++f) z[f] = static_cast<float>(static_cast<int32_t>(s.e[f]) >> 24);
+        z[7] = __fmaf_rn(z[7], 2.0f, parity);
       } else {
+        const bool c = s.coset_base != 0;
         const int32_t* minima = reinterpret_cast<const int32_t*>(smem + (minima0 - lds0)) + 1 + (c ? 1 : 0);
-        int z[8];
+        int v[8];
 #pragma unroll
         for (int f = 0; f < 8; ++f) {
-          if constexpr (MODE == kModeRank) z[f] = static_cast<int>(s.e[f]);
-          else z[f] = static_cast<int>(s.e[f] >> L::kSymShift) + minima[2 * f];
+          if constexpr (MODE == kModeRank) v[f] = static_cast<int>(s.e[f]);
+          else v[f] = static_cast<int>(s.e[f] >> L::kSymShift) + minima[2 * f];
         }
-        const int parity = (z[0] + z[1] + z[2] + z[3] + z[4] + z[5] + z[6]) & 1;
-        z[7] = 2 * z[7] + parity;
+        const int parity = (v[0] + v[1] + v[2] + v[3] + v[4] + v[5] + v[6]) & 1;
+        v[7] = 2 * v[7] + parity;
+#pragma unroll
+        for (int f = 0; f < 8; ++f) z[f] = static_cast<float>(v[f]);
+      }
+    };
+    auto weights_of = [&](const Pair& s, float scale, float (&w)[8]) {
+      const bool c = s.coset_base != 0;
+      float z[8];
+      lattice_point(s, z);
+      // 1e-30 <= scale <= 1e30 as one unsigned comparison of the bit patterns (fails for negative values and NaN).
+      const bool ordinary = __float_as_uint(scale) - 0x0DA24260u <= 0x7149F2CAu - 0x0DA24260u;
+      if (__builtin_expect(ordinary, 1)) {
+        const float half = c ? __fmul_rn(scale, 0.5f) : 0.0f;
+#pragma unroll
+        for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], scale, half);
+      } else {
         const float shift = c ? 0.5f : 0.0f;
 #pragma unroll
-        for (int f = 0; f < 8; ++f) p[f] = __fadd_rn(static_cast<float>(z[f]), shift);
+        for (int f = 0; f < 8; ++f) w[f] = __fmul_rn(__fadd_rn(z[f], shift), scale);
       }
-#pragma unroll
-      for (int f = 0; f < 8; ++f) w[f] = __fmul_rn(p[f], scale);
     };
 
     // bf16 pairs of a vector's weights, rounded to nearest even, saturated like the reference's CPU lane.

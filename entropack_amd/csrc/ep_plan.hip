@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void build_sym_tables_kernel(const int32_t* __
     const uint32_t f = freq[s];
     if (f == 0) continue;
     const uint32_t value = static_cast<uint32_t>(s + sym_min + 128);
-    fb[value] = make_uint2(f | (value << 24), running + folded);
+    fb[value] = make_uint2(f | (static_cast<uint32_t>(s + sym_min) << 24), running + folded);     // top byte: the value, two's complement
     for (uint32_t d = 0; d < f && running + d < size; ++d) slots[running + d] = static_cast<uint8_t>(value);
     running += f;
   }
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
       } else {
         uint32_t* lut = reinterpret_cast<uint32_t*>(tables) + (static_cast<size_t>(stream - 1) << prob_bits);
         if (kind == EP_TABLE_LDS_BYTE) {
-          lut[slot] = f | (d << 12) | (static_cast<uint32_t>(s + sym_min + 128) << 24);
+          lut[slot] = f | (d << 12) | (static_cast<uint32_t>(s + sym_min) << 24);     // top byte: the value, two's complement
         } else {
           lut[slot] = f | (d << 11) | (static_cast<uint32_t>(s) << 22);
         }

@@ -47,7 +47,7 @@ enum ep_hip_table_kind {
   EP_TABLE_LDS_WIDE = 2,    /* u32 per slot, LDS-resident; prob_bits <= 11, alphabets <= 1024, frequencies < 2048 */
   EP_TABLE_LDS_RANK = 3,    /* LDS-resident rank/select form: per 32 slots a bitmap of symbol ends + running symbol count,
                                per present symbol freq | cdf << 16 and an int16 value; any prob_bits whose tables fit LDS */
-  EP_TABLE_LDS_SYM = 4      /* two-level, LDS-resident: u8 per slot (the value + 128) and, per value, freq | (value+128) << 24
+  EP_TABLE_LDS_SYM = 4      /* two-level, LDS-resident: u8 per slot (the value + 128) and, per value, freq | (value & 0xFF) << 24
                                and cdf; a quarter of LDS_BYTE's size, so two workgroups share a CU. Same conditions as
                                LDS_BYTE. LDS_BYTE plans at prob_bits 11 carry it as a second section (sym_offset) that
                                large launches use; as a plan's own kind (force_kind only) every launch uses it */
