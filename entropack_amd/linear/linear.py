@@ -27,6 +27,7 @@ from ..registry import default_config, get_scheme, name_for_config, require_dtyp
 from ..schemes import EntroPackLossyConfig, RawConfig
 from . import convrot
 
+QUANT_STATE_LEAF = "entropack_quant_state"      # state_dict key suffix of a compressed weight (the reference's, linear.py:190-230)
 ENCODE_BACKEND = "eager"
 DECODE_BACKEND = "hip"
 FORWARD_MODES = ("decode_then_gemm", "fused")
@@ -210,56 +211,66 @@ class CompressedLinear(torch.nn.Linear):
         super()._save_to_state_dict(destination, prefix, keep_vars)
         if isinstance(self.weight, CompressedTensor):
             # the wrapper tensor has no storage a checkpoint could hold; the packed blob stands in for it
-            destination.pop(prefix + "weight")
-            blob = self.weight.entropack_quant_state
-            destination[prefix + "weight.entropack_quant_state"] = blob if keep_vars else blob.detach()
+            del destination[prefix + "weight"]
+            blob = getattr(self.weight, QUANT_STATE_LEAF)
+            destination[prefix + "weight." + QUANT_STATE_LEAF] = blob if keep_vars else blob.detach()
+
+    def _home_for(self, blob: torch.Tensor) -> torch.device:
+        """Where a loaded blob should live: with the weight it replaces, else with the bias, else where it is."""
+        for holder in (self._parameters.get("weight"), self.bias):
+            if holder is not None and holder.device.type != "meta":
+                return holder.device
+        return blob.device
+
+    def _adopt_blob(self, blob: torch.Tensor, in_place: bool) -> None:
+        """Make the container packed in `blob` this layer's weight. `in_place`: keep the existing Parameter object alive
+        (optimisers and hooks hold on to it) and keep its device."""
+        if in_place:
+            blob = blob.to(device=self._home_for(blob), copy=True)
+        container = CompressedTensor.unpack(blob)
+        self._check_weight_shape(container.shape)
+        fresh = torch.nn.Parameter(container, requires_grad=False)
+        present = self._parameters.get("weight")
+        if in_place and isinstance(present, CompressedTensor):
+            torch.utils.swap_tensors(present, fresh)
+        else:
+            self._parameters["weight"] = fresh
 
     def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
-        key = prefix + "weight.entropack_quant_state"
-        if key in state_dict:
+        entry = prefix + "weight." + QUANT_STATE_LEAF
+        blob = state_dict.pop(entry, None)
+        if blob is None:
+            if strict:
+                missing_keys.append(entry)
+        else:
             try:
-                blob = state_dict[key]
-                assign = local_metadata.get("assign_to_params_buffers", False)
-                current = self._parameters.get("weight")
-                if not assign:
-                    if current is not None and current.device.type != "meta":
-                        target = current.device
-                    elif self.bias is not None and self.bias.device.type != "meta":
-                        target = self.bias.device
-                    else:
-                        target = blob.device
-                    blob = blob.to(device=target, copy=True)
-                container = CompressedTensor.unpack(blob)
-                self._check_weight_shape(container.shape)
-                loaded = torch.nn.Parameter(container, requires_grad=False)
-                if not assign and isinstance(current, CompressedTensor):
-                    torch.utils.swap_tensors(current, loaded)
-                else:
-                    self._parameters["weight"] = loaded
-            except (TypeError, ValueError) as error:
-                error_msgs.append(f"{prefix[:-1]}: {error}")
-            state_dict.pop(key)
-        elif strict:
-            missing_keys.append(key)
-        weight = self._parameters.pop("weight")       # keep nn.Module from looking for a dense "weight" entry
-        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
-        self._parameters["weight"] = weight
+                self._adopt_blob(blob, in_place=not local_metadata.get("assign_to_params_buffers", False))
+            except (TypeError, ValueError) as problem:
+                error_msgs.append(f"{prefix[:-1]}: {problem}")
+        # nn.Module must neither look for a dense "weight" entry nor report the blob's key as unexpected
+        held = self._parameters.pop("weight")
+        try:
+            super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+        finally:
+            self._parameters["weight"] = held
 
 
 class _W8A8Function(torch.autograd.Function):
-    """Forward in int8; the input gradient uses the dequantised weight (the compressed weight itself is frozen)."""
+    """8-bit forward with a straight-through input gradient: d(out)/d(x) is taken through the dequantised weight, the
+    compressed weight itself gets no gradient."""
 
     @staticmethod
     def forward(ctx, x, layer):
-        ctx.layer, ctx.x_shape = layer, x.shape
+        ctx.layer = layer
+        ctx.input_shape = tuple(x.shape)
         return layer._forward8(x.detach())
 
     @staticmethod
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_output):
-        grad = grad_output.reshape(-1, grad_output.shape[-1])
-        weight = ctx.layer.dequantize(grad.device).to(grad.dtype)
-        return torch.mm(grad, weight).reshape(ctx.x_shape), None
+        rows = grad_output.reshape(-1, grad_output.shape[-1])
+        dense = ctx.layer.dequantize(rows.device).to(rows.dtype)
+        return (rows @ dense).reshape(ctx.input_shape), None
 
 
 class QuantizedLinear(CompressedLinear):
@@ -283,20 +294,18 @@ class QuantizedLinear(CompressedLinear):
 
     @classmethod
     def _coded(cls, config):
-        if config is None:
-            return RawConfig()
-        if isinstance(config, RawConfig):
+        """The config the codes are stored with: raw by default, or lattice-coded below the codes' own 8 bits."""
+        if config is None or isinstance(config, RawConfig):
+            return config or RawConfig()
+        if isinstance(config, EntroPackLossyConfig):
+            rate = config.target_bpp
+            usable = isinstance(rate, Real) and not isinstance(rate, bool) and 0.0 < float(rate) < 8.0
+            if not usable:
+                raise ValueError(f"{cls.__name__} stores {cls.code_dtype} codes, 8 bits wide, so a target_bpp only pays below 8; "
+                                 f"got {rate!r}. Pass RawConfig to store the codes uncoded.")
             return config
-        if not isinstance(config, EntroPackLossyConfig):
-            raise TypeError(
-                f"{cls.__name__} stores {cls.code_dtype} codes: either uncoded (RawConfig) or lattice-coded "
-                f"(EntroPackLossyConfig), got {type(config).__name__}")
-        rate = config.target_bpp
-        if isinstance(rate, bool) or not isinstance(rate, Real) or not 0.0 < float(rate) < 8.0:
-            raise ValueError(
-                f"{cls.__name__} stores {cls.code_dtype} codes, 8 bits wide, so a target_bpp only pays below 8; "
-                f"got {rate!r}. Pass RawConfig to store the codes uncoded.")
-        return config
+        raise TypeError(f"{cls.__name__} stores {cls.code_dtype} codes: either uncoded (RawConfig) or lattice-coded "
+                        f"(EntroPackLossyConfig), got {type(config).__name__}")
 
     def _quantize_rows(self, tensor: torch.Tensor):
         """Per-row absmax quantisation in plain torch (used for the weight, once, on any device)."""

@@ -1,14 +1,15 @@
-"""Scheme base class: a named codec with per-backend lanes.
+"""Scheme base class: a named codec whose work is done by per-backend lane modules.
 
-The contract follows the reference (entropack/schemes/base.py:40-98): a scheme lists `lanes` (backend name ->
-module name inside the scheme's package); `lane_for` asks the registry which backend to use and imports that lane
-module lazily; a lane module exposes module-level `encode(...)` / `decode(...)`. The config class of a scheme is
-whatever its `encode` annotates `config` with.
+Public contract = the reference's (entropack/schemes/base.py:40-98), so that scheme packages and lanes written against
+either code base plug into the other: class attributes `name`, `buffer_names`, `lossless`, `priority`, `dtypes`,
+`lanes` (backend name -> module name inside the scheme's package); `lane(backend)` imports that module on first use;
+`lane_for(tensor, backend)` lets the registry pick the backend; lane modules expose module-level `encode(...)` /
+`decode(...)`; a scheme's config class is whatever its `encode` annotates `config` with.
 """
+import dataclasses
 import importlib
+import typing
 from abc import ABC, abstractmethod
-from dataclasses import fields
-from typing import Any, get_type_hints
 
 import torch
 
@@ -17,77 +18,109 @@ from .config import CompressionConfig, RawConfig, validate_config
 
 __all__ = ["RawScheme", "Scheme", "cached_parse", "packed_buffers", "register_scheme"]
 
-_lanes_loaded: dict[tuple[type, str], Any] = {}
-_config_of: dict[type, type] = {}
-
 
 def packed_buffers(packed: dict, kind: type):
-    """Pick a scheme's buffers out of a name -> tensor mapping, as its NamedTuple."""
-    return kind(*(packed[name] for name in kind._fields))
+    """A scheme's buffers, picked out of a name -> tensor mapping in the order of its NamedTuple `kind`."""
+    return kind._make(packed[field] for field in kind._fields)
 
 
 def cached_parse(tensor: torch.Tensor, parse, attribute: str):
-    """Parse a small metadata tensor once and keep the answer on the tensor object itself."""
-    if not hasattr(tensor, attribute):
-        setattr(tensor, attribute, parse(tensor))
-    return getattr(tensor, attribute)
+    """`parse(tensor)`, computed once per tensor object and kept on it (small metadata tensors: layouts, lane modes)."""
+    try:
+        return getattr(tensor, attribute)
+    except AttributeError:
+        value = parse(tensor)
+        setattr(tensor, attribute, value)
+        return value
+
+
+class _LaneModules:
+    """Lane modules by (scheme class, backend), imported when first asked for."""
+
+    def __init__(self):
+        self._loaded = {}
+
+    def get(self, scheme: "Scheme", backend: str):
+        owner = type(scheme)
+        try:
+            return self._loaded[owner, backend]
+        except KeyError:
+            pass
+        module_name = scheme.lanes.get(backend)
+        if module_name is None:
+            raise DispatchError(scheme.name, {backend: f"scheme '{scheme.name}' declares no '{backend}' lane"})
+        try:
+            module = importlib.import_module("." + module_name, package=owner.__module__)
+        except Exception as error:
+            raise DispatchError(scheme.name, {backend: f"lane module failed to import: {error!r}"}) from error
+        self._loaded[owner, backend] = module
+        return module
+
+
+_lane_modules = _LaneModules()
+_config_classes: dict = {}
 
 
 class Scheme(ABC):
+    #: registry key and `compress_method` of the containers this scheme writes
     name: str
-    buffer_names: tuple[str, ...]
+    #: names of the tensors a container of this scheme holds, in blob order
+    buffer_names: tuple
     lossless: bool = True
+    #: the scheme with the highest priority that supports a dtype is that dtype's default
     priority: int = 0
-    dtypes: tuple[torch.dtype, ...] | None = None
-    lanes: dict[str, str] = {}
+    #: dtypes the scheme encodes; None = any
+    dtypes: typing.Optional[tuple] = None
+    #: backend name -> lane module name, relative to the scheme's package
+    lanes: dict = {}
 
-    def supports(self, dtype: torch.dtype) -> bool:
-        return self.dtypes is None or dtype in self.dtypes
-
-    def options_for(self, dtype: torch.dtype) -> dict[str, Any]:
-        return {}
-
-    def lane(self, backend: str):
-        key = (type(self), backend)
-        if key not in _lanes_loaded:
-            if backend not in self.lanes:
-                raise DispatchError(self.name, {backend: f"scheme '{self.name}' declares no '{backend}' lane"})
-            try:
-                _lanes_loaded[key] = importlib.import_module("." + self.lanes[backend], package=type(self).__module__)
-            except Exception as error:
-                raise DispatchError(self.name, {backend: f"lane module failed to import: {error!r}"}) from error
-        return _lanes_loaded[key]
-
-    def lane_for(self, tensor: torch.Tensor | None = None, backend: str | None = None, *, gate_dtype: bool = True):
-        chosen = select(self, tensor, None if backend in (None, "auto") else backend, gate_dtype=gate_dtype)
-        return self.lane(chosen), backend_device(chosen)
+    # -- what a scheme implements -----------------------------------------------------------------------------------
 
     @abstractmethod
     def encode(self, weight, config: CompressionConfig) -> dict:
-        ...
+        """tensor -> {buffer name: tensor}"""
 
     @abstractmethod
     def decode(self, packed: dict, *, shape, dtype, config: CompressionConfig):
-        ...
+        """{buffer name: tensor} -> tensor of `shape` and `dtype`"""
+
+    def validate_buffers(self, buffers: dict, shape, dtype) -> None:
+        """Raise ValueError / TypeError if `buffers` cannot be a container of `shape` and `dtype`."""
+
+    def options_for(self, dtype: torch.dtype) -> dict:
+        """Config options a layer uses for `dtype` when it was given no config."""
+        return {}
+
+    # -- what it inherits ---------------------------------------------------------------------------------------------
+
+    def supports(self, dtype: torch.dtype) -> bool:
+        return True if self.dtypes is None else dtype in self.dtypes
+
+    def lane(self, backend: str):
+        return _lane_modules.get(self, backend)
+
+    def lane_for(self, tensor: typing.Optional[torch.Tensor] = None, backend: typing.Optional[str] = None, *, gate_dtype: bool = True):
+        """(lane module, device its work runs on) for `tensor`; `backend` None or "auto" lets the registry choose."""
+        wanted = backend if backend not in (None, "auto") else None
+        chosen = select(self, tensor, wanted, gate_dtype=gate_dtype)
+        return self.lane(chosen), backend_device(chosen)
 
     @property
     def config_cls(self) -> type:
-        klass = type(self)
-        if klass not in _config_of:
-            _config_of[klass] = get_type_hints(klass.encode)["config"]
-        return _config_of[klass]
+        owner = type(self)
+        if owner not in _config_classes:
+            _config_classes[owner] = typing.get_type_hints(owner.encode)["config"]
+        return _config_classes[owner]
 
     def make_config(self, options: dict):
-        known = {f.name for f in fields(self.config_cls)}
-        unknown = sorted(set(options) - known)
-        if unknown:
-            raise TypeError(f"Unknown {self.name} options: {unknown}")
+        """This scheme's config from option names and values; unknown names and bad values both raise."""
+        accepted = [field.name for field in dataclasses.fields(self.config_cls)]
+        strangers = sorted(name for name in options if name not in accepted)
+        if strangers:
+            raise TypeError(f"Unknown {self.name} options: {strangers}")
         config = self.config_cls(**options)
         validate_config(config)
         return config
-
-    def validate_buffers(self, buffers: dict, shape, dtype) -> None:
-        ...
 
 
 class RawScheme(Scheme):
@@ -96,8 +129,6 @@ class RawScheme(Scheme):
     name = "raw"
     buffer_names = ("data",)
     priority = -1
-    dtypes = None
-    lanes = {}
 
     def encode(self, weight, config: RawConfig) -> dict:
         return {"data": weight.detach().contiguous().clone()}
@@ -107,7 +138,7 @@ class RawScheme(Scheme):
 
     def validate_buffers(self, buffers, shape, dtype) -> None:
         data = buffers["data"]
-        if data.dtype != dtype or tuple(data.shape) != tuple(shape):
+        if (data.dtype, tuple(data.shape)) != (dtype, tuple(shape)):
             raise ValueError(f"raw buffer must be {tuple(shape)} {dtype}, got {tuple(data.shape)} {data.dtype}")
 
 

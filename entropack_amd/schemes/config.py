@@ -1,98 +1,116 @@
 """Config dataclasses and their validation.
 
-Same user-facing contract as the reference (entropack/schemes/config.py:8-111): every scheme has a dataclass
-deriving from `CompressionConfig`; fields carry `Annotated[type, Range | OneOf]` markers; `validate_config` raises
-TypeError for a wrong kind of value and ValueError for one outside its marker. `execution_backend` is not
-validated here: any string reaches the registry, which rejects unknown names with a DispatchError.
+User-facing contract of the reference (entropack/schemes/config.py:8-111): every scheme has a dataclass deriving
+from `CompressionConfig`; a field's annotation may carry constraint markers, `Annotated[int | None, Range(1, None)]`
+or `Annotated[int, OneOf((9, 10), silent=(0,))]`; `validate_config` raises TypeError for the wrong kind of value and
+ValueError for a value its markers refuse. `execution_backend` is left to the registry, which rejects unknown names
+with a DispatchError.
+
+Here a config class is compiled once into a list of `_Rule`s (kind of value, whether None passes, markers), and
+validation walks that list.
 """
-from dataclasses import dataclass, fields
-from numbers import Real
-from typing import Annotated, get_args, get_origin, get_type_hints
+import dataclasses
+import numbers
+import typing
 
 __all__ = ["CompressionConfig", "OneOf", "Range", "RawConfig", "validate_config"]
 
 
-@dataclass
+@dataclasses.dataclass
 class CompressionConfig:
     """Execution settings shared by all schemes. Pick a concrete subclass to pick a scheme."""
 
     #: "auto" / None picks the best usable backend; otherwise "hip" or "eager".
-    execution_backend: str | None = "auto"
+    execution_backend: typing.Optional[str] = "auto"
 
 
-@dataclass
+@dataclasses.dataclass
 class RawConfig(CompressionConfig):
     """Keep the values as they are (no entropy coding)."""
 
 
 class Range:
-    """Inclusive bounds; None leaves a side open."""
+    """Marker: low <= value <= high, either side open when None. `message` replaces the generated complaint."""
 
-    def __init__(self, low=None, high=None, *, message: str | None = None):
+    def __init__(self, low=None, high=None, *, message=None):
         self.low, self.high, self.message = low, high, message
 
-    def holds(self, value) -> bool:
-        return (self.low is None or value >= self.low) and (self.high is None or value <= self.high)
-
-    def describe(self, name: str) -> str:
+    def refusal(self, name: str, value):
+        """None if `value` passes, else the text of the ValueError."""
+        below = self.low is not None and value < self.low
+        above = self.high is not None and value > self.high
+        if not (below or above):
+            return None
         if self.message:
             return self.message
-        if self.low is None:
-            return f"{name} must be <= {self.high}"
-        if self.high is None:
-            return f"{name} must be >= {self.low}"
-        return f"{name} must be in [{self.low}, {self.high}]"
+        if self.low is not None and self.high is not None:
+            return f"{name} must be in [{self.low}, {self.high}]"
+        return f"{name} must be >= {self.low}" if self.high is None else f"{name} must be <= {self.high}"
 
 
 class OneOf:
-    """A closed set; `silent` values mean "choose for me" and pass as well."""
+    """Marker: value in a closed set; `silent` values mean "choose for me" and pass without being advertised."""
 
-    def __init__(self, choices, *, silent=(), message: str | None = None):
-        self.choices, self.silent, self.message = tuple(choices), frozenset(silent), message
+    def __init__(self, choices, *, silent=(), message=None):
+        self.choices, self.silent, self.message = tuple(choices), tuple(silent), message
 
-    def holds(self, value) -> bool:
-        return value in self.choices or value in self.silent
-
-    def describe(self, name: str) -> str:
+    def refusal(self, name: str, value):
+        if value in self.choices or value in self.silent:
+            return None
         return self.message or f"{name} must be one of {self.choices}"
 
 
-_field_hints: dict[type, dict] = {}
+class _Rule(typing.NamedTuple):
+    name: str
+    kind: type                  # bool, int or float ("any real number")
+    none_passes: bool
+    markers: tuple
 
+    _NOUNS = {bool: "a bool", int: "an integer", float: "a real number"}
 
-def _hints_of(klass: type) -> dict:
-    if klass not in _field_hints:
-        hints = get_type_hints(klass, include_extras=True)
-        _field_hints[klass] = {f.name: hints[f.name] for f in fields(klass) if f.name != "execution_backend"}
-    return _field_hints[klass]
-
-
-def _validate_field(name: str, value, hint) -> None:
-    markers = ()
-    if get_origin(hint) is Annotated:
-        hint, *markers = get_args(hint)
-    members = get_args(hint) if get_origin(hint) is not None else (hint,)
-    kinds = [m for m in members if m is not type(None)]
-    nullable = len(kinds) != len(members)
-    base = kinds[0]
-    noun = {int: "an integer", bool: "a bool"}.get(base, "a real number")
-    if value is None:
-        if nullable:
+    def apply(self, value) -> None:
+        noun = self._NOUNS[self.kind]
+        if value is None:
+            if not self.none_passes:
+                raise TypeError(f"{self.name} must be {noun}")
             return
-        raise TypeError(f"{name} must be {noun}")
-    if base is bool:
-        right_kind = isinstance(value, bool)
-    elif base is int:
-        right_kind = isinstance(value, int) and not isinstance(value, bool)
-    else:
-        right_kind = isinstance(value, Real) and not isinstance(value, bool)
-    if not right_kind:
-        raise TypeError(f"{name} must be {noun}{' or None' if nullable else ''}")
-    for marker in markers:
-        if not marker.holds(value):
-            raise ValueError(marker.describe(name))
+        is_bool = isinstance(value, bool)
+        if self.kind is bool:
+            fits = is_bool
+        elif self.kind is int:
+            fits = isinstance(value, int) and not is_bool
+        else:
+            fits = isinstance(value, numbers.Real) and not is_bool
+        if not fits:
+            raise TypeError(f"{self.name} must be {noun}" + (" or None" if self.none_passes else ""))
+        for marker in self.markers:
+            complaint = marker.refusal(self.name, value)
+            if complaint is not None:
+                raise ValueError(complaint)
+
+
+def _rule_for(name: str, annotation) -> _Rule:
+    markers = ()
+    if typing.get_origin(annotation) is typing.Annotated:
+        annotation, *found = typing.get_args(annotation)
+        markers = tuple(found)
+    alternatives = typing.get_args(annotation) or (annotation,)           # `int | None` -> (int, NoneType)
+    concrete = [kind for kind in alternatives if kind is not type(None)]
+    kind = concrete[0] if concrete[0] in (bool, int) else float
+    return _Rule(name, kind, len(concrete) < len(alternatives), markers)
+
+
+_compiled: dict = {}
+
+
+def _rules(config_class: type) -> tuple:
+    if config_class not in _compiled:
+        annotations = typing.get_type_hints(config_class, include_extras=True)
+        _compiled[config_class] = tuple(_rule_for(field.name, annotations[field.name]) for field in dataclasses.fields(config_class)
+                                        if field.name != "execution_backend")
+    return _compiled[config_class]
 
 
 def validate_config(config) -> None:
-    for name, hint in _hints_of(type(config)).items():
-        _validate_field(name, getattr(config, name), hint)
+    for rule in _rules(type(config)):
+        rule.apply(getattr(config, rule.name))

@@ -1,69 +1,78 @@
-"""The `lattice_rans` scheme: E8-lattice vector quantisation entropy-coded with tiled, 32-way interleaved rANS."""
+"""The `lattice_rans` scheme: E8-lattice vector quantisation entropy-coded with tiled, 32-way interleaved rANS.
+
+Public behaviour of the reference scheme (entropack/schemes/lattice_rans/__init__.py:13-58): 2-D inputs of the
+supported dtypes, columns padded to whole 8-vectors for the lane and cut back after decoding, buffers returned on the
+device the input came from. Lanes here: `hip` decodes on an MI355X, `eager` encodes on the CPU.
+"""
 import torch
 
 from ..base import Scheme, packed_buffers, register_scheme
-from .format import (
-    LATTICE_DIM, PACKED_KEYS, SUPPORTED_DTYPES, EntroPackLossyConfig, LatticeBuffers, LatticeRANSConfig,
-    recommended_tile_elements, validate_packed,
-)
+from . import format as _format
+from .format import EntroPackLossyConfig, LatticeBuffers, LatticeRANSConfig
 
 __all__ = ["EntroPackLossyConfig", "LatticeRANSConfig", "LatticeRANSScheme"]
 
+#: config fields handed to a lane's `encode` unchanged
+_PASSED_ON = ("row_rdo_iterations", "row_rdo_candidates", "scale_search_iterations", "scale_search_max_vectors")
+
+
+def _moved(buffers: LatticeBuffers, device) -> LatticeBuffers:
+    if device is None or buffers.layout.device == device:
+        return buffers
+    return LatticeBuffers(*(tensor.to(device) for tensor in buffers))
+
 
 class LatticeRANSScheme(Scheme):
-    """Same public behaviour as the reference scheme (entropack/schemes/lattice_rans/__init__.py:13-58), with a
-    `hip` lane for decoding on MI355X and an `eager` lane that encodes on the CPU."""
-
     name = "lattice_rans"
-    buffer_names = PACKED_KEYS
+    buffer_names = _format.PACKED_KEYS
     lossless = False
-    priority = 0
-    dtypes = SUPPORTED_DTYPES
+    dtypes = _format.SUPPORTED_DTYPES
     lanes = {"hip": "hip", "eager": "eager"}
 
-    def encode(self, weight: torch.Tensor, config: EntroPackLossyConfig) -> dict:
-        if weight.dtype not in SUPPORTED_DTYPES:
-            raise ValueError(f"{self.name} does not support dtype {weight.dtype}")
+    def _refuse(self, what: str):
+        raise ValueError(f"{self.name} {what}")
+
+    def _check_input(self, weight: torch.Tensor) -> None:
+        if weight.dtype not in self.dtypes:
+            self._refuse(f"does not support dtype {weight.dtype}")
         if weight.ndim != 2:
-            raise ValueError(f"{self.name} encode requires exactly 2D input, got {weight.ndim}D")
+            self._refuse(f"encode requires exactly 2D input, got {weight.ndim}D")
         if weight.numel() == 0:
-            raise ValueError(f"{self.name} does not support empty tensors")
-        if weight.dtype.is_floating_point and not bool(torch.isfinite(weight.float()).all()):
-            raise ValueError(f"{self.name} input must contain only finite values")
-        weight = weight.contiguous()
-        width = 1.0 if weight.dtype == torch.bool else weight.element_size() * 8.0
-        target_bpp = min(float(config.target_bpp), width)
-        home = weight.device
+            self._refuse("does not support empty tensors")
+        if weight.dtype.is_floating_point and not torch.isfinite(weight.float()).all().item():
+            self._refuse("input must contain only finite values")
+
+    def encode(self, weight: torch.Tensor, config: EntroPackLossyConfig) -> dict:
+        self._check_input(weight)
+        origin = weight.device
+        bits_per_element = 1.0 if weight.dtype == torch.bool else 8.0 * weight.element_size()
+        rate = min(float(config.target_bpp), bits_per_element)              # no point in asking for more than the input holds
         rows, cols = weight.shape
-        pad = -cols % LATTICE_DIM
-        if pad:
-            weight = torch.cat([weight, weight.new_zeros(rows, pad)], dim=1)
-        lane, lane_device = self.lane_for(weight, config.execution_backend)
-        if lane_device is not None and weight.device != lane_device:
-            weight = weight.to(lane_device)
-        tile_elements = recommended_tile_elements(target_bpp) if config.tile_elements is None else int(config.tile_elements)
-        packed = lane.encode(
-            weight=weight, target_bpp=target_bpp, prob_bits=None if config.prob_bits in (None, 0) else int(config.prob_bits),
-            tile_elements=tile_elements, row_rdo_iterations=config.row_rdo_iterations,
-            row_rdo_candidates=config.row_rdo_candidates, scale_search_iterations=config.scale_search_iterations,
-            scale_search_max_vectors=config.scale_search_max_vectors,
-        )
-        return {key: value.to(home) for key, value in packed._asdict().items()}
+        loose = cols % _format.LATTICE_DIM
+        matrix = weight.contiguous()
+        if loose:
+            matrix = torch.nn.functional.pad(matrix, (0, _format.LATTICE_DIM - loose))
+        lane, device = self.lane_for(matrix, config.execution_backend)
+        if device is not None:
+            matrix = matrix.to(device)
+        options = {name: getattr(config, name) for name in _PASSED_ON}
+        options["prob_bits"] = int(config.prob_bits) if config.prob_bits else None
+        options["tile_elements"] = _format.recommended_tile_elements(rate) if config.tile_elements is None else int(config.tile_elements)
+        packed = lane.encode(weight=matrix, target_bpp=rate, **options)
+        return {key: tensor.to(origin) for key, tensor in zip(LatticeBuffers._fields, packed)}
 
     def validate_buffers(self, buffers, shape, dtype):
-        validate_packed(buffers, tuple(shape), dtype)
+        _format.validate_packed(buffers, tuple(shape), dtype)
 
     def decode(self, packed: dict, *, shape, dtype: torch.dtype, config: EntroPackLossyConfig) -> torch.Tensor:
-        buffers = packed_buffers(packed, LatticeBuffers)
-        home = buffers.layout.device
-        lane, lane_device = self.lane_for(buffers.layout, config.execution_backend, gate_dtype=False)
-        if lane_device is not None and home != lane_device:
-            buffers = LatticeBuffers._make(value.to(lane_device) for value in buffers)
-        out = lane.decode(buffers, shape=shape, dtype=dtype, threads_per_block=config.threads_per_block,
-                          l2_prefetch=config.l2_prefetch)
-        if shape and tuple(out.shape) != tuple(shape):
-            out = out[: shape[0], : shape[1]]
-        return out if out.device == home else out.to(home)
+        held = packed_buffers(packed, LatticeBuffers)
+        origin = held.layout.device
+        lane, device = self.lane_for(held.layout, config.execution_backend, gate_dtype=False)
+        dense = lane.decode(_moved(held, device), shape=shape, dtype=dtype, threads_per_block=config.threads_per_block,
+                            l2_prefetch=config.l2_prefetch)
+        if shape and tuple(dense.shape) != tuple(shape):                     # the lane returns the padded columns
+            dense = dense[:shape[0], :shape[1]]
+        return dense.to(origin) if dense.device != origin else dense
 
 
 register_scheme(LatticeRANSScheme())

@@ -1,55 +1,59 @@
-"""The `tile_ans` scheme: lossless byte-lane coding, each lane raw or 32-way interleaved rANS over 256-symbol tables."""
+"""The `tile_ans` scheme: lossless byte-lane coding, each lane raw or 32-way interleaved rANS over 256-symbol tables.
+
+Public behaviour of the reference scheme (entropack/schemes/tile_ans/__init__.py:8-52): any tensor of a supported
+dtype, flattened; `tile_elements = 0` means 4096, or 8192 above 32 MiB of storage; buffers come back on the device the
+input was on. Lanes here: `hip` decodes on an MI355X, `eager` encodes on the CPU.
+"""
 import torch
 
 from ..base import Scheme, packed_buffers, register_scheme
-from .format import OPTIONS_BY_DTYPE, PACKED_KEYS, TileANSConfig, TileBuffers, validate_packed
+from . import format as _format
+from .format import TileANSConfig, TileBuffers
 
 __all__ = ["TileANSConfig", "TileANSScheme"]
 
-LARGE_TENSOR_BYTES = 32 * 1024 * 1024
+#: storage size above which automatic tile selection doubles the tile
+LARGE_TENSOR_BYTES = 32 << 20
+
+
+def _automatic_tile(weight: torch.Tensor) -> int:
+    return 8192 if weight.numel() * weight.element_size() > LARGE_TENSOR_BYTES else 4096
 
 
 class TileANSScheme(Scheme):
-    """Same public behaviour as the reference scheme (entropack/schemes/tile_ans/__init__.py:8-52), with a `hip` lane
-    for decoding on MI355X and an `eager` lane that encodes on the CPU."""
-
     name = "tile_ans"
-    buffer_names = PACKED_KEYS
-    priority = 100
-    dtypes = tuple(OPTIONS_BY_DTYPE)
+    buffer_names = _format.PACKED_KEYS
+    priority = 100                                      # the default scheme for every dtype it stores
+    dtypes = tuple(_format.OPTIONS_BY_DTYPE)
     lanes = {"hip": "hip", "eager": "eager"}
 
     def options_for(self, dtype):
-        tile_elements, probability_bits = OPTIONS_BY_DTYPE[dtype]
-        return {"tile_elements": tile_elements, "probability_bits": probability_bits,
-                "raw_lane_threshold": TileANSConfig().raw_lane_threshold}
+        tile_elements, probability_bits = _format.OPTIONS_BY_DTYPE[dtype]
+        defaults = TileANSConfig()
+        return dict(tile_elements=tile_elements, probability_bits=probability_bits, raw_lane_threshold=defaults.raw_lane_threshold)
 
     def encode(self, weight: torch.Tensor, config: TileANSConfig) -> dict:
-        if weight.numel() == 0:
+        if not weight.numel():
             raise ValueError(f"{self.name} does not support empty tensors")
-        weight = weight.contiguous()
-        tile_elements = config.tile_elements
-        if tile_elements == 0:
-            tile_elements = 4096 if weight.numel() * weight.element_size() <= LARGE_TENSOR_BYTES else 8192
-        home = weight.device
-        lane, lane_device = self.lane_for(weight, config.execution_backend)
-        if lane_device is not None and home != lane_device:
-            weight = weight.to(lane_device)
-        buffers = lane.encode(weight=weight, tile_elements=tile_elements, probability_bits=config.probability_bits,
-                              raw_lane_threshold=config.raw_lane_threshold, threads_per_block=config.threads_per_block)
-        return {key: value.to(home) for key, value in buffers._asdict().items()}
+        origin = weight.device
+        lane, device = self.lane_for(weight, config.execution_backend)
+        source = weight.contiguous() if device is None else weight.contiguous().to(device)
+        packed = lane.encode(weight=source, tile_elements=config.tile_elements or _automatic_tile(weight),
+                             probability_bits=config.probability_bits, raw_lane_threshold=config.raw_lane_threshold,
+                             threads_per_block=config.threads_per_block)
+        return {key: tensor.to(origin) for key, tensor in zip(TileBuffers._fields, packed)}
 
     def validate_buffers(self, buffers, shape, dtype):
-        validate_packed(buffers, shape, dtype)
+        _format.validate_packed(buffers, shape, dtype)
 
     def decode(self, packed: dict, *, shape, dtype: torch.dtype, config: TileANSConfig) -> torch.Tensor:
-        buffers = packed_buffers(packed, TileBuffers)
-        home = buffers.layout.device
-        lane, lane_device = self.lane_for(buffers.layout, config.execution_backend, gate_dtype=False)
-        if lane_device is not None and home != lane_device:
-            buffers = TileBuffers._make(value.to(lane_device) for value in buffers)
-        out = lane.decode(buffers, dtype=dtype, threads_per_block=config.threads_per_block).reshape(shape)
-        return out if out.device == home else out.to(home)
+        held = packed_buffers(packed, TileBuffers)
+        origin = held.layout.device
+        lane, device = self.lane_for(held.layout, config.execution_backend, gate_dtype=False)
+        if device is not None and device != origin:
+            held = TileBuffers(*(tensor.to(device) for tensor in held))
+        restored = lane.decode(held, dtype=dtype, threads_per_block=config.threads_per_block).reshape(shape)
+        return restored.to(origin) if restored.device != origin else restored
 
 
 register_scheme(TileANSScheme())

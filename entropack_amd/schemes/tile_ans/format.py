@@ -105,58 +105,62 @@ def lane_modes_cached(buffers: "TileBuffers") -> tuple[int, ...]:
                         "_tile_ans_lane_modes")
 
 
+def _stream_lengths(offsets: torch.Tensor, lane: int, tiles: int) -> torch.Tensor:
+    """Words of each of a byte lane's `tiles` streams."""
+    begin = lane * tiles
+    return offsets[begin + 1:begin + tiles + 1] - offsets[begin:begin + tiles]
+
+
 def validate_packed(buffers: dict, shape, dtype: torch.dtype) -> None:
-    """Structural checks of a container, with the reference's messages (format.py:96-164)."""
-    missing = [key for key in PACKED_KEYS if key not in buffers]
-    if missing:
-        raise ValueError(f"tile_ans packed data is missing buffers: {missing}")
-    if not all(isinstance(buffers[key], torch.Tensor) for key in PACKED_KEYS):
-        raise TypeError("tile_ans packed buffers must be torch.Tensor values")
-    for key, (wanted, ndim) in BUFFER_LAYOUT.items():
-        tensor = buffers[key]
+    """Everything that can be told about a container without decoding it: the six tensors exist with their dtypes and
+    ranks on one device, the layout matches `shape` / `dtype`, every table, state and offset array has the size the
+    layout implies, offsets cover the payload monotonically, raw streams have exactly their tiles' bytes.
+    Same checks and exception types as the reference's (schemes/tile_ans/format.py:96-164)."""
+    absent = sorted(set(PACKED_KEYS) - set(buffers))
+    if absent:
+        raise ValueError(f"tile_ans container lacks buffers {absent}")
+    held = {key: buffers[key] for key in PACKED_KEYS}
+    strangers = [key for key, value in held.items() if not isinstance(value, torch.Tensor)]
+    if strangers:
+        raise TypeError(f"tile_ans buffers must be tensors; {strangers} are not")
+    for key, tensor in held.items():
+        wanted_dtype, wanted_rank = BUFFER_LAYOUT[key]
+        if (tensor.dtype, tensor.ndim) != (wanted_dtype, wanted_rank):
+            raise ValueError(f"tile_ans buffer '{key}' must be {wanted_dtype} of rank {wanted_rank}, got {tensor.dtype} of shape {tuple(tensor.shape)}")
         if not tensor.is_contiguous():
             raise ValueError(f"tile_ans buffer '{key}' must be contiguous")
-        if tensor.dtype != wanted or tensor.ndim != ndim:
-            raise ValueError(f"tile_ans buffer '{key}' must be {ndim}D {wanted}, got shape={tuple(tensor.shape)}, dtype={tensor.dtype}")
-    devices = {buffers[key].device for key in PACKED_KEYS}
-    if len(devices) != 1:
-        raise ValueError(f"tile_ans packed buffers must share one device, got {devices}")
+    if len({tensor.device for tensor in held.values()}) > 1:
+        raise ValueError(f"tile_ans buffers sit on different devices: { {key: str(t.device) for key, t in held.items()} }")
 
-    tile_elements, prob_bits, num_lanes, num_elements = parse_layout(buffers["layout"])
-    element_size = torch.empty((), dtype=dtype).element_size()
-    if num_lanes != element_size:
-        raise ValueError(f"tile_ans layout has {num_lanes} byte lanes but dtype {dtype} uses {element_size} bytes")
-    shape = tuple(shape)
-    if any(not isinstance(dim, int) or dim < 0 for dim in shape):
-        raise ValueError(f"invalid tile_ans tensor shape: {shape}")
-    if math.prod(shape) != num_elements:
-        raise ValueError(f"tile_ans shape {shape} does not match {num_elements} elements")
+    tile_elements, prob_bits, num_lanes, num_elements = parse_layout(held["layout"])
+    dims = tuple(shape)
+    if not all(isinstance(dim, int) and dim >= 0 for dim in dims):
+        raise ValueError(f"tile_ans tensor shape {dims} is not a tuple of sizes")
+    if math.prod(dims) != num_elements:
+        raise ValueError(f"tile_ans container holds {num_elements} elements, shape {dims} asks for {math.prod(dims)}")
+    width = torch.empty((), dtype=dtype).element_size()
+    if width != num_lanes:
+        raise ValueError(f"tile_ans container has {num_lanes} byte lanes, {dtype} elements have {width} bytes")
 
     tiles = num_tiles(num_elements, tile_elements)
-    streams = tiles * num_lanes
-    if tuple(buffers["decode_tables"].shape) != (num_lanes, 1 << prob_bits):
-        raise ValueError("tile_ans decode_tables shape does not match layout")
-    if buffers["lane_modes"].numel() != num_lanes:
-        raise ValueError("tile_ans lane_modes length does not match layout")
-    modes = buffers["lane_modes"].detach().cpu()
-    if ((modes != LANE_ANS) & (modes != LANE_RAW)).any():
-        raise ValueError("tile_ans lane_modes contains an unknown codec mode")
-    coded = int((modes == LANE_ANS).sum())
-    if tuple(buffers["states"].shape) != (tiles * coded, NUM_STATES):
-        raise ValueError("tile_ans states shape does not match ANS lanes/layout")
-    if buffers["offsets"].numel() != streams + 1:
-        raise ValueError("tile_ans offsets length does not match layout")
-    offsets = buffers["offsets"].detach().cpu().to(torch.int64)
-    if offsets[0] != 0 or offsets[-1] != buffers["payload"].numel():
-        raise ValueError("tile_ans offsets endpoints are invalid")
-    if (offsets[1:] < offsets[:-1]).any():
-        raise ValueError("tile_ans offsets must be monotone")
-    last = num_elements - (tiles - 1) * tile_elements
-    for lane, mode in enumerate(modes.tolist()):
-        if mode != LANE_RAW:
-            continue
-        sizes = offsets[lane * tiles + 1: (lane + 1) * tiles + 1] - offsets[lane * tiles: (lane + 1) * tiles]
-        wanted = torch.full_like(sizes, (tile_elements + 1) // 2)
-        wanted[-1] = (last + 1) // 2
-        if not torch.equal(sizes, wanted):
-            raise ValueError("tile_ans raw lane payload length is invalid")
+    modes = held["lane_modes"].detach().cpu().tolist()
+    if len(modes) != num_lanes or any(mode not in (LANE_ANS, LANE_RAW) for mode in modes):
+        raise ValueError(f"tile_ans lane_modes must be {num_lanes} values of {LANE_ANS} (coded) or {LANE_RAW} (raw), got {modes}")
+    sizes = {
+        "decode_tables": (num_lanes, 1 << prob_bits),
+        "states": (tiles * modes.count(LANE_ANS), NUM_STATES),
+        "offsets": (tiles * num_lanes + 1,),
+    }
+    for key, wanted in sizes.items():
+        if tuple(held[key].shape) != wanted:
+            raise ValueError(f"tile_ans buffer '{key}' must have shape {wanted} for this layout, got {tuple(held[key].shape)}")
+
+    offsets = held["offsets"].detach().cpu().to(torch.int64)
+    if int(offsets[0]) != 0 or int(offsets[-1]) != held["payload"].numel() or bool((offsets.diff() < 0).any()):
+        raise ValueError("tile_ans offsets must rise from 0 to the payload length")
+    tail = num_elements - (tiles - 1) * tile_elements
+    for lane, mode in enumerate(modes):
+        if mode == LANE_RAW:
+            expect = [(tile_elements + 1) // 2] * (tiles - 1) + [(tail + 1) // 2]
+            if _stream_lengths(offsets, lane, tiles).tolist() != expect:
+                raise ValueError(f"tile_ans raw lane {lane} does not hold exactly its tiles' bytes")
