@@ -277,3 +277,47 @@ def test_skinny_gemm_workspace_matches_its_split():
     for case in [(16, 8192, 57344, 256), (128, 8192, 57344, 256), (128, 100000, 4096, 256), (65, 300, 1 << 20, 256), (3, 77, 16, 8)]:
         assert size(*case) == expect(*case), case
     assert size(0, 10, 10, 256) == 0 and size(4, 10, 10, 0) == 0
+
+
+def test_entry_points_refuse_bad_arguments_before_touching_a_device():
+    """Argument checks of the C ABI run on the host: every call here must come back with EP_HIP_EINVAL (or
+    EUNSUPPORTED) without a GPU in the machine. Pointers are small non-null integers that are never dereferenced."""
+    import ctypes
+    lib = hip_backend.library()
+    EINVAL, EUNSUPPORTED = hip_backend.EINVAL, hip_backend.EUNSUPPORTED
+    fake = 0x1000
+    modes = (ctypes.c_uint8 * 8)(1, 0, 0, 0, 0, 0, 0, 0)
+
+    def tile_ans(**over):
+        call = dict(payload=fake, words=10, offsets=fake, states=fake, tables=fake, modes=ctypes.addressof(modes), tile=4096, pb=10, lanes=2,
+                    elements=100, out=fake, error=fake)
+        call.update(over)
+        return lib.ep_hip_decode_tile_ans(call["payload"], call["words"], call["offsets"], call["states"], call["tables"], call["modes"],
+                                          call["tile"], call["pb"], call["lanes"], call["elements"], call["out"], call["error"], None)
+
+    assert tile_ans(offsets=None) == EINVAL and tile_ans(tables=None) == EINVAL and tile_ans(modes=None) == EINVAL
+    assert tile_ans(out=None) == EINVAL and tile_ans(error=None) == EINVAL
+    assert tile_ans(payload=None) == EINVAL                                    # words announced, none given
+    assert tile_ans(tile=0) == EINVAL and tile_ans(elements=0) == EINVAL
+    assert tile_ans(pb=8) == EINVAL and tile_ans(pb=13) == EINVAL
+    assert tile_ans(lanes=3) == EINVAL and tile_ans(lanes=16) == EINVAL
+    assert tile_ans(payload=fake + 1) == EINVAL                                # words are 2-byte aligned
+    assert tile_ans(words=1 << 32) == EINVAL
+    assert tile_ans(states=None) == EINVAL                                     # lane 1 is coded: states are needed
+    bad_modes = (ctypes.c_uint8 * 8)(1, 2, 0, 0, 0, 0, 0, 0)
+    assert tile_ans(modes=ctypes.addressof(bad_modes)) == EINVAL
+
+    def rotate(**over):
+        call = dict(x=fake, kind=0, rows=4, inner=256, ldx=256, group=64, codes=fake, scales=fake)
+        call.update(over)
+        return lib.ep_hip_rotate_quantize_rows(call["x"], call["kind"], call["rows"], call["inner"], call["ldx"], call["group"],
+                                               call["codes"], call["scales"], None)
+
+    assert rotate(x=None) == EINVAL and rotate(codes=None) == EINVAL and rotate(scales=None) == EINVAL
+    assert rotate(rows=0) == EINVAL and rotate(inner=0) == EINVAL and rotate(ldx=128) == EINVAL and rotate(kind=7) == EINVAL
+    for group in (0, 2, 8, 32, 100, 128):
+        assert rotate(group=group) == EINVAL                                   # not a power of four
+    assert rotate(inner=320, ldx=320, group=256) == EINVAL                     # does not divide the row
+    assert rotate(inner=2048, ldx=2048, group=1024) == EUNSUPPORTED            # a valid group, but not one this kernel rotates
+    assert rotate(x=fake + 2) == EUNSUPPORTED                                  # rows it cannot load four elements at a time
+    assert lib.ep_hip_quantize_rows(None, 0, 4, 256, 256, fake, fake, None) == EINVAL
