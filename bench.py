@@ -23,8 +23,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 
 #: HBM bytes per decode launch measured with two rocprofv3 --pmc runs of this script (FETCH_SIZE, scaled by the 2.0
-#: a plain 512 MiB copy calibrates it to, plus WRITE_SIZE, factor 1.0). Only the default workload has been measured.
-MEASURED_TRAFFIC_BYTES = {"target": 600_500_000}
+#: a plain 512 MiB copy calibrates it to, plus WRITE_SIZE, factor 1.0): the default workload and the lossless one.
+MEASURED_TRAFFIC_BYTES = {"target": 600_500_000, "tile_ans": 804_100_000}
 
 WORKLOADS = {
     # name: (rows, cols, sigma, seed, target_bpp, outliers)
@@ -369,7 +369,7 @@ def lossless_workload(args, ep):
         },
         "roofline": {
             "bound": "hbm", "achieved": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9, 3), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": None,
+            "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": MEASURED_TRAFFIC_BYTES["tile_ans"],
             "kernel_ms_avg": round(kernel_avg_ms, 5), "kernel_ms_median": round(kernel_ms[len(kernel_ms) // 2], 5),
         },
     }
