@@ -301,17 +301,25 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, 
   const uint32_t slot = x & (kTable - 1u);
   const uint32_t word_at = (((x >> 5) & (kTable / 32u - 1u)) << 3) + rs_base;
   const u32x2 rs = *reinterpret_cast<lds_u2>(static_cast<uintptr_t>(word_at));
-  const uint32_t index = static_cast<uint32_t>(__builtin_popcount(rs.x & ((1u << (x & 31u)) - 1u))) + rs.y;
+  // The bit-field extract takes its width from the low five bits of x: the bits of rs.x below slot % 32.
+  const uint32_t index = static_cast<uint32_t>(__builtin_popcount(__builtin_amdgcn_ubfe(rs.x, 0u, x))) + rs.y;
   const uint32_t fb = *reinterpret_cast<lds_u32>(static_cast<uintptr_t>(index << 2));
   p.e[field] = static_cast<uint32_t>(static_cast<int32_t>(*reinterpret_cast<lds_i16>(static_cast<uintptr_t>((index << 1) + val0))));
   const uint32_t next = __umul24(fb & 0xFFFFu, x >> PB) + slot - (fb >> 16);
   p.x = (!MASKED || valid_lane) ? next : x;
   uint32_t t, d, na, nb;
   uint32_t pos = uniform(p.pos);
-  asm volatile(EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("0")
-               : [x0] "+v"(p.x), [pos0] "+s"(pos), [t0] "=&v"(t), [d0] "=&v"(d), [na] "=&s"(na), [nb] "=&s"(nb)
-               : [ring0] "v"(p.ring), [shv] "v"(k.shv)
-               : "vcc", "scc", "memory");
+  if constexpr (MASKED) {
+    asm volatile(EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("0")
+                 : [x0] "+v"(p.x), [pos0] "+s"(pos), [t0] "=&v"(t), [d0] "=&v"(d), [na] "=&s"(na), [nb] "=&s"(nb)
+                 : [ring0] "v"(p.ring), [shv] "v"(k.shv)
+                 : "vcc", "scc", "memory");
+  } else {
+    asm volatile(EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_FULL
+                 : [x0] "+v"(p.x), [pos0] "+s"(pos), [t0] "=&v"(t), [d0] "=&v"(d), [na] "=&s"(na), [nb] "=&s"(nb)
+                 : [ring0] "v"(p.ring), [shv] "v"(k.shv)
+                 : "vcc", "scc", "memory");
+  }
   p.pos = pos;
 }
 
