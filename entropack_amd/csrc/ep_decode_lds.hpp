@@ -123,11 +123,10 @@ struct Pair {
   "v_and_b32 %[t" S "], %[slotmask], %[x" S "]\n"                \
   "v_lshrrev_b32 %[h" S "], %[pb], %[x" S "]\n"                  \
   "v_cmp_le_u32 vcc, %[f0s], %[t" S "]\n"                        \
+  "v_cndmask_b32 %[cb" S "], 0, %[f0v], vcc\n"                   \
+  "v_sub_u32 %[t" S "], %[t" S "], %[cb" S "]\n"                 \
   "v_cndmask_b32 %[d" S "], %[f0v], %[f1v], vcc\n"               \
-  "v_mul_u32_u24 %[h" S "], %[d" S "], %[h" S "]\n"              \
-  "v_cndmask_b32 %[d" S "], 0, %[f0v], vcc\n"                    \
-  "v_sub_u32 %[t" S "], %[t" S "], %[d" S "]\n"                  \
-  "v_add_u32 %[x" S "], %[h" S "], %[t" S "]\n"                  \
+  "v_mad_u32_u24 %[x" S "], %[d" S "], %[h" S "], %[t" S "]\n"   \
   "v_cndmask_b32 %[cb" S "], 0, %[ktab], vcc\n"
 
 // Values the steps take in scalar registers. They are wave-uniform by construction; saying so explicitly keeps the
