@@ -373,11 +373,11 @@ __global__ __launch_bounds__(256) void rotate_quantize_rows_kernel(const void* _
 // instructions per 6 fragment reads, accumulators in 128 registers, two waves per SIMD so that one wave's reads hide
 // behind the other's multiplies. Two LDS stages alternate, so a K step costs one barrier: the tile for step k + 1 is
 // written while step k is multiplied, and the global loads for step k + 2 are already in flight in registers.
-constexpr int kBigM = 256, kBigN = 256, kBigThreads = 512;
-constexpr int kBigStageBytes = (kBigM + kBigN) * kRowStride;
-constexpr int kBigLdsBytes = 2 * kBigStageBytes;
+constexpr int kBigM = 256, kBigThreads = 512;
 
-template <bool INT8, bool GUARD>      // GUARD = false: M, N multiples of 256 and K of one tile step, no bounds checks on loads
+// BN = 256 or 192 output columns per block tile (wave tiles 64 x 128 or 64 x 96): the narrower one gives products such
+// as 4096 x 3072 one tile per CU (16 x 16) where the square one leaves a quarter of the CUs idle (16 x 12).
+template <bool INT8, bool GUARD, int BN>      // GUARD = false: M, N multiples of the tile and K of one tile step, no bounds checks on loads
 __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                           const float* __restrict__ scale_a, const float* __restrict__ scale_b,
                                                           const void* __restrict__ bias, void* __restrict__ y, int M, int N,
@@ -387,13 +387,16 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wave_m = wave >> 1, wave_n = wave & 1;          // 4 x 2 waves of 64 x 128
-  const int m0 = blockIdx.y * kBigM, n0 = blockIdx.x * kBigN;
+  constexpr int WN = BN / 2, NJ = WN / 32;                  // columns and 32-wide matrix-core tiles per wave
+  constexpr int B_CHUNKS = BN * 8 / kBigThreads;            // 16-byte pieces of the B tile each thread moves
+  constexpr int kStageBytes = (kBigM + BN) * kRowStride;
+  const int wave_m = wave >> 1, wave_n = wave & 1;          // 4 x 2 waves of 64 x WN
+  const int m0 = blockIdx.y * kBigM, n0 = blockIdx.x * BN;
   const int frag_row = lane & 31;
   const int frag_k = (lane >> 5) * 16;
 
   // Per operand tile: 256 rows of 8 chunks of 16 bytes; thread t moves chunks t, t + 512, ..., 4 per operand.
-  uint4 reg_a[4], reg_b[4];
+  uint4 reg_a[4], reg_b[B_CHUNKS];
   auto fetch = [&](int64_t kb) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -401,24 +404,34 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
       const int r = chunk >> 3;
       const int64_t at = kb + 16 * (chunk & 7);
       reg_a[i] = make_uint4(0, 0, 0, 0);
-      reg_b[i] = make_uint4(0, 0, 0, 0);
       if (!GUARD || (m0 + r < M && at < k_bytes)) reg_a[i] = *reinterpret_cast<const uint4*>(a + (m0 + r) * lda_bytes + at);
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+      const int chunk = tid + kBigThreads * i;
+      const int r = chunk >> 3;
+      const int64_t at = kb + 16 * (chunk & 7);
+      reg_b[i] = make_uint4(0, 0, 0, 0);
       if (!GUARD || (n0 + r < N && at < k_bytes)) reg_b[i] = *reinterpret_cast<const uint4*>(b + (n0 + r) * ldb_bytes + at);
     }
   };
   auto stash = [&](int stage) {
-    uint8_t* tile_a = big_smem + stage * kBigStageBytes;
+    uint8_t* tile_a = big_smem + stage * kStageBytes;
     uint8_t* tile_b = tile_a + kBigM * kRowStride;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int chunk = tid + kBigThreads * i;
       *reinterpret_cast<uint4*>(tile_a + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = reg_a[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+      const int chunk = tid + kBigThreads * i;
       *reinterpret_cast<uint4*>(tile_b + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = reg_b[i];
     }
   };
 
   using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
-  Acc acc[2][4] = {};
+  Acc acc[2][NJ] = {};
   const int64_t steps = (k_bytes + kTileBytesK - 1) / kTileBytesK;
   fetch(0);
   stash(0);
@@ -428,30 +441,30 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
     const int stage = static_cast<int>(step & 1);
     if (step + 1 < steps) stash(stage ^ 1);
     if (step + 2 < steps) fetch((step + 2) * kTileBytesK);
-    const uint8_t* tile_a = big_smem + stage * kBigStageBytes + (wave_m * 64 + frag_row) * kRowStride + frag_k;
-    const uint8_t* tile_b = big_smem + stage * kBigStageBytes + (kBigM + wave_n * 128 + frag_row) * kRowStride + frag_k;
+    const uint8_t* tile_a = big_smem + stage * kStageBytes + (wave_m * 64 + frag_row) * kRowStride + frag_k;
+    const uint8_t* tile_b = big_smem + stage * kStageBytes + (kBigM + wave_n * WN + frag_row) * kRowStride + frag_k;
 #pragma unroll
     for (int kk = 0; kk < kTileBytesK / 32; ++kk) {
       if constexpr (INT8) {
-        i32x4 fa[2], fb[4];
+        i32x4 fa[2], fb[NJ];
 #pragma unroll
         for (int t = 0; t < 2; ++t) fa[t] = *reinterpret_cast<const i32x4*>(tile_a + t * 32 * kRowStride + kk * 32);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) fb[t] = *reinterpret_cast<const i32x4*>(tile_b + t * 32 * kRowStride + kk * 32);
+        for (int t = 0; t < NJ; ++t) fb[t] = *reinterpret_cast<const i32x4*>(tile_b + t * 32 * kRowStride + kk * 32);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
       } else {
-        bf16x8 fa[2], fb[4];
+        bf16x8 fa[2], fb[NJ];
 #pragma unroll
         for (int t = 0; t < 2; ++t) fa[t] = *reinterpret_cast<const bf16x8*>(tile_a + t * 32 * kRowStride + kk * 32);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) fb[t] = *reinterpret_cast<const bf16x8*>(tile_b + t * 32 * kRowStride + kk * 32);
+        for (int t = 0; t < NJ; ++t) fb[t] = *reinterpret_cast<const bf16x8*>(tile_b + t * 32 * kRowStride + kk * 32);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
       }
     }
     __syncthreads();
@@ -461,8 +474,8 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + wave_n * 128 + j * 32 + (lane & 31);
+    for (int j = 0; j < NJ; ++j) {
+      const int n = n0 + wave_n * WN + j * 32 + (lane & 31);
       if (n >= N) continue;
       const bool has_bias = bias != nullptr;
       const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
@@ -486,37 +499,43 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
   }
 }
 
-template <bool INT8, bool GUARD>
+template <bool INT8, bool GUARD, int BN>
 static int launch_big_variant(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                       int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
   static thread_local int configured_for = -1;
+  constexpr int kLdsBytes = 2 * (kBigM + BN) * kRowStride;
   int device = 0;
   EP_HIP_TRY(hipGetDevice(&device));
   if (configured_for != device) {
-    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_big_kernel<INT8, GUARD>), hipFuncAttributeMaxDynamicSharedMemorySize, kBigLdsBytes));
+    EP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_big_kernel<INT8, GUARD, BN>), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
     configured_for = device;
   }
-  const dim3 grid(static_cast<unsigned>((N + kBigN - 1) / kBigN), static_cast<unsigned>((M + kBigM - 1) / kBigM));
+  const dim3 grid(static_cast<unsigned>((N + BN - 1) / BN), static_cast<unsigned>((M + kBigM - 1) / kBigM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
-  hipLaunchKernelGGL((gemm_big_kernel<INT8, GUARD>), grid, dim3(kBigThreads), kBigLdsBytes, stream, static_cast<const uint8_t*>(a),
+  hipLaunchKernelGGL((gemm_big_kernel<INT8, GUARD, BN>), grid, dim3(kBigThreads), kLdsBytes, stream, static_cast<const uint8_t*>(a),
                      static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
                      lda_bytes, ldb_bytes, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }
 
-template <bool INT8>
+template <bool INT8, int BN>
 static int launch_big(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                       int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
-  const bool interior = M % kBigM == 0 && N % kBigN == 0 && k_bytes % kTileBytesK == 0;
-  return interior ? launch_big_variant<INT8, false>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream)
-                  : launch_big_variant<INT8, true>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream);
+  const bool interior = M % kBigM == 0 && N % BN == 0 && k_bytes % kTileBytesK == 0;
+  return interior ? launch_big_variant<INT8, false, BN>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream)
+                  : launch_big_variant<INT8, true, BN>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream);
 }
 
-// The big tiles pay once a product has one of them for every CU of the device (256 on MI355X); below that the
-// 128 x 128 kernel spreads the work over more CUs (measured equal for bf16 and faster for int8 at 192 tiles).
-static bool big_tiles_pay(int64_t M, int64_t N) {
-  return M >= kBigM && N >= kBigN && ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN) >= 256;
+// Which block tile a product takes: 256 x 256 once there is one for every CU (256 on MI355X); else 256 x 192 if that
+// shape gives at least nine tenths of the CUs a tile; else the 128 x 128 kernel, which spreads small products over
+// more CUs. Returns the tile's column count, 0 for the 128 x 128 kernel.
+static int big_tile_columns(int64_t M, int64_t N) {
+  if (M < kBigM) return 0;
+  const int64_t rows = (M + kBigM - 1) / kBigM;
+  if (N >= 256 && rows * ((N + 255) / 256) >= 256) return 256;
+  if (N >= 192 && rows * ((N + 191) / 192) >= 230) return 192;
+  return 0;
 }
 
 // ---- few activation rows (M <= 128): the weight stream bounds the product ---------------------------------------------------
@@ -727,9 +746,10 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  if (big_tiles_pay(M, N)) {
-    return launch_big<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind,
-                             static_cast<hipStream_t>(stream));
+  if (const int columns = big_tile_columns(M, N)) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return columns == 256 ? launch_big<false, 256>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s)
+                          : launch_big<false, 192>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s);
   }
   const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
@@ -786,9 +806,10 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
   if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  if (big_tiles_pay(M, N)) {
-    return launch_big<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind,
-                            static_cast<hipStream_t>(stream));
+  if (const int columns = big_tile_columns(M, N)) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return columns == 256 ? launch_big<true, 256>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s)
+                          : launch_big<true, 192>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s);
   }
   const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
