@@ -8,10 +8,11 @@
 //
 //   tile_ans_stream_kernel   any container: one stream per 32-lane half, table and words read from global memory
 //                            (L2-resident), every renormalisation read bounds-checked, bytes stored one by one.
-//   tile_ans_tile_kernel     containers with exactly one coded lane (bf16 / f16: raw low byte + coded high byte,
-//                            f32: three raw + one coded, 1-byte types): one tile per 32-lane half, the lane's table
-//                            in LDS, the words through the LDS windows and the scalar vote of the lattice decoder,
-//                            raw bytes fetched one group ahead, whole elements stored.
+//   tile_ans_tile_kernel     containers with at most four coded lanes (weights: bf16 / f16 raw low byte + coded high
+//                            byte, f32 three raw + one coded, 1-byte types; integers with constant upper bytes; all
+//                            raw): one tile per 32-lane half, the coded lanes' tables in LDS, the words through the
+//                            LDS windows and the scalar vote of the lattice decoder, raw bytes fetched 256 elements
+//                            ahead, whole elements stored 8 at a time.
 #include "ep_decode_lds.hpp"
 
 namespace ep {
@@ -30,7 +31,6 @@ struct TileAnsArgs {
   int64_t tiles;
   int prob_bits;
   int lanes;
-  int coded_lane;                        // tile kernel: the one coded lane
   int wide_stores;                       // tile kernel: `out` is 16-byte aligned
   int* error;
   uint8_t raw[kMaxByteLanes];            // 1 = raw lane
@@ -114,12 +114,14 @@ __global__ __launch_bounds__(256) void tile_ans_stream_kernel(TileAnsArgs a) {
   decode_stream(a, stream, stream < a.tiles * a.lanes, half, lane & 31);
 }
 
-// ---- one coded lane ----------------------------------------------------------------------------------------------------
+// ---- tiles: every lane of a tile in one wave -------------------------------------------------------------------------------
 //
-// LDS: the coded lane's table as 2^pb entries freq[0:12) | (slot - cdf)[12:24) | symbol << 24 at offset 0 (the byte
-// form of the lattice decoder, so its step applies unchanged), then one 128-word window per half. A table that
-// holds a frequency of 4096 (a one-symbol lane at prob_bits 12) does not fit that entry; a workgroup that meets one
-// decodes its tiles stream by stream as the general kernel does.
+// One tile per 32-lane half, all of its byte lanes together, whole elements stored. LDS: per coded lane its table as
+// 2^pb entries freq[0:12) | (slot - cdf)[12:24) | symbol << 24 (the byte form of the lattice decoder, so its step
+// applies unchanged; table c at offset c * 4 * 2^pb, the first at 0), then per half and coded lane one 128-word
+// window and 256 bytes where the steps leave their symbols. A table that holds a frequency of 4096 (a one-symbol
+// lane at prob_bits 12) does not fit that entry; a workgroup that meets one decodes its tiles stream by stream as
+// the general kernel does.
 
 template <int BYTES> struct ElementWord;
 template <> struct ElementWord<1> { using type = uint8_t; };
@@ -145,12 +147,18 @@ __device__ __forceinline__ uint32_t tile_ans_step(Pair& p, uint32_t pb, uint32_t
   return e >> 24;
 }
 
-template <int BYTES>
-__global__ __launch_bounds__(1024, BYTES == 8 ? 4 : 8) void tile_ans_tile_kernel(TileAnsArgs a, int num_pairs) {
+constexpr int kTileChunk = 256;                      // elements a half gathers before it stores
+constexpr int tile_kernel_waves_per_simd(int bytes, int coded) { return (coded <= 1 && bytes <= 4) ? 8 : 4; }
+
+template <int BYTES, int CODED>
+__global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) void tile_ans_tile_kernel(TileAnsArgs a, int num_pairs) {
   extern __shared__ __align__(16) uint8_t smem[];
   using Word = typename ElementWord<BYTES>::type;
-  constexpr int RAW = BYTES - 1;
+  constexpr int RAW = BYTES - CODED;
+  constexpr int NC = CODED > 0 ? CODED : 1, NR = RAW > 0 ? RAW : 1;       // array sizes
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   const uint32_t pb = uniform(static_cast<uint32_t>(a.prob_bits));
   const uint32_t table_bytes = 4u << pb;
   const int waves = blockDim.x >> 6;
@@ -159,15 +167,34 @@ __global__ __launch_bounds__(1024, BYTES == 8 ? 4 : 8) void tile_ans_tile_kernel
   const int half = lane >> 5;
   const int l32 = lane & 31;
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr)smem));
-  const int coded_lane = __builtin_amdgcn_readfirstlane(a.coded_lane);
+  const uint32_t windows0 = CODED * table_bytes;
+  const uint32_t stages0 = windows0 + static_cast<uint32_t>(waves) * 2 * CODED * kRingBytes;
+  const uint32_t flag0 = stages0 + static_cast<uint32_t>(waves) * 2 * CODED * kTileChunk;
 
-  // One word behind the windows says whether the table holds a frequency the 12-bit field cannot.
-  volatile uint32_t* wide_flag = reinterpret_cast<volatile uint32_t*>(smem + table_bytes + static_cast<uint32_t>(waves) * 2 * kRingBytes);
+  // Byte positions inside an element: the coded lanes and the raw lanes, each ascending.
+  int coded_pos[NC], raw_pos[NR];
+  {
+    int c = 0, r = 0;
+#pragma unroll
+    for (int b = 0; b < BYTES; ++b) {
+      const bool is_raw = __builtin_amdgcn_readfirstlane(static_cast<int>(a.raw[b])) != 0;
+#pragma unroll
+      for (int i = 0; i < NC; ++i) if (CODED > 0 && !is_raw && c == i) coded_pos[i] = b;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) if (RAW > 0 && is_raw && r == i) raw_pos[i] = b;
+      c += is_raw ? 0 : 1;
+      r += is_raw ? 1 : 0;
+    }
+  }
+
+  // One word behind the staging areas says whether a table holds a frequency the 12-bit field cannot.
+  volatile uint32_t* wide_flag = reinterpret_cast<volatile uint32_t*>(smem + flag0);
   if (threadIdx.x == 0) *wide_flag = 0u;
   __syncthreads();
-  {
-    const uint32_t* table = a.tables + (static_cast<size_t>(coded_lane) << pb);
-    uint32_t* dst = reinterpret_cast<uint32_t*>(smem);
+#pragma unroll
+  for (int c = 0; c < CODED; ++c) {
+    const uint32_t* table = a.tables + (static_cast<size_t>(coded_pos[c]) << pb);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(smem + c * table_bytes);
     for (uint32_t slot = threadIdx.x; slot < (1u << pb); slot += blockDim.x) {
       const uint32_t entry = table[slot];
       const uint32_t freq = (entry >> 8) & 0xFFFu;
@@ -177,7 +204,7 @@ __global__ __launch_bounds__(1024, BYTES == 8 ? 4 : 8) void tile_ans_tile_kernel
   }
   __syncthreads();
   const bool wide = *wide_flag != 0u;
-  if (lds0 != 0) {      // the step addresses the table from LDS offset 0
+  if (lds0 != 0) {      // the step addresses the tables from LDS offset 0
     if (threadIdx.x == 0) tile_ans_flag(a.error, EP_DECODE_BAD_OFFSETS);
     return;
   }
@@ -191,101 +218,107 @@ __global__ __launch_bounds__(1024, BYTES == 8 ? 4 : 8) void tile_ans_tile_kernel
   }
 
   const uint32_t kslot = table_bytes - 4u;
-  uint32_t shv = half ? 16u : 0u, table_at = 0u;
-  asm volatile("" : "+v"(shv), "+v"(table_at));     // the step names them as vector operands
+  uint32_t shv = half ? 16u : 0u;
+  uint32_t table_at[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) table_at[c] = static_cast<uint32_t>(c) * table_bytes;
+  asm volatile("" : "+v"(shv));                           // the step names it as a vector operand
+#pragma unroll
+  for (int c = 0; c < NC; ++c) asm volatile("" : "+v"(table_at[c]));
   const uint32_t* payload32 = reinterpret_cast<const uint32_t*>(a.payload);
   const uint8_t* payload8 = reinterpret_cast<const uint8_t*>(a.payload);
-  const uint32_t window_at = lds0 + table_bytes + static_cast<uint32_t>(wave * 2 + half) * kRingBytes;
-  // Byte positions of the raw lanes inside an element: every lane but the coded one, ascending.
-  int raw_lane[RAW > 0 ? RAW : 1];
-#pragma unroll
-  for (int j = 0; j < RAW; ++j) raw_lane[j] = j + (j >= coded_lane ? 1 : 0);
+  const uint32_t mine_at = static_cast<uint32_t>(wave * 2 + half) * CODED;
   const int tile_elements = static_cast<int>(a.tile_elements);
-  constexpr int kChunk = 256;                     // elements a half gathers before it stores
-  const uint32_t stage_at = lds0 + table_bytes + static_cast<uint32_t>(waves) * 2 * kRingBytes + 16u + static_cast<uint32_t>(wave * 2 + half) * kChunk;
 
   for (int pair = static_cast<int>(blockIdx.x) * waves + wave; pair < num_pairs; pair += stride) {
-    Pair s;
+    Pair st[NC];
     const int64_t tile = 2 * static_cast<int64_t>(pair) + half;
-    uint32_t word_begin = 0, word_end = 0;
+    uint32_t begin[NC], end[NC];
+    uint32_t raw_at[NR];       // a raw lane's bytes of this tile are consecutive payload bytes: this tile's first
     int count = 0;
-    uint32_t raw_at[RAW > 0 ? RAW : 1];       // a raw lane's bytes of this tile are consecutive payload bytes: this lane's first
 #pragma unroll
-    for (int j = 0; j < RAW; ++j) raw_at[j] = 0;
-    s.x = kStateMin;
+    for (int c = 0; c < NC; ++c) {
+      begin[c] = end[c] = 0;
+      st[c].x = kStateMin;
+    }
+#pragma unroll
+    for (int j = 0; j < NR; ++j) raw_at[j] = 0;
     if (tile < a.tiles) {
       const int64_t left = a.elements - tile * a.tile_elements;
       count = static_cast<int>(left < a.tile_elements ? left : a.tile_elements);
-      const int64_t coded_stream = static_cast<int64_t>(coded_lane) * a.tiles + tile;
-      word_begin = a.offsets[coded_stream];
-      word_end = a.offsets[coded_stream + 1];
-      bool good = word_begin <= word_end && word_end <= a.payload_words;
+      bool good = true;
+#pragma unroll
+      for (int c = 0; c < CODED; ++c) {
+        const int64_t stream = static_cast<int64_t>(coded_pos[c]) * a.tiles + tile;
+        begin[c] = a.offsets[stream];
+        end[c] = a.offsets[stream + 1];
+        good = good && begin[c] <= end[c] && end[c] <= a.payload_words;
+      }
 #pragma unroll
       for (int j = 0; j < RAW; ++j) {
-        const int64_t raw_stream = static_cast<int64_t>(raw_lane[j]) * a.tiles + tile;
-        const uint32_t from = a.offsets[raw_stream], to = a.offsets[raw_stream + 1];
+        const int64_t stream = static_cast<int64_t>(raw_pos[j]) * a.tiles + tile;
+        const uint32_t from = a.offsets[stream], to = a.offsets[stream + 1];
         good = good && from <= to && to <= a.payload_words && to - from == static_cast<uint32_t>((count + 1) >> 1);
-        raw_at[j] = 2u * from + static_cast<uint32_t>(l32);      // the launcher keeps the payload below 4 GiB
+        raw_at[j] = 2u * from;                                   // the launcher keeps the payload below 4 GiB
       }
       if (!good) {
         if (l32 == 0) tile_ans_flag(a.error, EP_DECODE_BAD_OFFSETS);
         count = 0;
-        word_begin = word_end = 0;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) begin[c] = end[c] = 0;
       } else {
-        s.x = a.states[tile * kStatesPerTile + l32];
+#pragma unroll
+        for (int c = 0; c < CODED; ++c) st[c].x = a.states[(static_cast<int64_t>(c) * a.tiles + tile) * kStatesPerTile + l32];
       }
     }
-    open_window(s, window_at, word_begin, word_end, a.payload, a.payload_words, l32);
+#pragma unroll
+    for (int c = 0; c < CODED; ++c) open_window(st[c], lds0 + windows0 + (mine_at + c) * kRingBytes, begin[c], end[c], a.payload, a.payload_words, l32);
     // Wave-uniform base, 32-bit lane offsets: the addresses cost one vector add per access.
     Word* out = reinterpret_cast<Word*>(a.out) + 2 * static_cast<int64_t>(pair) * a.tile_elements;
-    const uint32_t out_lane = static_cast<uint32_t>(half * tile_elements + l32);
+    const uint32_t out_half = static_cast<uint32_t>(half * tile_elements);
 
-    auto fetch_raw = [&](int at, bool valid_lane, uint32_t (&bytes)[RAW > 0 ? RAW : 1]) {
-#pragma unroll
-      for (int j = 0; j < RAW; ++j) bytes[j] = valid_lane ? payload8[raw_at[j] + static_cast<uint32_t>(at)] : 0u;
-    };
-    auto emit = [&](int at, uint32_t symbol, const uint32_t (&bytes)[RAW > 0 ? RAW : 1]) {
-      Word value = static_cast<Word>(static_cast<Word>(symbol) << (8 * coded_lane));
-#pragma unroll
-      for (int j = 0; j < RAW; ++j) value |= static_cast<Word>(static_cast<Word>(bytes[j]) << (8 * raw_lane[j]));
-      __builtin_nontemporal_store(value, out + (out_lane + static_cast<uint32_t>(at)));
-    };
-
-    const bool full = count == tile_elements && (tile_elements % kChunk) == 0 && a.wide_stores != 0;
+    const bool full = count == tile_elements && (tile_elements % kTileChunk) == 0 && a.wide_stores != 0;
     const bool all_full = __builtin_amdgcn_readfirstlane(__all(full) ? 1 : 0) != 0;
     if (all_full) {
-      // Chunks of eight groups. The steps leave their symbols in this half's 256 bytes of LDS; then lane l takes
-      // elements 8 l .. 8 l + 7 of the chunk: their symbols from LDS, 8 bytes of each raw lane from the payload
-      // (requested before the steps), and stores the 8 elements as one piece. One memory instruction per raw lane
-      // and 16 bytes of output per chunk, instead of one per group: the per-CU address path is the bottleneck otherwise.
-      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      // Chunks of eight groups. The steps leave their symbols in LDS; then lane l takes elements 8 l .. 8 l + 7 of
+      // the chunk: their symbols from LDS, 8 bytes of each raw lane from the payload (requested before the steps),
+      // and stores the 8 elements as one piece. One memory instruction per raw lane and per 16 bytes of output for a
+      // whole chunk, instead of one per group: the per-CU address path is the bottleneck otherwise.
       const uint32_t mine = 8u * static_cast<uint32_t>(l32);
 #pragma unroll 1
-      for (int at = tile_elements - kChunk; at >= 0; at -= kChunk) {
-        u32x2 raw[RAW > 0 ? RAW : 1];
+      for (int at = tile_elements - kTileChunk; at >= 0; at -= kTileChunk) {
+        u32x2 raw[NR], symbols[NC];
 #pragma unroll
-        for (int j = 0; j < RAW; ++j) __builtin_memcpy(&raw[j], payload8 + (raw_at[j] - static_cast<uint32_t>(l32) + static_cast<uint32_t>(at) + mine), 8);
+        for (int j = 0; j < RAW; ++j) __builtin_memcpy(&raw[j], payload8 + (raw_at[j] + static_cast<uint32_t>(at) + mine), 8);
 #pragma unroll
-        for (int g = kChunk / 32 - 1; g >= 0; --g) {
-          const uint32_t symbol = tile_ans_step<false>(s, pb, kslot, table_at, shv, ~0ull);
-          *reinterpret_cast<__attribute__((address_space(3))) uint8_t*>(static_cast<uintptr_t>(stage_at + 32u * g + l32)) = static_cast<uint8_t>(symbol);
-          if ((g & 1) == 0) slide_window(s, half, payload32);     // a step takes at most 32 words, the window holds 64
+        for (int g = kTileChunk / 32 - 1; g >= 0; --g) {
+#pragma unroll
+          for (int c = 0; c < CODED; ++c) {
+            const uint32_t symbol = tile_ans_step<false>(st[c], pb, kslot, table_at[c], shv, ~0ull);
+            const uint32_t stage = lds0 + stages0 + (mine_at + c) * kTileChunk;
+            *reinterpret_cast<__attribute__((address_space(3))) uint8_t*>(static_cast<uintptr_t>(stage + 32u * g + l32)) = static_cast<uint8_t>(symbol);
+            if ((g & 1) == 0) slide_window(st[c], half, payload32);     // a step takes at most 32 words, the window holds 64
+          }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        const u32x2 symbols = *reinterpret_cast<__attribute__((address_space(3))) const u32x2*>(static_cast<uintptr_t>(stage_at + mine));
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        Word* to = out + (out_lane - static_cast<uint32_t>(l32) + static_cast<uint32_t>(at) + mine);
+        if constexpr (CODED > 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int c = 0; c < CODED; ++c) {
+            symbols[c] = *reinterpret_cast<__attribute__((address_space(3))) const u32x2*>(static_cast<uintptr_t>(lds0 + stages0 + (mine_at + c) * kTileChunk + mine));
+          }
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        Word* to = out + (out_half + static_cast<uint32_t>(at) + mine);
         if constexpr (BYTES == 1) {
-          __builtin_nontemporal_store(symbols, reinterpret_cast<u32x2*>(to));
-        } else if constexpr (BYTES == 2) {
+          __builtin_nontemporal_store(CODED == 1 ? symbols[0] : raw[0], reinterpret_cast<u32x2*>(to));
+        } else if constexpr (BYTES == 2 && CODED == 1) {
           // v_perm_b32 picks bytes from {second operand: 0..3, first operand: 4..7}.
           u32x4 v;
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            const uint32_t low = coded_lane == 0 ? symbols[d >> 1] : raw[0][d >> 1];
-            const uint32_t high = coded_lane == 0 ? raw[0][d >> 1] : symbols[d >> 1];
+            const uint32_t low = coded_pos[0] == 0 ? symbols[0][d >> 1] : raw[0][d >> 1];
+            const uint32_t high = coded_pos[0] == 0 ? raw[0][d >> 1] : symbols[0][d >> 1];
             v[d] = __builtin_amdgcn_perm(high, low, (d & 1) ? 0x07030602u : 0x05010400u);
           }
           __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(to));
@@ -293,20 +326,28 @@ __global__ __launch_bounds__(1024, BYTES == 8 ? 4 : 8) void tile_ans_tile_kernel
           Word e[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            e[i] = static_cast<Word>(static_cast<Word>((symbols[i >> 2] >> (8 * (i & 3))) & 0xFFu) << (8 * coded_lane));
+            e[i] = 0;
 #pragma unroll
-            for (int j = 0; j < RAW; ++j) e[i] |= static_cast<Word>(static_cast<Word>((raw[j][i >> 2] >> (8 * (i & 3))) & 0xFFu) << (8 * raw_lane[j]));
+            for (int c = 0; c < CODED; ++c) e[i] |= static_cast<Word>(static_cast<Word>((symbols[c][i >> 2] >> (8 * (i & 3))) & 0xFFu) << (8 * coded_pos[c]));
+#pragma unroll
+            for (int j = 0; j < RAW; ++j) e[i] |= static_cast<Word>(static_cast<Word>((raw[j][i >> 2] >> (8 * (i & 3))) & 0xFFu) << (8 * raw_pos[j]));
           }
+          if constexpr (BYTES == 2) {
+            const u32x4 v = {static_cast<uint32_t>(e[0]) | static_cast<uint32_t>(e[1]) << 16, static_cast<uint32_t>(e[2]) | static_cast<uint32_t>(e[3]) << 16,
+                             static_cast<uint32_t>(e[4]) | static_cast<uint32_t>(e[5]) << 16, static_cast<uint32_t>(e[6]) | static_cast<uint32_t>(e[7]) << 16};
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(to));
+          } else {
 #pragma unroll
-          for (int q = 0; q < BYTES / 2; ++q) {
-            u32x4 v;
-            if constexpr (BYTES == 4) {
-              v = u32x4{e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]};
-            } else {
-              v = u32x4{static_cast<uint32_t>(e[2 * q]), static_cast<uint32_t>(static_cast<uint64_t>(e[2 * q]) >> 32),
-                        static_cast<uint32_t>(e[2 * q + 1]), static_cast<uint32_t>(static_cast<uint64_t>(e[2 * q + 1]) >> 32)};
+            for (int q = 0; q < BYTES / 2; ++q) {
+              u32x4 v;
+              if constexpr (BYTES == 4) {
+                v = u32x4{static_cast<uint32_t>(e[4 * q]), static_cast<uint32_t>(e[4 * q + 1]), static_cast<uint32_t>(e[4 * q + 2]), static_cast<uint32_t>(e[4 * q + 3])};
+              } else {
+                v = u32x4{static_cast<uint32_t>(e[2 * q]), static_cast<uint32_t>(static_cast<uint64_t>(e[2 * q]) >> 32),
+                          static_cast<uint32_t>(e[2 * q + 1]), static_cast<uint32_t>(static_cast<uint64_t>(e[2 * q + 1]) >> 32)};
+              }
+              __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(to) + q);
             }
-            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(to) + q);
           }
         }
       }
@@ -319,47 +360,102 @@ __global__ __launch_bounds__(1024, BYTES == 8 ? 4 : 8) void tile_ans_tile_kernel
       for (int round = 0; round < rounds; ++round) {
         const int lanes_now = (round == 0 && rem != 0) ? rem : 32;
         const bool valid_lane = round < groups && l32 < lanes_now;
-        const int at = (groups - 1 - round) << 5;
-        uint32_t now[RAW > 0 ? RAW : 1];
-        fetch_raw(at, valid_lane, now);
-        const uint32_t symbol = tile_ans_step<true>(s, pb, kslot, table_at, shv, __builtin_amdgcn_ballot_w64(valid_lane));
-        if (valid_lane) emit(at, symbol, now);
-        slide_window(s, half, payload32);
+        const uint32_t at = static_cast<uint32_t>((groups - 1 - round) << 5) + static_cast<uint32_t>(l32);
+        Word value = 0;
+#pragma unroll
+        for (int j = 0; j < RAW; ++j) {
+          const uint32_t byte = valid_lane ? payload8[raw_at[j] + at] : 0u;
+          value |= static_cast<Word>(static_cast<Word>(byte) << (8 * raw_pos[j]));
+        }
+        const uint64_t valid = __builtin_amdgcn_ballot_w64(valid_lane);
+#pragma unroll
+        for (int c = 0; c < CODED; ++c) {
+          const uint32_t symbol = tile_ans_step<true>(st[c], pb, kslot, table_at[c], shv, valid);
+          value |= static_cast<Word>(static_cast<Word>(symbol) << (8 * coded_pos[c]));
+          slide_window(st[c], half, payload32);
+        }
+        if (valid_lane) __builtin_nontemporal_store(value, out + (out_half + at));
       }
     }
 
     // A valid stream ends with every word consumed.
     const uint64_t live = __builtin_amdgcn_ballot_w64(count > 0);
     const bool liveA = (live & 1u) != 0, liveB = ((live >> 32) & 1u) != 0;
-    const int ptrA = window_pointer_a(s), ptrB = window_pointer_b(s);
-    if (((liveA && ptrA != s.beginA) || (liveB && ptrB != s.beginB)) && lane == 0) {
-      const bool over = (liveA && ptrA < s.beginA) || (liveB && ptrB < s.beginB);
-      tile_ans_flag(a.error, over ? EP_DECODE_OVERREAD : EP_DECODE_NOT_CONSUMED);
+#pragma unroll
+    for (int c = 0; c < CODED; ++c) {
+      const int ptrA = window_pointer_a(st[c]), ptrB = window_pointer_b(st[c]);
+      if (((liveA && ptrA != st[c].beginA) || (liveB && ptrB != st[c].beginB)) && lane == 0) {
+        const bool over = (liveA && ptrA < st[c].beginA) || (liveB && ptrB < st[c].beginB);
+        tile_ans_flag(a.error, over ? EP_DECODE_OVERREAD : EP_DECODE_NOT_CONSUMED);
+      }
     }
   }
 }
 
-template <int BYTES>
+constexpr size_t kLdsLimitBytes = 160 * 1024;
+
+static size_t tile_kernel_lds_bytes(int prob_bits, int coded, int waves) {
+  return static_cast<size_t>(coded) * (size_t{4} << prob_bits) + static_cast<size_t>(waves) * 2 * coded * (kRingBytes + kTileChunk) + 16;
+}
+
+template <int BYTES, int CODED>
 static hipError_t launch_tile_kernel(const TileAnsArgs& args, int compute_units, hipStream_t stream) {
+  static thread_local int configured_for = -1;
   const int64_t pairs = (args.tiles + 1) / 2;
-  const int64_t resident = (BYTES == 8 ? 1 : 2) * static_cast<int64_t>(compute_units);
-  // A pair is one long serial chain, so the grid walks the pairs in rounds, and a round costs about as much as it
-  // has waves per SIMD (the steps are issue-bound from two waves per SIMD up): take the workgroup size whose last
-  // round is fullest.
-  int waves = 16;
+  const int waves_per_cu = 4 * tile_kernel_waves_per_simd(BYTES, CODED);
+  // A pair is one long serial chain, so the grid walks the pairs in passes, and a pass costs about as much as it has
+  // waves per SIMD (the steps are issue-bound from a few waves per SIMD up): among the workgroup sizes that fit LDS
+  // and registers, take the one whose passes are fullest.
+  int waves = 0, resident = 0;
   int64_t best = INT64_MAX;
-  for (int w = 16; w >= 8; --w) {
-    const int64_t rounds = (pairs + resident * w - 1) / (resident * w);
-    if (rounds * w < best) {
-      best = rounds * w;
+  for (int w = 16; w >= 1; --w) {
+    const size_t lds = tile_kernel_lds_bytes(args.prob_bits, CODED, w);
+    if (lds > kLdsLimitBytes) continue;
+    int blocks_per_cu = static_cast<int>(kLdsLimitBytes / lds);
+    if (blocks_per_cu > 2) blocks_per_cu = 2;
+    if (blocks_per_cu * w > waves_per_cu) blocks_per_cu = waves_per_cu / w;
+    if (blocks_per_cu < 1) continue;
+    const int64_t slots = static_cast<int64_t>(blocks_per_cu) * w * compute_units;
+    const int64_t cost = (pairs + slots - 1) / slots * blocks_per_cu * w;
+    if (cost < best) {
+      best = cost;
       waves = w;
+      resident = blocks_per_cu;
     }
   }
+  if (waves == 0) return hipErrorInvalidConfiguration;
   const int64_t wanted = (pairs + waves - 1) / waves;
-  const unsigned blocks = static_cast<unsigned>(wanted < resident ? wanted : resident);
-  const size_t lds = (size_t{4} << args.prob_bits) + static_cast<size_t>(waves) * 2 * (kRingBytes + 256) + 16;
-  hipLaunchKernelGGL(tile_ans_tile_kernel<BYTES>, dim3(blocks), dim3(waves * 64), lds, stream, args, static_cast<int>(pairs));
+  const int64_t most = static_cast<int64_t>(resident) * compute_units;
+  const unsigned blocks = static_cast<unsigned>(wanted < most ? wanted : most);
+  const size_t lds = tile_kernel_lds_bytes(args.prob_bits, CODED, waves);
+  int device = 0;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return status;
+  if (configured_for != device) {
+    status = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_ans_tile_kernel<BYTES, CODED>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 static_cast<int>(kLdsLimitBytes));
+    if (status != hipSuccess) return status;
+    configured_for = device;
+  }
+  hipLaunchKernelGGL((tile_ans_tile_kernel<BYTES, CODED>), dim3(blocks), dim3(waves * 64), lds, stream, args, static_cast<int>(pairs));
   return hipGetLastError();
+}
+
+// Containers the tile kernel is built for: up to four coded lanes (more: registers and LDS run out; the general
+// kernel takes those).
+constexpr int kMaxTileCodedLanes = 4;
+
+template <int BYTES>
+static hipError_t launch_tile_kernel_for(int coded, const TileAnsArgs& args, int compute_units, hipStream_t stream) {
+  switch (coded) {
+    case 0: return launch_tile_kernel<BYTES, 0>(args, compute_units, stream);
+    case 1: return launch_tile_kernel<BYTES, 1>(args, compute_units, stream);
+    case 2: if constexpr (BYTES >= 2) return launch_tile_kernel<BYTES, 2>(args, compute_units, stream); break;
+    case 3: if constexpr (BYTES >= 4) return launch_tile_kernel<BYTES, 3>(args, compute_units, stream); break;
+    case 4: if constexpr (BYTES >= 4) return launch_tile_kernel<BYTES, 4>(args, compute_units, stream); break;
+    default: break;
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace ep
@@ -387,7 +483,6 @@ extern "C" int ep_hip_decode_tile_ans(const uint16_t* payload_dev, uint64_t payl
   args.tiles = (num_elements + tile_elements - 1) / tile_elements;
   args.prob_bits = prob_bits;
   args.lanes = num_lanes;
-  args.coded_lane = -1;
   args.wide_stores = reinterpret_cast<uintptr_t>(out_dev) % 16 == 0;
   args.error = error_dev;
   int coded = 0;
@@ -397,25 +492,22 @@ extern "C" int ep_hip_decode_tile_ans(const uint16_t* payload_dev, uint64_t payl
     if (b < num_lanes) {
       if (lane_modes_host[b] > 1) return EP_HIP_EINVAL;
       args.raw[b] = lane_modes_host[b];
-      if (!args.raw[b]) {
-        args.coded_lane = b;
-        ++coded;
-      }
+      if (!args.raw[b]) ++coded;
     }
   }
   if (coded > 0 && states_dev == nullptr) return EP_HIP_EINVAL;
   const int64_t streams = args.tiles * num_lanes;
   if (streams >= (int64_t{1} << 31)) return EP_HIP_EUNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (coded == 1 && args.tile_elements < (int64_t{1} << 28) && payload_words < (uint64_t{1} << 31)) {
+  if (coded <= kMaxTileCodedLanes && args.tile_elements < (int64_t{1} << 28) && payload_words < (uint64_t{1} << 31)) {
     int device = 0, compute_units = 0;
     EP_HIP_TRY(hipGetDevice(&device));
     EP_HIP_TRY(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
     switch (num_lanes) {
-      case 1: EP_HIP_TRY(launch_tile_kernel<1>(args, compute_units, s)); break;
-      case 2: EP_HIP_TRY(launch_tile_kernel<2>(args, compute_units, s)); break;
-      case 4: EP_HIP_TRY(launch_tile_kernel<4>(args, compute_units, s)); break;
-      default: EP_HIP_TRY(launch_tile_kernel<8>(args, compute_units, s)); break;
+      case 1: EP_HIP_TRY(launch_tile_kernel_for<1>(coded, args, compute_units, s)); break;
+      case 2: EP_HIP_TRY(launch_tile_kernel_for<2>(coded, args, compute_units, s)); break;
+      case 4: EP_HIP_TRY(launch_tile_kernel_for<4>(coded, args, compute_units, s)); break;
+      default: EP_HIP_TRY(launch_tile_kernel_for<8>(coded, args, compute_units, s)); break;
     }
     return EP_HIP_OK;
   }

@@ -133,8 +133,8 @@ def fused_linear_usable(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool
 def fused_linear_pays(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
     """Usable, and measured faster than decoding and multiplying separately.
 
-    With rank/select tables the four-row kernel needs more registers than two resident blocks per CU allow and loses
-    to decode + the split-K product; one row still wins there.
+    One row always pays. With rank/select tables the four-row kernel needs more registers than two resident blocks
+    per CU allow and loses to decode + the split-K product.
     """
     if not fused_linear_usable(buffers, shape, x):
         return False
@@ -144,7 +144,17 @@ def fused_linear_pays(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
     if plan.desc.table_kind == _hip.TABLE_GLOBAL64:
         return False
     rows = x.numel() // x.shape[-1]
-    return rows == 1 or plan.desc.table_kind != _hip.TABLE_LDS_RANK
+    if rows == 1:
+        return True
+    if plan.desc.table_kind == _hip.TABLE_LDS_RANK:
+        return False
+    # Two to four rows: the four-row kernel costs a third more than a plain decode. A weight small enough that its
+    # decode lasts as long as one tile's chain anyway (at most 16 tile pairs per CU) hides that; a large one is decoded
+    # at full rate and multiplied by the split-K product faster (8192 x 28672 @ 4 bpp: 239 us against 270 us).
+    device = buffers.payload.device
+    caps = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device())
+    pairs = (int(buffers.states.shape[0]) + 1) // 2
+    return pairs <= 16 * caps.compute_units
 
 
 def linear_rows(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:

@@ -190,3 +190,27 @@ def test_compressed_linear_with_lossless_weights(mode):
         got = fresh(x)
         error = ((got.float() - expect).norm() / expect.norm()).item()
         assert got.dtype == torch.bfloat16 and error <= 4e-3, (rows, error)            # one bf16 rounding of the output
+
+
+@pytest.mark.parametrize("probability_bits", [0, 9, 12])
+def test_several_coded_lanes_and_none(probability_bits):
+    """Containers with two, three and four coded lanes (the tile kernel carries one rANS state per coded lane and half),
+    with none (every lane raw: a byte-plane interleave), and with more than four (general kernel); whole 256-element
+    chunks, other tile sizes and short last tiles. At 12 bits a constant lane has frequency 4096 (stream-by-stream path)."""
+    print("case", probability_bits, flush=True)
+    torch.manual_seed(21 + probability_bits)
+    shape = (97, 1031)
+    small16 = torch.randint(-300, 300, shape, dtype=torch.int16)                       # both bytes structured
+    small32 = torch.randint(-40000, 40000, shape, dtype=torch.int32)                   # two structured bytes + two near-constant
+    tiny32 = torch.randint(0, 200, shape, dtype=torch.int32)                           # one structured + three constant
+    mixed32 = (torch.randint(0, 256, shape, dtype=torch.int32) << 8) | torch.randint(0, 7, shape, dtype=torch.int32)   # raw in the middle
+    ids64 = torch.randint(0, 50000, shape, dtype=torch.int64)                          # six constant bytes: more than four coded lanes
+    noise = torch.randint(-128, 128, shape, dtype=torch.int8)
+    seen = set()
+    for tensor in (small16, small32, tiny32, mixed32, ids64, noise):
+        for tile_elements in (256, 1000, 4096):
+            container = round_trip(tensor, tile_elements=tile_elements, probability_bits=probability_bits)
+            modes = container.buffers["lane_modes"].tolist()
+            seen.add((len(modes), modes.count(0)))
+    counts = {coded for _, coded in seen}
+    assert 0 in counts and counts & {2, 3, 4} and max(counts) > 4, seen          # all raw, the multi-lane tile kernel, the general kernel
