@@ -114,7 +114,7 @@ def _median_ms(fn, steps, warmup=5):
 
 
 def linear_section(ep, steps):
-    """BASELINE config 3: W 3072x3072 @ 4 bpp + bias, X [4096, 3072] bf16, seed 2; whole forward (decode + GEMM)."""
+    """Benchmark configuration 3: W 3072x3072 @ 4 bpp + bias, X [4096, 3072] bf16, seed 2; whole forward (decode + GEMM)."""
     from torch.nn import functional as F
     torch.manual_seed(2)
     dense = torch.nn.Linear(3072, 3072, dtype=torch.bfloat16)
@@ -187,7 +187,7 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
 
 
 def small_m_section(ep, on_gpu, rows, cols, bpp, steps):
-    """BASELINE config 5, linear part: X [M, cols] bf16 N(0, 1), M in {1, 16, 128}, on the container just decoded.
+    """Benchmark configuration 5, linear part: X [M, cols] bf16 N(0, 1), M in {1, 16, 128}, on the container just decoded.
 
     The weight stream bounds this regime, so each mode is priced in GB/s on the bytes it has to move: fused = the
     compressed container + x + y; decode_then_gemm adds one write and one read of the dense weight.
@@ -226,7 +226,7 @@ STACK_RATES = (2.3, 4.0, 5.0, 6.0, 8.0)
 
 
 def stack_workload(args, ep):
-    """BASELINE config 4: `--stack-blocks` blocks x 4 layers, N(0, 0.02) seed 3, rates round-robin; one pass decodes all."""
+    """Benchmark configuration 4: `--stack-blocks` blocks x 4 layers, N(0, 0.02) seed 3, rates round-robin; one pass decodes all."""
     from entropack_amd.schemes.lattice_rans import hip as hip_lane
     from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
     device = torch.device("cuda", 0)

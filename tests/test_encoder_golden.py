@@ -24,7 +24,7 @@ def test_compress_reproduces_the_reference_container(golden):
 
 
 def test_config_1_rate_and_error_window():
-    """BASELINE config 1: 256x256 bf16 N(0, 0.02), seed 0, 3.5 bpp -> actual_bpp in [3.5, 3.6], rel-L2 near the
+    """Benchmark configuration 1: 256x256 bf16 N(0, 0.02), seed 0, 3.5 bpp -> actual_bpp in [3.5, 3.6], rel-L2 near the
     E8 high-rate closed form 1.1065 * 2**-R for the payload rate R (container overhead excluded)."""
     golden = Golden("c1_256x256_bf16_3p5")
     torch.manual_seed(0)

@@ -73,7 +73,7 @@ ALL_KINDS = (None, hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_b
 
 
 def test_config_2_outliers_4096x4096():
-    """BASELINE config 2: 4096x4096, 0.1 % of entries x20, seed 1, 4.0 bpp; bit-exact against the oracle."""
+    """Benchmark configuration 2: 4096x4096, 0.1 % of entries x20, seed 1, 4.0 bpp; bit-exact against the oracle."""
     container, used = decode_and_check(gauss(1, 4096, 4096, outliers=True), kinds=ALL_KINDS, target_bpp=4.0)
     assert "lds_wide" in used and "global64" in used        # the outliers push the alphabets past a byte
     assert 4.0 < container.actual_bpp < 4.25
@@ -81,7 +81,7 @@ def test_config_2_outliers_4096x4096():
 
 @pytest.mark.parametrize("bpp", [2.3, 4.0, 5.0, 6.0, 8.0])
 def test_dit_like_layer_at_each_rate(bpp):
-    """BASELINE config 4, one representative of each rate on the out-projection shape (3840 x 3840), seed 3."""
+    """Benchmark configuration 4, one representative of each rate on the out-projection shape (3840 x 3840), seed 3."""
     print("case bpp", bpp, flush=True)
     container, used = decode_and_check(gauss(3, 3840, 3840), kinds=(None, hip_backend.TABLE_GLOBAL64), target_bpp=bpp)
     assert abs(container.actual_bpp - bpp) < 0.12
@@ -125,7 +125,7 @@ def test_int8_code_container_decodes_to_int8():
 
 
 def test_full_size_target_8192x28672():
-    """The headline shape at 2.0, 4.0 and 8.0 bpp (BASELINE config 5 + the 4 bpp target): bit-exact against the oracle,
+    """The headline shape at 2.0, 4.0 and 8.0 bpp (Benchmark configuration 5 + the 4 bpp target): bit-exact against the oracle,
     decode is idempotent, and no tile reports an error."""
     weight = gauss(4, 8192, 28672, sigma=0.015)
     for bpp in (4.0, 2.0, 8.0):

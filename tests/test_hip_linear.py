@@ -10,7 +10,7 @@ import entropack_amd as ep
 from entropack_amd.linear import kernels
 
 pytestmark = pytest.mark.gpu
-REL_L2 = 1e-3          # tolerance BASELINE states for linear outputs (bf16 accumulate-order differences)
+REL_L2 = 1e-3          # tolerance stated for linear outputs (bf16 accumulate-order differences)
 
 
 def rel_l2(got, expect):
@@ -125,7 +125,7 @@ def _c3_layer(mode, rows=3072, cols=3072, cls=None, bpp=4.0):
 
 @pytest.mark.parametrize("mode", ["decode_then_gemm", "fused"])
 def test_compressed_linear_forward_config_3(mode):
-    """BASELINE config 3: W 3072x3072 @ 4 bpp, bias, X [4096, 3072]; output rel-L2 vs F.linear(x, W_dec, b) <= 1e-3."""
+    """Benchmark configuration 3: W 3072x3072 @ 4 bpp, bias, X [4096, 3072]; output rel-L2 vs F.linear(x, W_dec, b) <= 1e-3."""
     layer, weight, bias = _c3_layer(mode)
     torch.manual_seed(2)
     x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
