@@ -139,6 +139,38 @@ def linear_section(ep, steps):
     return out
 
 
+MFMA_PEAK_INT8_TOPS = 5000.0
+
+
+def int8_linear_section(ep, steps):
+    """Configuration 3's layer as W8A8 (`CompressedINT8Linear`, int8 codes lattice-coded at 4 bpp, per-row activation
+    quantiser, int8 matrix cores): whole forward in both modes, against the layer's own definition in float64."""
+    from entropack_amd.linear import kernels
+    torch.manual_seed(2)
+    dense = torch.nn.Linear(3072, 3072, dtype=torch.bfloat16)
+    dense.weight.data.copy_((torch.randn(3072, 3072) * 0.02).to(torch.bfloat16))
+    dense.bias.data.copy_((torch.randn(3072) * 0.01).to(torch.bfloat16))
+    x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
+    ops = 2.0 * 4096 * 3072 * 3072
+    out = {"workload": "CompressedINT8Linear 3072x3072, codes @ 4.0 bpp, + bias, X [4096, 3072] bf16, seed 2", "ops": ops}
+    for mode in ("decode_then_gemm", "fused"):
+        layer = ep.CompressedINT8Linear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
+        y = layer(x)
+        codes, (qa, sa) = layer.codes("cuda"), kernels.quantize_rows(x)
+        definition = ((qa.double() @ codes.double().T) * sa.double().unsqueeze(1) * layer.weight_quant_scale.cuda().double().unsqueeze(0)
+                      + dense.bias.data.cuda().double())
+        rounded = definition.float().to(torch.bfloat16).double()                  # the layer rounds its float32 result once
+        rel = ((y.double() - rounded).norm() / rounded.norm()).item()
+        dense_rel = ((y.double() - torch.nn.functional.linear(x.double(), dense.weight.data.cuda().double(), dense.bias.data.cuda().double())).norm()
+                     / definition.norm()).item()
+        ms = _median_ms(lambda: layer(x), steps)
+        out[mode] = {"ms": round(ms, 5), "tops": round(ops / ms / 1e9, 2), "frac_of_int8_mfma_peak": round(ops / ms / 1e9 / MFMA_PEAK_INT8_TOPS, 5),
+                     "rel_l2_vs_definition_in_bf16": rel, "rel_l2_vs_dense_layer": dense_rel}
+    out["quantize_rows_ms"] = round(_median_ms(lambda: kernels.quantize_rows(x), steps), 5)
+    out["int8_gemm_ms"] = round(_median_ms(lambda: kernels.int8_gemm(qa, codes, sa, layer.weight_quant_scale.cuda(), None, torch.bfloat16), steps), 5)
+    return out
+
+
 def stack_linear_section(ep, steps, layers_total=48, distinct=4):
     """Config 3's layer repeated as a stack (M = 4096, 3072 x 3072 @ 4 bpp + bias): a model's forward, where the weights of
     `group` layers are decoded per pass on a second stream while the previous group multiplies (DecodeAhead). Per-layer
@@ -487,6 +519,7 @@ def main():
     if not args.no_linear:
         result["linear"] = linear_section(ep, args.steps)
         result["linear_stack"] = stack_linear_section(ep, args.steps)
+        result["linear_int8"] = int8_linear_section(ep, args.steps)
         if rows * cols >= 1 << 27:
             result["linear_small_m"] = small_m_section(ep, on_gpu, rows, cols, bpp, args.steps)
 
