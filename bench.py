@@ -136,6 +136,15 @@ def linear_section(ep, steps):
         ms = _median_ms(lambda: layer(x), steps)
         out[mode] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2),
                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5), "rel_l2_vs_f32_reference": rel}
+    # The same layer with its weight stored losslessly (tile_ans, the scheme a layer takes when given no config).
+    layer = ep.CompressedLinear.from_linear(dense).cuda()
+    y = layer(x)
+    exact = F.linear(x.float(), dense.weight.data.cuda().float(), dense.bias.data.cuda().float()).to(torch.bfloat16).double()
+    ms = _median_ms(lambda: layer(x), steps)
+    out["lossless_decode_then_gemm"] = {
+        "ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2), "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5),
+        "decode_ms": round(_median_ms(lambda: layer.dequantize("cuda"), steps), 5), "stored_bits_per_weight": round(layer.compressed_bits, 3),
+        "rel_l2_vs_dense_layer": ((y.double() - exact).norm() / exact.norm()).item()}
     return out
 
 
