@@ -53,16 +53,19 @@ struct Layout {
 struct Pair {
   uint32_t x;            // rANS state
   uint32_t prefetch;     // the 64 payload words below the ring, 2 per lane
-  int32_t fetch_dword;   // absolute dword index `prefetch` came from
+  uint32_t fetch_at;     // byte offset from `origin` of the dword `prefetch` came from
+  const uint8_t* origin; // wave-uniform: a 64-word boundary of the payload at or below every word the pair still needs
   uint32_t ring;         // LDS byte address of this half's 128-word window
   uint32_t ring_lane;    // ring + 4 * (lane & 31): where this lane's dword of a 64-word chunk goes
   uint32_t vector0;      // first vector of this lane's tile
   int count;             // vectors in this lane's tile (0 = no tile)
   uint32_t pos;          // (pA + 64) | (pB + 64) << 16: read positions inside the windows, biased by kPosBias so that the
                          // scalar arithmetic of a step never borrows across the fields while pA, pB fall to 0
-  int windowA, windowB;  // window starts, relative to a 64-aligned base below each tile (may go negative)
+  int windowA, windowB;  // where the windows started, relative to a 64-aligned base below each tile's first word
+  uint64_t slid;         // slides so far: the lower half's count from bit 7 (16 bits), the upper half's from bit 23
   int beginA, beginB;    // position of each tile's first word, relative to that base
   uint32_t coset_base;   // LDS byte offset of this lane's coset inside a field's table pair (0 or one table)
+  uint64_t coset_mask;   // wave-uniform: the lanes whose current vector lies in coset 1
   uint32_t e[8];         // slot-table entries of the eight fields of the current vector
   int dot_row;           // multiply-on-the-fly only: the weight row `dot_acc` belongs to (same in all lanes of a half), -1 = none
   float dot_acc[kDotRows];
@@ -89,21 +92,24 @@ struct Pair {
   "v_bfe_u32 %[d" S "], %[e" S "], %[dshift], %[dwidth]\n"       \
   "v_mad_u32_u24 %[x" S "], %[t" S "], %[h" S "], %[d" S "]\n"
 
-// Vote, per-half counts, new positions, window address, issue the window read. Leaves the vote in vcc.
-// pos stays >= 32 in both halves, so neither subtraction borrows across the 16-bit fields.
+// Vote, per-half counts, window address, issue the window read, new positions. Leaves the vote in vcc.
+// With n_a, n_b the halves' counts: lane l of the lower half reads at p_a - n_a + rank(l), and a lane of the upper
+// half, whose rank as the two mbcnt instructions count it includes n_a, at p_b - (n_a + n_b) + rank(l). Both bases
+// come from one subtraction of (n_a | (n_a + n_b) << 16); the positions themselves (p - n per half) follow after
+// the read is issued. pos stays >= 32 in both halves, so no subtraction borrows across the 16-bit fields.
 #define EP_ASM_VOTE(S)                                          \
   "v_cmp_gt_u32 vcc, 0x8000, %[x" S "]\n"                        \
   "s_bcnt1_i32_b32 %[na], vcc_lo\n"                              \
-  "s_bcnt1_i32_b32 %[nb], vcc_hi\n"                              \
+  "s_bcnt1_i32_b64 %[nb], vcc\n"                                 \
   "s_pack_ll_b32_b16 %[nb], %[na], %[nb]\n"                      \
-  "s_sub_u32 %[pos" S "], %[pos" S "], %[nb]\n"                  \
-  "s_lshl_b32 %[na], %[na], 16\n"                                \
-  "s_sub_u32 %[na], %[pos" S "], %[na]\n"                        \
-  "v_bfe_u32 %[t" S "], %[na], %[shv], 16\n"                     \
+  "s_sub_u32 %[nb], %[pos" S "], %[nb]\n"                        \
+  "v_bfe_u32 %[t" S "], %[nb], %[shv], 16\n"                     \
   "v_mbcnt_lo_u32_b32 %[t" S "], vcc_lo, %[t" S "]\n"            \
   "v_mbcnt_hi_u32_b32 %[t" S "], vcc_hi, %[t" S "]\n"            \
   "v_lshl_add_u32 %[t" S "], %[t" S "], 1, %[ring" S "]\n"       \
-  "ds_read_u16 %[d" S "], %[t" S "]\n"
+  "ds_read_u16 %[d" S "], %[t" S "]\n"                           \
+  "s_lshl_b32 %[na], %[na], 16\n"                                \
+  "s_add_u32 %[pos" S "], %[nb], %[na]\n"
 
 // x = voted ? x << 16 | word : x
 #define EP_ASM_TAKE_VCC(S)                                      \
@@ -118,11 +124,13 @@ struct Pair {
 #define EP_ASM_TAKE_EXEC_SAVED(S) "s_mov_b64 exec, %[m0]\n v_lshl_or_b32 %[x" S "], %[x" S "], 16, %[d" S "]\n"
 #define EP_ASM_RESTORE_FULL "s_mov_b64 exec, -1\n"
 
-// Coset symbol in closed form: c = slot >= f0; freq = c ? T - f0 : f0; begin = c ? f0 : 0.
+// Coset symbol in closed form: c = slot >= f0; freq = c ? T - f0 : f0; begin = c ? f0 : 0. The lanes with c = 1
+// are also left as a mask in scalar registers (cm), for selections that would otherwise compare cb with 0 again.
 #define EP_ASM_COSET(S)                                         \
   "v_and_b32 %[t" S "], %[slotmask], %[x" S "]\n"                \
   "v_lshrrev_b32 %[h" S "], %[pb], %[x" S "]\n"                  \
   "v_cmp_le_u32 vcc, %[f0s], %[t" S "]\n"                        \
+  "s_mov_b64 %[cm" S "], vcc\n"                                  \
   "v_cndmask_b32 %[cb" S "], 0, %[f0v], vcc\n"                   \
   "v_sub_u32 %[t" S "], %[t" S "], %[cb" S "]\n"                 \
   "v_cndmask_b32 %[d" S "], %[f0v], %[f1v], vcc\n"               \
@@ -154,7 +162,7 @@ __device__ __forceinline__ void field_step_single(Pair& p, int field, uint32_t o
   using L = Layout<PB, MODE>;
   uint32_t t, h, d, e, na, nb;
   uint64_t sv;
-  const uint32_t kslot = L::kSlotMask4, kring = 0xFEu;
+  const uint32_t kslot = L::kSlotMask4;
   uint32_t pos = uniform(p.pos);
   valid = uniform(valid);
 #define EP_FIELD_SINGLE_BODY                                                                           \
@@ -166,7 +174,7 @@ __device__ __forceinline__ void field_step_single(Pair& p, int field, uint32_t o
 #define EP_FIELD_SINGLE_OPERANDS(OFF)                                                                           \
   : [x0] "+v"(p.x), [pos0] "+s"(pos), [e0] "=&v"(e), [t0] "=&v"(t), [h0] "=&v"(h), [d0] "=&v"(d), [na] "=&s"(na),   \
     [nb] "=&s"(nb), [sv] "=&s"(sv)                                                                               \
-  : [cb0] "v"(cb), [ring0] "v"(p.ring), [shv] "v"(k.shv), [kslot] "s"(kslot), [kring] "s"(kring), [valid] "s"(valid), \
+  : [cb0] "v"(cb), [ring0] "v"(p.ring), [shv] "v"(k.shv), [kslot] "s"(kslot), [valid] "s"(valid), \
     [off] "n"(OFF), [pb] "n"(PB), [fmask] "n"(L::kFreqMask), [dshift] "n"(L::kDeltaShift), [dwidth] "n"(L::kDeltaWidth)                           \
   : "vcc", "scc", "memory"
   // The LDS offset must be an immediate, so the four field positions inside a group are spelled out.
@@ -189,7 +197,7 @@ __device__ __forceinline__ void field_step_dual(Pair& p0, Pair& p1, int field, u
   using L = Layout<PB, MODE>;
   uint32_t t0, h0, d0, e0, t1, h1, d1, e1, na, nb;
   uint64_t sv, m0;
-  const uint32_t kslot = L::kSlotMask4, kring = 0xFEu;
+  const uint32_t kslot = L::kSlotMask4;
   uint32_t pos0 = uniform(p0.pos), pos1 = uniform(p1.pos);
   valid = uniform(valid);
   // Issue order: both gathers, pair 0 advances and issues its ring read while pair 1's gather lands, and so on;
@@ -208,7 +216,7 @@ __device__ __forceinline__ void field_step_dual(Pair& p0, Pair& p1, int field, u
     [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(h0), [h1] "=&v"(h1), [d0] "=&v"(d0), [d1] "=&v"(d1), [na] "=&s"(na), \
     [nb] "=&s"(nb), [sv] "=&s"(sv), [m0] "=&s"(m0)                                                               \
   : [cb0] "v"(cb0), [cb1] "v"(cb1), [ring0] "v"(p0.ring), [ring1] "v"(p1.ring), [shv] "v"(k.shv),                \
-    [kslot] "s"(kslot), [kring] "s"(kring), [valid] "s"(valid), [off] "n"(OFF), [pb] "n"(PB),                    \
+    [kslot] "s"(kslot), [valid] "s"(valid), [off] "n"(OFF), [pb] "n"(PB),                    \
     [fmask] "n"(L::kFreqMask), [dshift] "n"(L::kDeltaShift), [dwidth] "n"(L::kDeltaWidth)                                                      \
   : "vcc", "scc", "memory"
 #define EP_FIELD_DUAL_CASE(OFF)                                                                            \
@@ -230,8 +238,8 @@ template <int PB, int MODE, bool MASKED>
 __device__ __forceinline__ void coset_step_single(Pair& p, const StepConsts& k, uint64_t valid) {
   using L = Layout<PB, MODE>;
   uint32_t t, h, d, cb, na, nb;
-  uint64_t sv;
-  const uint32_t kring = 0xFEu, f0s = k.f0s;
+  uint64_t sv, cm;
+  const uint32_t f0s = k.f0s;
   uint32_t pos = uniform(p.pos);
   valid = uniform(valid);
 #define EP_COSET_SINGLE_BODY EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_VCC("0")
@@ -239,13 +247,14 @@ __device__ __forceinline__ void coset_step_single(Pair& p, const StepConsts& k, 
   EP_ASM_COSET("0") EP_ASM_VOTE("0") "s_waitcnt lgkmcnt(0)\n" EP_ASM_TAKE_EXEC_VCC("0") EP_ASM_RESTORE_FULL
 #define EP_COSET_SINGLE_OPERANDS                                                                                \
   : [x0] "+v"(p.x), [pos0] "+s"(pos), [cb0] "=&v"(cb), [t0] "=&v"(t), [h0] "=&v"(h), [d0] "=&v"(d), [na] "=&s"(na),  \
-    [nb] "=&s"(nb), [sv] "=&s"(sv)                                                                               \
+    [nb] "=&s"(nb), [sv] "=&s"(sv), [cm0] "=&s"(cm)                                                              \
   : [ring0] "v"(p.ring), [shv] "v"(k.shv), [f0v] "v"(k.f0v), [f1v] "v"(k.f1v), [ktab] "v"(k.ktab), [f0s] "s"(f0s),  \
-    [kring] "s"(kring), [valid] "s"(valid), [pb] "n"(PB), [slotmask] "n"(L::kTable - 1)                          \
+    [valid] "s"(valid), [pb] "n"(PB), [slotmask] "n"(L::kTable - 1)                          \
   : "vcc", "scc", "memory"
   if constexpr (MASKED) asm volatile(EP_ASM_MASK_ON EP_COSET_SINGLE_BODY EP_ASM_MASK_OFF EP_COSET_SINGLE_OPERANDS);
   else asm volatile(EP_COSET_SINGLE_FAST EP_COSET_SINGLE_OPERANDS);
   p.coset_base = cb;
+  p.coset_mask = cm;
   p.pos = pos;
 }
 
@@ -253,8 +262,8 @@ template <int PB, int MODE, bool MASKED>
 __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepConsts& k, uint64_t valid) {
   using L = Layout<PB, MODE>;
   uint32_t t0, h0, d0, cb0, t1, h1, d1, cb1, na, nb;
-  uint64_t sv, m0;
-  const uint32_t kring = 0xFEu, f0s = k.f0s;
+  uint64_t sv, m0, cm0, cm1;
+  const uint32_t f0s = k.f0s;
   uint32_t pos0 = uniform(p0.pos), pos1 = uniform(p1.pos);
   valid = uniform(valid);
 #define EP_COSET_DUAL_BODY                                                                              \
@@ -267,15 +276,17 @@ __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepCo
 #define EP_COSET_DUAL_OPERANDS                                                                                    \
   : [x0] "+v"(p0.x), [x1] "+v"(p1.x), [pos0] "+s"(pos0), [pos1] "+s"(pos1), [cb0] "=&v"(cb0), [cb1] "=&v"(cb1),     \
     [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(h0), [h1] "=&v"(h1), [d0] "=&v"(d0), [d1] "=&v"(d1), [na] "=&s"(na),   \
-    [nb] "=&s"(nb), [sv] "=&s"(sv), [m0] "=&s"(m0)                                                                 \
+    [nb] "=&s"(nb), [sv] "=&s"(sv), [m0] "=&s"(m0), [cm0] "=&s"(cm0), [cm1] "=&s"(cm1)                             \
   : [ring0] "v"(p0.ring), [ring1] "v"(p1.ring), [shv] "v"(k.shv), [f0v] "v"(k.f0v), [f1v] "v"(k.f1v),              \
-    [ktab] "v"(k.ktab), [f0s] "s"(f0s), [kring] "s"(kring), [valid] "s"(valid), [pb] "n"(PB),                      \
+    [ktab] "v"(k.ktab), [f0s] "s"(f0s), [valid] "s"(valid), [pb] "n"(PB),                      \
     [slotmask] "n"(L::kTable - 1)                                                                                  \
   : "vcc", "scc", "memory"
   if constexpr (MASKED) asm volatile(EP_ASM_MASK_ON EP_COSET_DUAL_BODY EP_ASM_MASK_OFF EP_COSET_DUAL_OPERANDS);
   else asm volatile(EP_COSET_DUAL_FAST EP_COSET_DUAL_OPERANDS);
   p0.coset_base = cb0;
   p1.coset_base = cb1;
+  p0.coset_mask = cm0;
+  p1.coset_mask = cm1;
   p0.pos = pos0;
   p1.pos = pos1;
 }
@@ -364,11 +375,18 @@ __device__ __forceinline__ void lds_store32(uint32_t at, uint32_t value) {
 }
 
 // Opens the window of each half's stream, words [word_begin, word_end) of `payload` (per-half values; lanes of a
-// half agree): fills the 128 LDS words at `window_at` with the stream's last one or two 64-word chunks, requests the
-// 64 words below them, and sets the biased positions and the bookkeeping the end-of-stream check needs.
-__device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_t word_begin, uint32_t word_end,
-                                            const uint16_t* __restrict__ payload, uint64_t payload_words, int l32) {
-  const uint32_t* payload32 = reinterpret_cast<const uint32_t*>(payload);
+// half agree; `live` = the half has a stream): fills the 128 LDS words at `window_at` with the stream's last one or
+// two 64-word chunks, requests the 64 words below them, and sets the biased positions and the bookkeeping the
+// end-of-stream check needs.
+//
+// Prefetches address the payload as one wave-uniform origin plus a 32-bit byte offset per lane, the form that
+// costs no address arithmetic. The origin lies three chunks below the lower live stream's first chunk (or at the
+// payload's start): lower than anything a valid stream consumes. Offsets saturate at the origin, so requests that
+// reach further down (the last ones of a stream always do) re-read the origin chunk, and those words are never used.
+// `readable` points at four readable bytes that stand in for a payload of fewer than two words.
+__device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_t word_begin, uint32_t word_end, bool live,
+                                            const uint16_t* __restrict__ payload, uint64_t payload_words, const void* readable,
+                                            int l32) {
   s.ring = window_at - 2u * kPosBias;                   // positions are kept biased, see Pair::pos
   const uint32_t base = word_begin & ~63u;               // absolute index of relative position 0
   const int begin = static_cast<int>(word_begin - base);
@@ -383,10 +401,17 @@ __device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_
     if (at + 1 >= 0 && static_cast<uint64_t>(at + 1) < payload_words) hi = payload[at + 1];
     lds_store32(s.ring_lane + 128u * c, lo | (hi << 16));
   }
-  s.fetch_dword = static_cast<int32_t>((static_cast<int64_t>(base) + low - 64) >> 1) + l32;
-  s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
+  const uint32_t floor_of = live ? (base >= 192u ? base - 192u : 0u) : ~0u;
+  const uint32_t floor_a = __builtin_amdgcn_readlane(floor_of, 0), floor_b = __builtin_amdgcn_readlane(floor_of, 32);
+  const uint32_t lowest = floor_a < floor_b ? floor_a : floor_b;
+  const uint32_t origin_word = lowest == ~0u ? 0u : lowest;
+  s.origin = payload_words >= 2 ? reinterpret_cast<const uint8_t*>(payload) + 2ull * origin_word : static_cast<const uint8_t*>(readable);
+  const int64_t wanted = 2 * (static_cast<int64_t>(base) + low - 64 - static_cast<int64_t>(origin_word)) + 4 * l32;
+  s.fetch_at = live && wanted > 0 ? static_cast<uint32_t>(wanted) : 0u;
+  s.prefetch = *reinterpret_cast<const uint32_t*>(s.origin + s.fetch_at);
   const int p = ptr - low + static_cast<int>(kPosBias);  // position in [64, 128), stored biased
   s.pos = static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 0)) | (static_cast<uint32_t>(__builtin_amdgcn_readlane(p, 32)) << 16);
+  s.slid = 0;
   s.windowA = __builtin_amdgcn_readlane(low, 0);
   s.windowB = __builtin_amdgcn_readlane(low, 32);
   s.beginA = __builtin_amdgcn_readlane(begin, 0);
@@ -395,27 +420,33 @@ __device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_
 
 // After a step (or two): a half whose position fell below 64 slides its window down by 64 words. All 32 lanes of the
 // half (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
-// the next 64 words down.
-__device__ __forceinline__ void slide_window(Pair& s, int half, const uint32_t* __restrict__ payload32) {
+// the next 64 words down. Which halves slide is a scalar decision, and the lanes are picked by a mask built from it;
+// the scalar side is kept short (it is what the common, non-sliding case pays for: three instructions).
+__device__ __forceinline__ void slide_window(Pair& s) {
   const uint32_t low_bits = ~s.pos & 0x00800080u;        // bit 7 of a biased field clear <=> that position < 64
   if (__builtin_expect(low_bits != 0, 0)) {
     asm volatile("" ::: "memory");     // keep this a scalar branch: the common case must cost no vector work
-    if ((low_bits >> (half ? 23 : 7)) & 1u) {
+    const uint32_t lower = static_cast<uint32_t>(static_cast<int32_t>(low_bits << 24) >> 31);
+    const uint32_t upper = static_cast<uint32_t>(static_cast<int32_t>(low_bits << 8) >> 31);
+    if (__builtin_amdgcn_inverse_ballot_w64(static_cast<uint64_t>(lower) | (static_cast<uint64_t>(upper) << 32))) {
       const uint32_t kept = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(s.ring_lane));
       lds_store32(s.ring_lane + 128u, kept);
       lds_store32(s.ring_lane, s.prefetch);
-      s.fetch_dword -= 32;
-      s.prefetch = s.fetch_dword >= 0 ? payload32[s.fetch_dword] : 0u;
+      s.fetch_at = s.fetch_at >= 128u ? s.fetch_at - 128u : 0u;
+      s.prefetch = *reinterpret_cast<const uint32_t*>(s.origin + s.fetch_at);
     }
     s.pos += low_bits >> 1;             // + 64 in the fields that slid
-    s.windowA -= static_cast<int>((low_bits >> 1) & 0x40u);
-    s.windowB -= static_cast<int>((low_bits >> 17) & 0x40u);
+    s.slid += low_bits;                 // one more slide for them
   }
 }
 
 // Where each half's stream stands, relative to the same base as Pair::beginA / beginB.
-__device__ __forceinline__ int window_pointer_a(const Pair& s) { return s.windowA + static_cast<int>(s.pos & 0xFFFFu) - static_cast<int>(kPosBias); }
-__device__ __forceinline__ int window_pointer_b(const Pair& s) { return s.windowB + static_cast<int>(s.pos >> 16) - static_cast<int>(kPosBias); }
+__device__ __forceinline__ int window_pointer_a(const Pair& s) {
+  return s.windowA - 64 * static_cast<int>((s.slid >> 7) & 0xFFFFu) + static_cast<int>(s.pos & 0xFFFFu) - static_cast<int>(kPosBias);
+}
+__device__ __forceinline__ int window_pointer_b(const Pair& s) {
+  return s.windowB - 64 * static_cast<int>(s.slid >> 23) + static_cast<int>(s.pos >> 16) - static_cast<int>(kPosBias);
+}
 
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
@@ -465,7 +496,6 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   k.shv = half ? 16u : 0u;
   // Keep the per-lane constants in vector registers (the steps name them as VGPR operands).
   asm volatile("" : "+v"(k.f0v), "+v"(k.f1v), "+v"(k.ktab), "+v"(k.shv));
-  const uint32_t* payload32 = reinterpret_cast<const uint32_t*>(a.payload);
   const uint64_t all_lanes = ~0ull;
 
   for (int first_pair = pair_begin + wave * ILP; first_pair < pair_end; first_pair += pair_stride) {
@@ -483,6 +513,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       s.x = kStateMin;
       s.vector0 = 0;
       s.coset_base = 0;
+      s.coset_mask = 0;
       s.dot_row = -1;
 #pragma unroll
       for (int m = 0; m < kDotRows; ++m) s.dot_acc[m] = 0.0f;
@@ -502,14 +533,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         }
       }
       full = full && s.count == a.tile_vectors;
-      open_window(s, window_at, word_begin, word_end, a.payload, a.payload_words, l32);
+      open_window(s, window_at, word_begin, word_end, s.count > 0, a.payload, a.payload_words, a.offsets, l32);
     }
     const bool all_full = __builtin_amdgcn_readfirstlane(__all(full) ? 1 : 0) != 0;
 
     // After a step: a half whose position fell below 64 slides its window down by 64 words. All 32 lanes of the half
     // (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
     // the next 64 words down.
-    auto top_up = [&](Pair& s) { slide_window(s, half, payload32); };
+    auto top_up = [&](Pair& s) { slide_window(s); };
 
     // E8 point and row scale of the vector each valid lane just decoded. The reference forms (z + c / 2) * scale with
     // one rounding. For an ordinary scale (positive, neither tiny nor huge) fma(z, scale, c * scale / 2) is the same
@@ -664,38 +695,32 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       s.dot_row = any ? low : -1;
     };
 
-    // Two-level tables: LDS address of the lane's coset's slot table of field 0 (coset_base is 0 or one FB stream).
-    auto sym_slot_base = [](uint32_t coset_base) {
-      return static_cast<uint32_t>(kSymFbBytes) + (coset_base != 0 ? L::kTable : 0u);
+    // Two-level tables: LDS address of the lane's coset's slot table of field 0.
+    auto sym_slot_base = [](const Pair& s) {
+      return __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? static_cast<uint32_t>(kSymFbBytes) + L::kTable : static_cast<uint32_t>(kSymFbBytes);
     };
 
-    // One group of 32 vectors per half, both interleaved pairs in lock step. `valid` is the wave's lane mask.
-    auto group_dual = [&](auto masked_tag, int offset, bool valid_lane, uint64_t valid) {
+    using Masked = std::integral_constant<bool, true>;
+    using Unmasked = std::integral_constant<bool, false>;
+
+    // The nine steps of a group for the wave's pairs in lock step, windows kept filled. `valid` is the wave's lane mask.
+    // A window is checked (and slid) after every second step: a step consumes at most 32 words per half and a check
+    // leaves at least 64 in the window. The checks sit after fields 0, 2, 4, 6 and after the group's last step.
+    auto group_steps = [&](auto masked_tag, bool valid_lane, uint64_t valid) {
       constexpr bool MASKED = decltype(masked_tag)::value;
-      uint32_t vector[ILP];
-      float scale[ILP];
-      DotInput dot_in[ILP];
-#pragma unroll
-      for (int j = 0; j < ILP; ++j) {
-        vector[j] = st[j].vector0 + static_cast<uint32_t>(offset) + l32;
-        const uint32_t row = row_of(a, vector[j]);
-        scale[j] = valid_lane ? a.scales[row] : 0.0f;
-        if constexpr (DOT_ROWS > 0) dot_prefetch(vector[j], row, valid_lane, dot_in[j]);
-      }
-      // A window is checked (and slid) after every second step: a step consumes at most 32 words per half and a check
-      // leaves at least 64 in the window. The checks sit after fields 0, 2, 4, 6 and after the group's last step.
       if constexpr (ILP == 2) coset_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], k, valid);
       else coset_step_single<PB, MODE, MASKED>(st[0], k, valid);
       uint32_t high[ILP];
 #pragma unroll
       for (int j = 0; j < ILP; ++j) high[j] = st[j].coset_base + L::kHighBase;
+      const uint32_t slot_base = MODE == kModeSym ? sym_slot_base(st[0]) : 0u;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
           rank_step<PB, MASKED>(st[0], f, st[0].coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)),
                                 rank_val0, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
-          sym_step<PB, MASKED>(st[0], f, sym_slot_base(st[0].coset_base), k, valid_lane);
+          sym_step<PB, MASKED>(st[0], f, slot_base, k, valid_lane);
         } else if constexpr (ILP == 2) {
           field_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], f, f & 3, f < 4 ? st[0].coset_base : high[0],
                                             f < 4 ? st[ILP - 1].coset_base : high[ILP - 1], k, valid);
@@ -707,12 +732,89 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
           for (int j = 0; j < ILP; ++j) top_up(st[j]);
         }
       }
+    };
+
+    // The whole groups of a wave of full tiles (all lanes valid) carry the row's scale from group to group: a lane's
+    // vectors walk down through its tile 32 at a time and change rows rarely. Positions are kept relative to the
+    // pair's lower tile, in units of one bf16 vector's bytes: the same number is the lane's store offset from a
+    // wave-uniform address and, compared with where the lane's current row begins, says when that row is left.
+    struct RowCursor {
+      int32_t row_begin;      // position of the first vector of the lane's row (INT32_MIN: at or below the pair's first)
+      float scale, half_scale;
+      uint64_t unusual;       // wave-uniform: lanes whose scale needs the literal formula
+    };
+    auto lower_tile_of = [&](int j) { return static_cast<uint32_t>(2 * static_cast<int64_t>(first_pair + j) * a.tile_vectors); };
+
+    // One group of 32 vectors per half; every lane looks its row and scale up.
+    auto group_dual = [&](auto masked_tag, int offset, bool valid_lane, uint64_t valid) {
+      uint32_t vector[ILP];
+      float scale[ILP];
+      DotInput dot_in[ILP];
+#pragma unroll
+      for (int j = 0; j < ILP; ++j) {
+        vector[j] = st[j].vector0 + static_cast<uint32_t>(offset) + l32;
+        const uint32_t row = row_of(a, vector[j]);
+        scale[j] = valid_lane ? a.scales[row] : 0.0f;
+        if constexpr (DOT_ROWS > 0) dot_prefetch(vector[j], row, valid_lane, dot_in[j]);
+      }
+      group_steps(masked_tag, valid_lane, valid);
       if constexpr (DOT_ROWS > 0) {
 #pragma unroll
         for (int j = 0; j < ILP; ++j) dot_emit(st[j], scale[j], valid_lane, dot_in[j]);
       } else if (valid_lane) {
 #pragma unroll
         for (int j = 0; j < ILP; ++j) emit(st[j], vector[j], scale[j]);
+      }
+    };
+
+    // A whole group on the carried scales. A lane that has left its row makes the wave look its rows up first.
+    RowCursor cursor[ILP];
+    const uint32_t lane_at = 16u * (static_cast<uint32_t>(half ? a.tile_vectors : 0) + static_cast<uint32_t>(l32));
+#pragma unroll
+    for (int j = 0; j < ILP; ++j) cursor[j] = RowCursor{0x7FFFFFFF, 0.0f, 0.0f, 0};
+    auto group_tracked = [&](int offset) {
+      const uint32_t at = lane_at + 16u * static_cast<uint32_t>(offset);
+      bool left = false;
+#pragma unroll
+      for (int j = 0; j < ILP; ++j) left = left || static_cast<int32_t>(at) < cursor[j].row_begin;
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(left) != 0, 0)) {
+#pragma unroll
+        for (int j = 0; j < ILP; ++j) {
+          const uint32_t row = row_of(a, lower_tile_of(j) + (at >> 4));
+          const float scale = a.scales[row];
+          const int64_t begins = static_cast<int64_t>(row) * a.vecs_per_row - lower_tile_of(j);
+          cursor[j].row_begin = begins > 0 ? static_cast<int32_t>(begins * 16) : static_cast<int32_t>(0x80000000u);
+          cursor[j].scale = scale;
+          cursor[j].half_scale = __fmul_rn(scale, 0.5f);
+          cursor[j].unusual = __builtin_amdgcn_ballot_w64(!(__float_as_uint(scale) - 0x0DA24260u <= 0x7149F2CAu - 0x0DA24260u));
+        }
+      }
+      group_steps(Unmasked{}, true, all_lanes);
+#pragma unroll
+      for (int j = 0; j < ILP; ++j) {
+        const RowCursor& c = cursor[j];
+        const Pair& s = st[j];
+        if constexpr (KIND == EP_STORE_BF16 && !WIDE) {
+          float w[8];
+          uint32_t packed[4];
+          if (__builtin_expect(c.unusual == 0, 1)) {
+            float z[8];
+            lattice_point(s, z);
+            const float shift = __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? c.half_scale : 0.0f;
+#pragma unroll
+            for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], c.scale, shift);
+            pack_bf16(w, 1.0f, packed);
+          } else {
+            weights_of(s, c.scale, w);
+            pack_bf16(w, c.scale, packed);
+          }
+          typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+          const u32x4 quad = {packed[0], packed[1], packed[2], packed[3]};
+          uint8_t* lower_out = static_cast<uint8_t*>(a.out) + 16ull * lower_tile_of(j);
+          __builtin_nontemporal_store(quad, reinterpret_cast<u32x4*>(lower_out + at));
+        } else {
+          emit(s, lower_tile_of(j) + (at >> 4), c.scale);
+        }
       }
     };
 
@@ -726,13 +828,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       if constexpr (DOT_ROWS > 0) dot_prefetch(vector, row, valid_lane, dot_in);
       coset_step_single<PB, MODE, true>(s, k, valid);
       const uint32_t high = s.coset_base + L::kHighBase;
+      const uint32_t slot_base = MODE == kModeSym ? sym_slot_base(s) : 0u;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
           rank_step<PB, true>(s, f, s.coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)), rank_val0, k,
                               valid_lane);
         } else if constexpr (MODE == kModeSym) {
-          sym_step<PB, true>(s, f, sym_slot_base(s.coset_base), k, valid_lane);
+          sym_step<PB, true>(s, f, slot_base, k, valid_lane);
         } else {
           field_step_single<PB, MODE, true>(s, f, f & 3, f < 4 ? s.coset_base : high, k, valid);
         }
@@ -742,9 +845,6 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       else if (valid_lane) emit(s, vector, scale);
     };
 
-    using Masked = std::integral_constant<bool, true>;
-    using Unmasked = std::integral_constant<bool, false>;
-
     if (all_full) {
       // Every tile of this wave is full: one schedule for all halves. The short first group, then whole groups.
       const int rem = a.tile_vectors & 31;
@@ -753,10 +853,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         const bool valid_lane = l32 < rem;
         group_dual(Masked{}, offset, valid_lane, __builtin_amdgcn_ballot_w64(valid_lane));
       }
+      // Nothing read so far may still be in flight when the loop starts: the compiler would otherwise wait for it
+      // inside the loop, on every pass, and each such wait also covers the loop's own newest payload request.
+      __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
 #pragma unroll 1
       while (offset > 0) {
         offset -= 32;
-        group_dual(Unmasked{}, offset, true, all_lanes);
+        if constexpr (DOT_ROWS == 0) group_tracked(offset);
+        else group_dual(Unmasked{}, offset, true, all_lanes);
       }
     } else {
 #pragma unroll

@@ -225,7 +225,6 @@ __global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) voi
   asm volatile("" : "+v"(shv));                           // the step names it as a vector operand
 #pragma unroll
   for (int c = 0; c < NC; ++c) asm volatile("" : "+v"(table_at[c]));
-  const uint32_t* payload32 = reinterpret_cast<const uint32_t*>(a.payload);
   const uint8_t* payload8 = reinterpret_cast<const uint8_t*>(a.payload);
   const uint32_t mine_at = static_cast<uint32_t>(wave * 2 + half) * CODED;
   const int tile_elements = static_cast<int>(a.tile_elements);
@@ -272,7 +271,7 @@ __global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) voi
       }
     }
 #pragma unroll
-    for (int c = 0; c < CODED; ++c) open_window(st[c], lds0 + windows0 + (mine_at + c) * kRingBytes, begin[c], end[c], a.payload, a.payload_words, l32);
+    for (int c = 0; c < CODED; ++c) open_window(st[c], lds0 + windows0 + (mine_at + c) * kRingBytes, begin[c], end[c], count > 0, a.payload, a.payload_words, a.offsets, l32);
     // Wave-uniform base, 32-bit lane offsets: the addresses cost one vector add per access.
     Word* out = reinterpret_cast<Word*>(a.out) + 2 * static_cast<int64_t>(pair) * a.tile_elements;
     const uint32_t out_half = static_cast<uint32_t>(half * tile_elements);
@@ -297,7 +296,7 @@ __global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) voi
             const uint32_t symbol = tile_ans_step<false>(st[c], pb, kslot, table_at[c], shv, ~0ull);
             const uint32_t stage = lds0 + stages0 + (mine_at + c) * kTileChunk;
             *reinterpret_cast<__attribute__((address_space(3))) uint8_t*>(static_cast<uintptr_t>(stage + 32u * g + l32)) = static_cast<uint8_t>(symbol);
-            if ((g & 1) == 0) slide_window(st[c], half, payload32);     // a step takes at most 32 words, the window holds 64
+            if ((g & 1) == 0) slide_window(st[c]);     // a step takes at most 32 words, the window holds 64
           }
         }
         if constexpr (CODED > 0) {
@@ -372,7 +371,7 @@ __global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) voi
         for (int c = 0; c < CODED; ++c) {
           const uint32_t symbol = tile_ans_step<true>(st[c], pb, kslot, table_at[c], shv, valid);
           value |= static_cast<Word>(static_cast<Word>(symbol) << (8 * coded_pos[c]));
-          slide_window(st[c], half, payload32);
+          slide_window(st[c]);
         }
         if (valid_lane) __builtin_nontemporal_store(value, out + (out_half + at));
       }
@@ -499,7 +498,8 @@ extern "C" int ep_hip_decode_tile_ans(const uint16_t* payload_dev, uint64_t payl
   const int64_t streams = args.tiles * num_lanes;
   if (streams >= (int64_t{1} << 31)) return EP_HIP_EUNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (coded <= kMaxTileCodedLanes && args.tile_elements < (int64_t{1} << 28) && payload_words < (uint64_t{1} << 31)) {
+  // The tile kernel counts a stream's window slides (one per 64 words, at most one word per element) in 16 bits.
+  if (coded <= kMaxTileCodedLanes && args.tile_elements <= (int64_t{1} << 22) && payload_words < (uint64_t{1} << 31)) {
     int device = 0, compute_units = 0;
     EP_HIP_TRY(hipGetDevice(&device));
     EP_HIP_TRY(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
