@@ -55,7 +55,7 @@ struct Pair {
   uint32_t prefetch;     // the 64 payload words below the ring, 2 per lane
   uint32_t fetch_at;     // byte offset from `origin` of the dword `prefetch` came from
   const uint8_t* origin; // wave-uniform: a 64-word boundary of the payload at or below every word the pair still needs
-  uint32_t ring;         // LDS byte address of this half's 128-word window
+  uint32_t ring;         // half the LDS byte address of position 0 of this half's 128-word window
   uint32_t ring_lane;    // ring + 4 * (lane & 31): where this lane's dword of a 64-word chunk goes
   uint32_t vector0;      // first vector of this lane's tile
   int count;             // vectors in this lane's tile (0 = no tile)
@@ -96,17 +96,18 @@ struct Pair {
 // With n_a, n_b the halves' counts: lane l of the lower half reads at p_a - n_a + rank(l), and a lane of the upper
 // half, whose rank as the two mbcnt instructions count it includes n_a, at p_b - (n_a + n_b) + rank(l). Both bases
 // come from one subtraction of (n_a | (n_a + n_b) << 16); the positions themselves (p - n per half) follow after
-// the read is issued. pos stays >= 32 in both halves, so no subtraction borrows across the 16-bit fields.
+// the read is issued. The lane ranks are counted on top of half the window's byte address while the scalar side is
+// still busy, so that only two vector instructions separate the scalar result from the read. pos stays >= 32 in both halves, so no subtraction borrows across the 16-bit fields.
 #define EP_ASM_VOTE(S)                                          \
   "v_cmp_gt_u32 vcc, 0x8000, %[x" S "]\n"                        \
   "s_bcnt1_i32_b32 %[na], vcc_lo\n"                              \
   "s_bcnt1_i32_b64 %[nb], vcc\n"                                 \
+  "v_mbcnt_lo_u32_b32 %[t" S "], vcc_lo, %[ring" S "]\n"         \
   "s_pack_ll_b32_b16 %[nb], %[na], %[nb]\n"                      \
-  "s_sub_u32 %[nb], %[pos" S "], %[nb]\n"                        \
-  "v_bfe_u32 %[t" S "], %[nb], %[shv], 16\n"                     \
-  "v_mbcnt_lo_u32_b32 %[t" S "], vcc_lo, %[t" S "]\n"            \
   "v_mbcnt_hi_u32_b32 %[t" S "], vcc_hi, %[t" S "]\n"            \
-  "v_lshl_add_u32 %[t" S "], %[t" S "], 1, %[ring" S "]\n"       \
+  "s_sub_u32 %[nb], %[pos" S "], %[nb]\n"                        \
+  "v_bfe_u32 %[d" S "], %[nb], %[shv], 16\n"                     \
+  "v_add_lshl_u32 %[t" S "], %[t" S "], %[d" S "], 1\n"          \
   "ds_read_u16 %[d" S "], %[t" S "]\n"                           \
   "s_lshl_b32 %[na], %[na], 16\n"                                \
   "s_add_u32 %[pos" S "], %[nb], %[na]\n"
@@ -387,7 +388,7 @@ __device__ __forceinline__ void lds_store32(uint32_t at, uint32_t value) {
 __device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_t word_begin, uint32_t word_end, bool live,
                                             const uint16_t* __restrict__ payload, uint64_t payload_words, const void* readable,
                                             int l32) {
-  s.ring = window_at - 2u * kPosBias;                   // positions are kept biased, see Pair::pos
+  s.ring = window_at / 2u - kPosBias;                    // positions are kept biased, see Pair::pos
   const uint32_t base = word_begin & ~63u;               // absolute index of relative position 0
   const int begin = static_cast<int>(word_begin - base);
   const int ptr = static_cast<int>(word_end - base);
