@@ -795,26 +795,28 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       for (int j = 0; j < ILP; ++j) {
         const RowCursor& c = cursor[j];
         const Pair& s = st[j];
-        if constexpr (KIND == EP_STORE_BF16 && !WIDE) {
-          float w[8];
-          uint32_t packed[4];
-          if (__builtin_expect(c.unusual == 0, 1)) {
-            float z[8];
-            lattice_point(s, z);
-            const float shift = __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? c.half_scale : 0.0f;
+        float w[8];
+        if (__builtin_expect(c.unusual == 0, 1)) {
+          float z[8];
+          lattice_point(s, z);
+          const float shift = __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? c.half_scale : 0.0f;
 #pragma unroll
-            for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], c.scale, shift);
-            pack_bf16(w, 1.0f, packed);
-          } else {
-            weights_of(s, c.scale, w);
-            pack_bf16(w, c.scale, packed);
-          }
+          for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], c.scale, shift);
+        } else {
+          weights_of(s, c.scale, w);
+        }
+        if constexpr (KIND == EP_STORE_BF16) {
+          uint32_t packed[4];
+          if (__builtin_expect(c.unusual == 0, 1)) pack_bf16(w, 1.0f, packed);     // an ordinary scale never saturates
+          else pack_bf16(w, c.scale, packed);
           typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
           const u32x4 quad = {packed[0], packed[1], packed[2], packed[3]};
           uint8_t* lower_out = static_cast<uint8_t*>(a.out) + 16ull * lower_tile_of(j);
           __builtin_nontemporal_store(quad, reinterpret_cast<u32x4*>(lower_out + at));
+        } else if constexpr (KIND == EP_STORE_I8) {
+          store_vector_i8(a.out, lower_tile_of(j) + (at >> 4), w);
         } else {
-          emit(s, lower_tile_of(j) + (at >> 4), c.scale);
+          store_vector(a.out, a.store_kind, lower_tile_of(j) + (at >> 4), w);
         }
       }
     };
