@@ -45,6 +45,8 @@ inline int tile_vectors_of(int tile_elements) {
   const int v = tile_elements / 9;
   return v > 32 ? v : 32;
 }
+// Largest tile the LDS-table kernels take (plans for larger tiles use the global tables).
+constexpr int kMaxLdsTileVectors = 1 << 18;
 
 // LDS_RANK plan layout after the header: FB u32[P] | VAL i16[P] | RS {u32 bits, u32 count}[16][2^pb / 32], each part
 // starting on a multiple of 16 bytes and RS on a multiple of one stream's RS size (its base is OR-ed with word offsets).

@@ -166,7 +166,7 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
 
   // The LDS-table kernels address a pair of tiles with 32-bit byte offsets (16 bytes per vector) and count a tile's
   // window slides (one per 64 payload words, at most nine words per vector) in 16 bits.
-  if (desc->table_kind != EP_TABLE_GLOBAL64 && tv > (1 << 18)) return EP_HIP_EUNSUPPORTED;
+  if (desc->table_kind != EP_TABLE_GLOBAL64 && tv > kMaxLdsTileVectors) return EP_HIP_EUNSUPPORTED;
   switch (desc->table_kind) {
     case EP_TABLE_GLOBAL64:
       return EP_HIP_OK;

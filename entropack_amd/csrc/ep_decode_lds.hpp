@@ -10,16 +10,19 @@
 // checked: when p has dropped below 64 it slides down by 64 words (its lower chunk moves up, the prefetched words
 // become the lower chunk and the next 64 are requested), so p is in [64, 128) before a pair of steps, at least 32
 // between them and at least 0 after them, whatever the stream holds, and no renormalisation ever waits on HBM.
-// Both halves' p live in one scalar register, biased by 64 so that the packed arithmetic never borrows.
+// Both halves' p live in one scalar register, biased by 64 so that the packed arithmetic never borrows; the
+// requests address the payload as a wave-uniform origin plus a saturating 32-bit offset per lane, and slides are
+// counted (the end-of-tile check needs to know where each window ended up).
 //
 // The nine dependent symbol steps of a group are written in inline assembly: the compiler's version of the same
-// C++ spent more scalar than vector instructions on mask bookkeeping. Per step and pair: 12 VALU, 9 SALU, one
+// C++ spent more scalar than vector instructions on mask bookkeeping. Per step and pair: 12 VALU, 8 SALU, one
 // ds_read_b32 (slot table) and one ds_read_u16 (window). The scalar part turns the vote of "state < 2^15" into
 // the two halves' word counts; lane l then reads window[p_half - n_half + rank_in_half(l)], which is the
 // reference's "i-th reader in ascending lane order takes words[ptr - n + i]".
 //
 // Everything around the steps (tile set-up, ring refill, E8 reconstruction, row scale, container cast, stores,
-// end-of-tile checks) is ordinary HIP C++.
+// end-of-tile checks) is ordinary HIP C++. Tiles hold at most kMaxLdsTileVectors vectors: positions inside a pair
+// of tiles are 32-bit byte offsets and a tile's slides are counted in 16 bits.
 #pragma once
 
 #include <type_traits>

@@ -241,9 +241,12 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   if (cursor != static_cast<int64_t>(n_freq)) return EP_HIP_EINVAL;
   if (meta[0 * 4 + 3] == 0) return EP_HIP_EINVAL;
 
-  const bool lds_fits = prob_bits <= 11 && ep::lds_decode_bytes(prob_bits, 1, 1) <= lds_limit_bytes;
+  // The LDS-table kernels take tiles of at most 2^18 vectors (32-bit byte offsets inside a tile pair, 16-bit slide
+  // counts); larger tiles get the global tables.
+  const bool tile_fits = ep::tile_vectors_of(tile_elements) <= ep::kMaxLdsTileVectors;
+  const bool lds_fits = tile_fits && prob_bits <= 11 && ep::lds_decode_bytes(prob_bits, 1, 1) <= lds_limit_bytes;
   const bool sym_ok = byte_ok && lds_fits;
-  rank_ok = rank_ok && present <= 65535 && ep::lds_rank_decode_bytes(static_cast<int>(present), prob_bits, 4) <= lds_limit_bytes;
+  rank_ok = rank_ok && tile_fits && present <= 65535 && ep::lds_rank_decode_bytes(static_cast<int>(present), prob_bits, 4) <= lds_limit_bytes;
   int kind = EP_TABLE_GLOBAL64;
   if (lds_fits && byte_ok) kind = EP_TABLE_LDS_BYTE;
   else if (lds_fits && wide_ok) kind = EP_TABLE_LDS_WIDE;

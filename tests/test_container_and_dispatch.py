@@ -231,6 +231,10 @@ def test_plan_describe_rejects_inconsistent_tables():
     assert _describe(meta, freq, 11, lds=2 * 1024)[1].table_kind == hip_backend.TABLE_GLOBAL64
     assert _describe(meta, freq, 11, force=hip_backend.TABLE_GLOBAL64)[1].table_kind == hip_backend.TABLE_GLOBAL64
     assert _describe(meta, freq, 11, tile_elements=0)[0] == hip_backend.EINVAL
+    # Tiles beyond 2**18 vectors are outside what the LDS-table kernels address: such plans take the global tables.
+    assert _describe(meta, freq, 11, tile_elements=9 << 18)[1].table_kind == hip_backend.TABLE_LDS_BYTE
+    assert _describe(meta, freq, 11, tile_elements=(9 << 18) + 9)[1].table_kind == hip_backend.TABLE_GLOBAL64
+    assert _describe(meta, freq, 11, tile_elements=(9 << 18) + 9, force=hip_backend.TABLE_LDS_BYTE)[0] == hip_backend.EUNSUPPORTED
     wide_only = Golden("huge_alpha_16x1024_bf16_7p0")
     assert _describe(wide_only.buffers["stream_meta"], wide_only.buffers["freq_tables"], 11,
                      force=hip_backend.TABLE_LDS_BYTE)[0] == hip_backend.EUNSUPPORTED

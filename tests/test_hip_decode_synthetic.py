@@ -108,6 +108,14 @@ def test_rates_precisions_and_tile_sizes(options):
     decode_and_check(gauss(22, 512, 1024), kinds=ALL_KINDS, **options)
 
 
+def test_tiles_beyond_the_lds_kernels_take_the_global_tables():
+    """A tile of more than 2**18 vectors is outside what the LDS-table kernels address; its plan picks the general
+    kernel by itself, and forcing an LDS form is refused rather than run."""
+    container, used = decode_and_check(gauss(24, 640, 4096), kinds=(None, hip_backend.TABLE_LDS_BYTE), target_bpp=4.0,
+                                       tile_elements=(9 << 18) + 9)
+    assert used == ["global64"]
+
+
 def test_constant_and_zero_tensors():
     decode_and_check(torch.zeros(64, 256, dtype=torch.bfloat16), kinds=ALL_KINDS, target_bpp=4.0)
     decode_and_check(torch.full((64, 256), 0.5, dtype=torch.bfloat16), kinds=ALL_KINDS, target_bpp=4.0)
