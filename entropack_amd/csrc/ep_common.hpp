@@ -26,7 +26,7 @@ constexpr size_t kHeaderBytes = kHeaderWords * 4;
 // GLOBAL64 entry: symbol[0:16) | freq[16:32) | (slot - cdf)[32:64)
 
 // Payload ring kept in LDS per tile by the LDS-table kernels: 2 chunks of 64 words.
-constexpr int kRingWords = 128;
+constexpr int kRingWords = 192;       // a stream's LDS window: three chunks of 64 payload words
 constexpr int kRingBytes = kRingWords * 2;
 constexpr int kChunkWords = 64;
 

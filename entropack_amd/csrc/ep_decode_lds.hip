@@ -33,8 +33,24 @@ static int lds_bytes_for(int table_kind, int prob_bits, int lut_bytes, int waves
   return lds_decode_bytes(prob_bits, waves, ilp);
 }
 
+// Workgroups per CU and the largest workgroup (in waves) for a table form: two workgroups when their tables and
+// at least 12 waves' windows each fit the CU's LDS together (8 waves per SIMD with 16), else one of 16 waves.
+static void lds_block_shape(int table_kind, int prob_bits, int lut_bytes, int& resident, int& most_waves) {
+  for (int waves = 16; waves >= 12; --waves) {
+    if (2 * lds_bytes_for(table_kind, prob_bits, lut_bytes, waves, 1) <= 160 * 1024) {
+      resident = 2;
+      most_waves = waves;
+      return;
+    }
+  }
+  resident = 1;
+  most_waves = 16;
+}
+
 int lds_resident_blocks(int table_kind, int prob_bits, int lut_bytes) {
-  return 2 * lds_bytes_for(table_kind, prob_bits, lut_bytes, 16, 1) <= 160 * 1024 ? 2 : 1;
+  int resident = 1, most_waves = 16;
+  lds_block_shape(table_kind, prob_bits, lut_bytes, resident, most_waves);
+  return resident;
 }
 
 int effective_table_kind(const ep_hip_plan_desc& desc, int kind, int64_t pairs, int cus) {
@@ -51,11 +67,12 @@ LdsLaunch choose_lds_launch(int table_kind, int prob_bits, int lut_bytes, int ki
   cfg.kind = kind;
   // Tables that leave room for two blocks per CU run one pair per wave on twice the waves, which hides latency best.
   // Otherwise one block per CU, and two interleaved pairs per wave once 16 waves on every CU cannot hold all pairs.
-  const int resident = lds_resident_blocks(table_kind, prob_bits, lut_bytes);
+  int resident = 1, most_waves = 16;
+  lds_block_shape(table_kind, prob_bits, lut_bytes, resident, most_waves);
   const bool single_pair_only = table_kind == EP_TABLE_LDS_RANK || table_kind == EP_TABLE_LDS_SYM;
   cfg.ilp = !single_pair_only && resident == 1 && pairs > cus * 16 ? 2 : 1;
   int waves = (pairs + cus * resident * cfg.ilp - 1) / (cus * resident * cfg.ilp);
-  waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
+  waves = waves < 1 ? 1 : (waves > most_waves ? most_waves : waves);
   int blocks = (pairs + waves * cfg.ilp - 1) / (waves * cfg.ilp);
   cfg.blocks = blocks > cus * resident ? cus * resident : blocks;
   cfg.threads = waves * 64;

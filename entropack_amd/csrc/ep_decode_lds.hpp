@@ -5,7 +5,7 @@
 // CU stages the 16 field tables once (u32 per slot: frequency | slot - cdf | symbol) and then walks its pairs.
 //
 // Payload. Renormalisation words are consumed from the tile's end downwards, at most 32 per step. Each half keeps
-// a 128-word LDS window holding payload[W, W + 128), W a multiple of 64, with the read position p = ptr - W. The 64
+// a 192-word LDS window holding payload[W, W + 192), W a multiple of 64, with the read position p = ptr - W. The 64
 // words below W are already in flight in a register (one dword per lane). After every second step the window is
 // checked: when p has dropped below 64 it slides down by 64 words (its lower chunk moves up, the prefetched words
 // become the lower chunk and the next 64 are requested), so p is in [64, 128) before a pair of steps, at least 32
@@ -422,25 +422,32 @@ __device__ __forceinline__ void open_window(Pair& s, uint32_t window_at, uint32_
   s.beginB = __builtin_amdgcn_readlane(begin, 32);
 }
 
-// After a step (or two): a half whose position fell below 64 slides its window down by 64 words. All 32 lanes of the
-// half (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
-// the next 64 words down. Which halves slide is a scalar decision, and the lanes are picked by a mask built from it;
-// the scalar side is kept short (it is what the common, non-sliding case pays for: three instructions).
+// After a step (or two): a half whose position fell below 64 slides its window down by 64 words, and the other half
+// slides along if it can (its position is below 128, so that it stays inside the 192-word window afterwards): the two
+// streams of a wave are consumed at about the same rate, so this keeps their slides together, one event and one
+// request for both instead of two. All 32 lanes of a sliding half (voting or not) move their dwords of the two lower
+// chunks up, drop their prefetched dword in the lowest and ask for the next 64 words down. Which halves slide is a
+// scalar decision, and the lanes are picked by a mask built from it; the scalar side is kept short (it is what the
+// common, non-sliding case pays for: three instructions).
 __device__ __forceinline__ void slide_window(Pair& s) {
   const uint32_t low_bits = ~s.pos & 0x00800080u;        // bit 7 of a biased field clear <=> that position < 64
   if (__builtin_expect(low_bits != 0, 0)) {
     asm volatile("" ::: "memory");     // keep this a scalar branch: the common case must cost no vector work
-    const uint32_t lower = static_cast<uint32_t>(static_cast<int32_t>(low_bits << 24) >> 31);
-    const uint32_t upper = static_cast<uint32_t>(static_cast<int32_t>(low_bits << 8) >> 31);
+    const uint32_t sliding = ~(s.pos & (s.pos << 1)) & 0x00800080u;    // bits 7 and 6 not both set <=> position < 128
+    const uint32_t lower = static_cast<uint32_t>(static_cast<int32_t>(sliding << 24) >> 31);
+    const uint32_t upper = static_cast<uint32_t>(static_cast<int32_t>(sliding << 8) >> 31);
     if (__builtin_amdgcn_inverse_ballot_w64(static_cast<uint64_t>(lower) | (static_cast<uint64_t>(upper) << 32))) {
-      const uint32_t kept = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uintptr_t>(s.ring_lane));
-      lds_store32(s.ring_lane + 128u, kept);
+      typedef __attribute__((address_space(3))) uint32_t* lds_u32;
+      const uint32_t kept0 = *reinterpret_cast<lds_u32>(static_cast<uintptr_t>(s.ring_lane));
+      const uint32_t kept1 = *reinterpret_cast<lds_u32>(static_cast<uintptr_t>(s.ring_lane + 128u));
+      lds_store32(s.ring_lane + 256u, kept1);
+      lds_store32(s.ring_lane + 128u, kept0);
       lds_store32(s.ring_lane, s.prefetch);
       s.fetch_at = s.fetch_at >= 128u ? s.fetch_at - 128u : 0u;
       s.prefetch = *reinterpret_cast<const uint32_t*>(s.origin + s.fetch_at);
     }
-    s.pos += low_bits >> 1;             // + 64 in the fields that slid
-    s.slid += low_bits;                 // one more slide for them
+    s.pos += sliding >> 1;              // + 64 in the fields that slid
+    s.slid += sliding;                  // one more slide for them
   }
 }
 
