@@ -98,7 +98,8 @@ int ep_hip_device_query(int device, ep_hip_device_info* info);
 /* Chooses the table representation from host copies of the container's stream_meta (int32[17][4] =
  * n_symbols, sym_min, freq_offset, alphabet) and freq_tables (u16[n_freq]), and validates them (offsets
  * contiguous, every stream's frequencies sum to 2^prob_bits). Pure host code, no GPU needed. `tile_elements` is
- * the container's layout[2] (must be positive).
+ * the container's layout[2] (must be positive); tiles of more than 2^18 vectors (tile_elements above 2 359 296) get
+ * EP_TABLE_GLOBAL64, the LDS forms do not address them.
  * Reference: _decode_plan's representation choice, entropack/schemes/lattice_rans/cuda.py:697-732.
  * `force_kind` < 0 lets the library choose; otherwise it must be a kind the container qualifies for. */
 int ep_hip_plan_describe(const int32_t* stream_meta_host, const uint16_t* freq_tables_host, size_t n_freq,
@@ -117,7 +118,8 @@ int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_table
 /* Entropy-decodes every tile and reconstructs straight into `out_dev` ([rows][cols_padded] of `store_kind`,
  * row-major, 16-byte aligned): rANS symbol steps, shared renormalisation, field minima, E8 point, row scale and
  * container cast, in one kernel. payload_dev must be 4-byte aligned. `error_dev` (int32, caller-zeroed) receives
- * an ep_hip_decode_error; it is never read back here.
+ * an ep_hip_decode_error; it is never read back here. EP_HIP_EUNSUPPORTED for an LDS plan with tiles of more than
+ * 2^18 vectors (ep_hip_plan_describe never makes one unless forced).
  * Reference: decode() + _decode_launch() and the e8_decode_vector_* kernels they launch,
  * entropack/schemes/lattice_rans/cuda.py:744-805, lattice_rans.cu:732-1141. */
 int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t payload_words, const uint32_t* offsets_dev,
