@@ -105,3 +105,40 @@ def test_corrupt_payload_sets_the_error_flag_and_stays_in_bounds():
         with pytest.raises(ValueError, match="decode error"):
             hip_lane.check_errors(lattice)
         hip_lane.check_errors(lattice)                         # the flag was cleared by the read
+
+
+@pytest.mark.parametrize("damage", ["payload", "boundaries", "order"])
+def test_damaged_streams_decode_to_completion_with_the_flag_set(damage):
+    """Streams that are readable but wrong (flipped payload words, tile boundaries moved inside the payload, two
+    tiles' boundaries swapped) take every kernel through its window refills with positions the encoder never made:
+    the decode must finish, and such damage is reported."""
+    golden = Golden("c1_256x256_bf16_3p5")
+    generator = torch.Generator().manual_seed(5)
+    for kind in (hip_backend.TABLE_GLOBAL64, hip_backend.TABLE_LDS_BYTE, hip_backend.TABLE_LDS_RANK, hip_backend.TABLE_LDS_SYM):
+        hip_lane.FORCE_TABLE_KIND = kind
+        try:
+            compressed = _container(golden)
+            buffers = dict(compressed.buffers)
+            if damage == "payload":
+                payload = buffers["payload"].clone().view(torch.int16)
+                where = torch.randint(0, payload.numel(), (max(1, payload.numel() // 50),), generator=generator)
+                payload[where.to(payload.device)] ^= 0x5A5A
+                buffers["payload"] = payload.view(torch.uint16)
+            else:
+                offsets = buffers["offsets"].clone().view(torch.int32)
+                assert offsets.numel() > 4
+                if damage == "boundaries":
+                    offsets[1:-1] += 7                              # every inner boundary 7 words too high, still ordered
+                    offsets[1:-1] = torch.minimum(offsets[1:-1], offsets[-1])
+                else:
+                    offsets[[1, 2]] = offsets[[2, 1]]                   # tile 1 now ends before it begins
+                buffers["offsets"] = offsets.view(torch.uint32)
+            lattice = LatticeBuffers(**buffers)
+            out = hip_lane.decode(lattice, shape=golden.shape, dtype=torch.bfloat16)
+            torch.cuda.synchronize()
+            assert tuple(out.shape)[0] == golden.shape[0]
+            with pytest.raises(ValueError, match="decode error"):
+                hip_lane.check_errors(lattice)
+        finally:
+            hip_lane.FORCE_TABLE_KIND = None
+
