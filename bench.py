@@ -24,7 +24,7 @@ HBM_PEAK_GBPS = 8000.0
 
 #: HBM bytes per decode launch measured with two rocprofv3 --pmc runs of this script (FETCH_SIZE, scaled by the 2.0
 #: a plain 512 MiB copy calibrates it to, plus WRITE_SIZE, factor 1.0): the default workload and the lossless one.
-MEASURED_TRAFFIC_BYTES = {"target": 600_500_000, "tile_ans": 820_400_000}
+MEASURED_TRAFFIC_BYTES = {"target": 600_700_000, "tile_ans": 818_700_000}
 
 WORKLOADS = {
     # name: (rows, cols, sigma, seed, target_bpp, outliers)
