@@ -23,6 +23,7 @@ import torch
 from torch.utils._python_dispatch import return_and_correct_aliasing
 
 from ..registry import get_scheme
+from ..schemes.base import HOST_MIRROR, HOST_MIRROR_LIMIT
 
 ALIGNMENT = 16          # every component starts 16-byte aligned: the kernels read them with 16-byte loads
 PREFIX_BYTES = 8
@@ -145,21 +146,36 @@ class CompressedTensor(torch.Tensor):
         self._bind(pack_quant_state(header, buffers, shape, dtype if encoded_dtype is None else encoded_dtype))
 
     @classmethod
-    def _wrap(cls, blob: torch.Tensor, shape, dtype) -> "CompressedTensor":
+    def _wrap(cls, blob: torch.Tensor, shape, dtype, parsed=None) -> "CompressedTensor":
         made = torch.Tensor._make_wrapper_subclass(cls, tuple(shape), dtype=dtype, device=blob.device, requires_grad=False)
-        made._bind(blob)
+        made._bind(blob, parsed)
         return made
 
-    def _bind(self, blob: torch.Tensor) -> None:
-        document, start = parse_quant_state(blob)
+    def _bind(self, blob: torch.Tensor, parsed=None) -> None:
+        """`parsed` = (document, first buffer's offset) of a blob with the same bytes, already parsed and validated."""
+        document, start = parse_quant_state(blob) if parsed is None else parsed
         self.entropack_quant_state = blob
+        self._parsed = (document, start)
         self.header = document["header"]
         self.encoded_dtype = _name_to_dtype(document["dtype"])
         self.buffers = buffer_views(blob, document, start)
-        self.validate()
+        if parsed is None:
+            self.validate()
 
     def _rewrap(self, transform, dtype=None) -> "CompressedTensor":
-        return type(self)._wrap(transform(self.entropack_quant_state), self.shape, self.dtype if dtype is None else dtype)
+        """The same bytes in another tensor (a copy, another device, an alias): nothing is parsed again, which for a
+        device blob would mean reading it back. Small metadata buffers that leave the host take a host copy along
+        (`host_copy`), so that planning a decode does not read them back either."""
+        twin = type(self)._wrap(transform(self.entropack_quant_state), self.shape, self.dtype if dtype is None else dtype, self._parsed)
+        for name, view in twin.buffers.items():
+            source = self.buffers[name]
+            mirror = getattr(source, HOST_MIRROR, None)
+            if mirror is None and source.device.type == "cpu" and view.device.type != "cpu" \
+                    and source.numel() * source.element_size() <= HOST_MIRROR_LIMIT:
+                mirror = source.detach().clone()
+            if mirror is not None and view.device.type != "cpu":
+                setattr(view, HOST_MIRROR, mirror)
+        return twin
 
     @classmethod
     def unpack(cls, quant_state: torch.Tensor) -> "CompressedTensor":
@@ -256,10 +272,7 @@ class CompressedTensor(torch.Tensor):
 
     def storage_nbytes(self, include_header: bool = True) -> int:
         total = self.entropack_quant_state.numel()
-        if include_header:
-            return total
-        length = int.from_bytes(bytes(self.entropack_quant_state[:PREFIX_BYTES].detach().cpu().tolist()), "little")
-        return total - _round_up(PREFIX_BYTES + length)
+        return total if include_header else total - self._parsed[1]
 
     def validate(self) -> None:
         """Scheme known, dtype supported, buffer names as the scheme expects. Contents are not inspected."""

@@ -225,9 +225,12 @@ class CompressedLinear(torch.nn.Linear):
     def _adopt_blob(self, blob: torch.Tensor, in_place: bool) -> None:
         """Make the container packed in `blob` this layer's weight. `in_place`: keep the existing Parameter object alive
         (optimisers and hooks hold on to it) and keep its device."""
-        if in_place:
-            blob = blob.to(device=self._home_for(blob), copy=True)
+        # Unpacked where the blob is (a checkpoint's is on the host: the header is read there) and moved as a container,
+        # which takes host copies of the small tables along for the decode plan.
         container = CompressedTensor.unpack(blob)
+        if in_place:
+            home = self._home_for(blob)
+            container = container.to(device=home, copy=True) if home != blob.device else container.clone()
         self._check_weight_shape(container.shape)
         fresh = torch.nn.Parameter(container, requires_grad=False)
         present = self._parameters.get("weight")

@@ -16,12 +16,24 @@ import torch
 from ..registry import DispatchError, backend_device, register_scheme, select
 from .config import CompressionConfig, RawConfig, validate_config
 
-__all__ = ["RawScheme", "Scheme", "cached_parse", "packed_buffers", "register_scheme"]
+__all__ = ["RawScheme", "Scheme", "cached_parse", "host_copy", "packed_buffers", "register_scheme"]
 
 
 def packed_buffers(packed: dict, kind: type):
     """A scheme's buffers, picked out of a name -> tensor mapping in the order of its NamedTuple `kind`."""
     return kind._make(packed[field] for field in kind._fields)
+
+
+#: Attribute a device-resident buffer view carries when a host copy of the same values came along with it (containers
+#: attach it when they move to a device), and the largest buffer that gets one.
+HOST_MIRROR = "_entropack_host_mirror"
+HOST_MIRROR_LIMIT = 64 * 1024
+
+
+def host_copy(tensor: torch.Tensor) -> torch.Tensor:
+    """The values of a small metadata buffer on the host: the copy that travelled with it, else a read-back."""
+    mirror = getattr(tensor, HOST_MIRROR, None)
+    return mirror if mirror is not None else tensor.detach().cpu()
 
 
 def cached_parse(tensor: torch.Tensor, parse, attribute: str):

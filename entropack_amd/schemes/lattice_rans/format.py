@@ -19,7 +19,7 @@ from typing import Annotated, NamedTuple
 
 import torch
 
-from ..base import cached_parse
+from ..base import cached_parse, host_copy
 from ..config import CompressionConfig, OneOf, Range
 
 log = logging.getLogger("entropack.lattice_rans")
@@ -116,7 +116,7 @@ def make_layout(cols: int, prob_bits: int, tile_elements: int) -> torch.Tensor:
 def parse_layout(layout: torch.Tensor) -> dict:
     if layout.dtype != torch.int64 or layout.ndim != 1 or layout.numel() != 3:
         raise ValueError("lattice_rans layout must be int64[3]")
-    cols, prob_bits, tile_elements = (int(v) for v in layout.detach().cpu().tolist())
+    cols, prob_bits, tile_elements = (int(v) for v in host_copy(layout).tolist())
     if cols <= 0 or cols % LATTICE_DIM:
         raise ValueError("lattice_rans vector-plane format requires positive cols divisible by 8")
     if prob_bits not in SUPPORTED_PROB_BITS:

@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from ...backends import hip as _hip
+from ..base import host_copy
 from .format import LatticeBuffers, decode_geometry, snap_to_container
 
 #: float8 formats without a store kernel are decoded to float32 and cast on the device, as the reference does.
@@ -45,8 +46,9 @@ def _plan_for(buffers: LatticeBuffers, info: dict) -> DecodePlan:
         return plan
 
     lib = _hip.library()
-    meta_host = np.ascontiguousarray(meta.detach().cpu().numpy(), dtype=np.int32)      # one small D2H, first call only
-    freq_host = np.ascontiguousarray(freq.detach().cpu().view(torch.int16).numpy()).view(np.uint16)
+    # Host values of the two small tables: the copies that came with the container, else one small read-back each.
+    meta_host = np.ascontiguousarray(host_copy(meta).numpy(), dtype=np.int32)
+    freq_host = np.ascontiguousarray(host_copy(freq).view(torch.int16).numpy()).view(np.uint16)
     if meta_host.shape != (17, 4):
         raise ValueError(f"lattice_rans stream_meta must be (17, 4), got {meta_host.shape}")
     desc = _hip.PlanDesc()

@@ -19,7 +19,7 @@ from typing import Annotated, NamedTuple
 
 import torch
 
-from ..base import cached_parse
+from ..base import cached_parse, host_copy
 from ..config import CompressionConfig, OneOf, Range
 
 AUTO_PROB_BITS = 0
@@ -88,7 +88,7 @@ def parse_layout(layout: torch.Tensor) -> tuple[int, int, int, int]:
     """(tile_elements, prob_bits, lanes, elements)"""
     if layout.dtype != torch.int64 or layout.ndim != 1 or layout.numel() != 4:
         raise ValueError("tile_ans layout must be int64[4]")
-    tile_elements, prob_bits, num_lanes, num_elements = (int(v) for v in layout.detach().cpu().tolist())
+    tile_elements, prob_bits, num_lanes, num_elements = (int(v) for v in host_copy(layout).tolist())
     if tile_elements <= 0 or prob_bits not in SUPPORTED_PROB_BITS or num_lanes <= 0 or num_elements <= 0:
         raise ValueError(f"invalid tile_ans layout values: tile_elements={tile_elements}, prob_bits={prob_bits}, "
                          f"num_lanes={num_lanes}, num_elements={num_elements}")
@@ -101,7 +101,7 @@ def parse_layout_cached(layout: torch.Tensor) -> tuple[int, int, int, int]:
 
 def lane_modes_cached(buffers: "TileBuffers") -> tuple[int, ...]:
     """The lane modes as Python ints, read from the device once per container (kept on the layout tensor object)."""
-    return cached_parse(buffers.layout, lambda _: tuple(int(v) for v in buffers.lane_modes.detach().cpu().tolist()),
+    return cached_parse(buffers.layout, lambda _: tuple(int(v) for v in host_copy(buffers.lane_modes).tolist()),
                         "_tile_ans_lane_modes")
 
 

@@ -63,6 +63,26 @@ def test_state_dict_round_trip_and_sharing():
         container.requires_grad_(True)
 
 
+def test_moving_a_container_parses_nothing_and_takes_host_copies_of_its_small_tables():
+    """A container that leaves the host is not parsed again (on a device that would be two read-backs), and its small
+    tables keep a host copy for the decode plan. The meta device stands in for a GPU: reading a meta tensor back
+    raises, so this passes only if nothing does."""
+    from entropack_amd.schemes.base import HOST_MIRROR, host_copy
+    golden = Golden("c1_256x256_bf16_3p5")
+    container = ep.CompressedTensor.unpack(_blob(golden))
+    moved = container.to("meta")
+    assert moved.device.type == "meta" and moved.shape == container.shape and moved.header == container.header
+    assert moved.storage_nbytes(include_header=False) == container.storage_nbytes(include_header=False)
+    for name in ("layout", "stream_meta", "freq_tables", "scales"):
+        assert torch.equal(host_copy(moved.buffers[name]), container.buffers[name]), name
+        assert host_copy(moved.buffers[name]).data_ptr() != container.buffers[name].data_ptr()      # a copy, not a view
+    assert not hasattr(container.buffers["layout"], HOST_MIRROR)                                   # host buffers need none
+    big = ep.compress((torch.randn(512, 1024) * 0.02).to(torch.bfloat16), ep.EntroPackLossyConfig(target_bpp=4.0, execution_backend="eager"))
+    assert not hasattr(big.to("meta").buffers["payload"], HOST_MIRROR)                              # only small buffers
+    again = moved.clone()                                                                           # copies travel on
+    assert torch.equal(host_copy(again.buffers["stream_meta"]), container.buffers["stream_meta"])
+
+
 def test_torch_save_load_weights_only(tmp_path):
     golden = Golden("ragged_66x200_bf16_4p0")
     container = ep.CompressedTensor.unpack(_blob(golden))
