@@ -177,6 +177,26 @@ def int8_linear_section(ep, steps):
                      "rel_l2_vs_definition_in_bf16": rel, "rel_l2_vs_dense_layer": dense_rel}
     out["quantize_rows_ms"] = round(_median_ms(lambda: kernels.quantize_rows(x), steps), 5)
     out["int8_gemm_ms"] = round(_median_ms(lambda: kernels.int8_gemm(qa, codes, sa, layer.weight_quant_scale.cuda(), None, torch.bfloat16), steps), 5)
+
+    # The same layer as a stack of 32 (own device buffers each), code containers decoded 16 at a time beside the products.
+    import copy
+    stack = [copy.deepcopy(layer).cuda() for _ in range(32)]
+
+    def forward():
+        y = None
+        for member in stack:
+            y = member(x)
+        return y
+
+    reference = forward()
+    alone = _median_ms(forward, max(3, steps // 5), warmup=2) / len(stack)
+    with ep.DecodeAhead(stack, group_size=16) as ahead:
+        same = bool(torch.equal(forward(), reference))
+        ahead_ms = _median_ms(forward, max(3, steps // 5), warmup=2) / len(stack)
+        ahead.check_errors()
+    out["stack_of_32"] = {"layer_by_layer_ms_per_layer": round(alone, 5), "decode_ahead_group_16_ms_per_layer": round(ahead_ms, 5),
+                          "tops": round(ops / ahead_ms / 1e9, 2), "frac_of_int8_mfma_peak": round(ops / ahead_ms / 1e9 / MFMA_PEAK_INT8_TOPS, 5),
+                          "identical_to_layer_by_layer": same}
     return out
 
 
