@@ -93,9 +93,11 @@ def test_dit_like_wide_and_tall_shapes(shape):
     decode_and_check(gauss(3, *shape), target_bpp=4.0)
 
 
-@pytest.mark.parametrize("shape", [(1, 8), (3, 8), (1000, 8), (5, 16), (7, 200), (33, 1001), (2, 29120), (64, 14560), (1, 232960)])
+@pytest.mark.parametrize("shape", [(1, 8), (3, 8), (1000, 8), (5, 16), (7, 200), (33, 1001), (2, 29120), (64, 14560), (1, 232960),
+                                   (20000, 8), (5000, 40), (700, 264)])
 def test_edge_shapes(shape):
-    """One-vector rows, padded columns, single short tile, rows that are exactly one or sixteen tiles long."""
+    """One-vector rows, padded columns, single short tile, rows that are exactly one or sixteen tiles long; full tiles
+    whose 32-vector groups span many rows (rows of 1, 5 and 33 vectors)."""
     print("case", shape, flush=True)
     decode_and_check(gauss(21, *shape, sigma=1.0), kinds=ALL_KINDS, target_bpp=4.0)
 
@@ -114,6 +116,45 @@ def test_tiles_beyond_the_lds_kernels_take_the_global_tables():
     container, used = decode_and_check(gauss(24, 640, 4096), kinds=(None, hip_backend.TABLE_LDS_BYTE), target_bpp=4.0,
                                        tile_elements=(9 << 18) + 9)
     assert used == ["global64"]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16, torch.int8])
+def test_rows_with_unusual_scales_take_the_literal_formula(dtype):
+    """Row scales that are zero, negative, subnormal, tiny or near the top of the float range (no encoder makes them,
+    a container may hold them) must give the reference's (z + c / 2) * scale, then its container cast, bit for bit:
+    the kernels' fused multiply-add is only used for ordinary scales. Ordinary and unusual rows alternate, so both
+    forms run inside one tile, in whole groups and in a tile's short first group."""
+    container = ep.compress(gauss(25, 96, 512), ep.EntroPackLossyConfig(target_bpp=4.0, execution_backend="eager"))
+    odd = [0.0, -0.0, -0.02, 1e-41, 3e-39, 1e-31, 9e-31, 2e30, 7e36, 3e38, -3e38]
+    scales = container.buffers["scales"].clone()
+    for row in range(0, scales.numel(), 2):
+        scales[row] = odd[(row // 2) % len(odd)]
+    buffers = dict(container.buffers)
+    buffers["scales"] = scales
+    host = host_buffers(container)
+    host["scales"] = scales.numpy()
+    name = str(dtype).removeprefix("torch.")
+    expect = c_oracle.decode(host, (96, 512), name, threads=4)
+    for kind in ALL_KINDS:
+        hip_lane.FORCE_TABLE_KIND = kind
+        try:
+            lattice = LatticeBuffers(**{k: v.cuda() for k, v in buffers.items()})
+            got = hip_lane.decode(lattice, shape=(96, 512), dtype=dtype)
+        except hip_backend.HipError as error:
+            if error.status == hip_backend.EUNSUPPORTED:
+                continue
+            raise
+        finally:
+            hip_lane.FORCE_TABLE_KIND = None
+        torch.cuda.synchronize()
+        hip_lane.check_errors(lattice)
+        if dtype in (torch.bfloat16, torch.float16):                 # the oracle returns their bit patterns
+            got, reference = got.view(torch.int16).cpu().numpy().view(np.uint16), expect
+        elif dtype == torch.float32:
+            got, reference = got.cpu().numpy().view(np.int32), expect.view(np.int32)
+        else:
+            got, reference = got.cpu().numpy(), expect
+        assert np.array_equal(got, reference), f"kind {kind}"
 
 
 def test_constant_and_zero_tensors():
