@@ -129,9 +129,27 @@ __device__ __forceinline__ void store_vector(void* out, int kind, int64_t vector
       break;
     }
     case EP_STORE_F16: {
+      // Saturation to the largest finite half is needed by very few vectors: one magnitude test for all eight
+      // values, then packed round-to-nearest-even conversions.
+      float v[8];
+      float top = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        v[i] = w[i];
+        top = __builtin_fmaxf(top, __builtin_fabsf(w[i]));
+      }
+      if (__builtin_expect(top > 65504.0f, 0)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __builtin_fminf(__builtin_fmaxf(w[i], -65504.0f), 65504.0f);
+      }
       uint32_t p[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p[i] = f16_bits(w[2 * i]) | (f16_bits(w[2 * i + 1]) << 16);
+      for (int i = 0; i < 4; ++i) {
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        const float2v two = {v[2 * i], v[2 * i + 1]};
+        p[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(two, half2v));
+      }
       stream_store16(reinterpret_cast<uint4*>(out) + vector, p[0], p[1], p[2], p[3]);
       break;
     }
