@@ -99,9 +99,18 @@ __device__ __forceinline__ void stream_store8(void* at, uint32_t a, uint32_t b) 
 __device__ __forceinline__ void store_vector_i8(void* out, int64_t vector, const float (&w)[8]) {
   float magic = 12582912.0f;
   asm volatile("" : "+v"(magic));          // a vector register: the sub-dword form takes no literal
+  // Few vectors hold a value outside [-128, 127]: one magnitude test for all eight instead of eight clamps.
   float c[8];
+  float top = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) c[i] = __builtin_fminf(__builtin_fmaxf(w[i], -128.0f), 127.0f);
+  for (int i = 0; i < 8; ++i) {
+    c[i] = w[i];
+    top = __builtin_fmaxf(top, __builtin_fabsf(w[i]));
+  }
+  if (__builtin_expect(top > 127.0f, 0)) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = __builtin_fminf(__builtin_fmaxf(w[i], -128.0f), 127.0f);
+  }
   uint32_t low, high;
   // The two words alternate: an instruction that keeps the other bytes of its destination must not directly follow
   // the one that wrote them (sub-dword writes need one instruction in between on this hardware).
