@@ -88,6 +88,30 @@ def test_quantize_rows_is_exact(rows, inner, dtype):
     assert codes[0].abs().max() == 0
 
 
+def test_quantize_rows_is_exact_next_to_rounding_boundaries():
+    """Quotients within a few units in the last place of k + 1/2, on both sides, for scales that are not powers of
+    two: where multiplying by a reciprocal and dividing can round to different integers. The kernel must give the
+    division's answer everywhere."""
+    torch.manual_seed(17)
+    rows, inner = 64, 2048
+    top = (torch.rand(rows, dtype=torch.float64) * 900 + 0.37)                      # row maxima, so scale = top / 127
+    scale = (top.float() / torch.tensor(127.0)).double()
+    k = torch.randint(-126, 126, (rows, inner)).double() + 0.5
+    nudge = torch.randint(-3, 4, (rows, inner)).double() * 2.0 ** -23                  # relative: a few ulps either way
+    x = (k * scale.unsqueeze(1) * (1.0 + nudge)).float()
+    x[:, 0] = top.float()                                                              # pins each row's maximum
+    x = x.cuda()
+    codes, got_scale = kernels.quantize_rows(x)
+    flat = x.cpu()
+    expect_scale = (flat.abs().amax(dim=1) / torch.tensor(127.0)).clamp(min=torch.finfo(torch.float32).eps)
+    expect_codes = (flat / expect_scale.unsqueeze(1)).round().clamp(-127, 127).to(torch.int8)
+    assert torch.equal(got_scale.cpu(), expect_scale)
+    assert torch.equal(codes.cpu(), expect_codes)
+    # the construction does what it says: a reciprocal multiply alone gets some of these wrong
+    naive = (flat * (1.0 / expect_scale).unsqueeze(1)).round().clamp(-127, 127).to(torch.int8)
+    assert (naive != expect_codes).any()
+
+
 @pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040), (4100, 4200, 528), (1, 300, 4112), (128, 1000, 28672),
                                    (33, 257, 16), (4096, 3000, 272)])
 def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
