@@ -304,7 +304,7 @@ __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepCo
 // freq | cdf << 16; its value (symbol + minimum, int16) is read off the critical path. The lookups are ordinary C++;
 // renormalisation is the same scalar vote as above.
 template <int PB, bool MASKED>
-__device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, uint32_t val0, const StepConsts& k,
+__device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_group, uint32_t val0, const StepConsts& k,
                                           bool valid_lane) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   typedef __attribute__((address_space(3))) const u32x2* lds_u2;
@@ -313,8 +313,11 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_base, 
   constexpr uint32_t kTable = 1u << PB;
   const uint32_t x = p.x;
   const uint32_t slot = x & (kTable - 1u);
-  const uint32_t word_at = (((x >> 5) & (kTable / 32u - 1u)) << 3) + rs_base;
-  const u32x2 rs = *reinterpret_cast<lds_u2>(static_cast<uintptr_t>(word_at));
+  // rs_group = the LDS address of field 0's words for this lane's coset, a multiple of one stream's size: the word
+  // offset is OR-ed in, and the field's distance is a constant the read takes as its immediate offset.
+  constexpr uint32_t kStreamBytes = (kTable / 32u) * 8u;
+  const uint32_t word_at = ((x >> 2) & (kStreamBytes - 8u)) | rs_group;
+  const u32x2 rs = *reinterpret_cast<lds_u2>(static_cast<uintptr_t>(word_at + static_cast<uint32_t>(2 * field) * kStreamBytes));
   // The bit-field extract takes its width from the low five bits of x: the bits of rs.x below slot % 32.
   const uint32_t index = static_cast<uint32_t>(__builtin_popcount(__builtin_amdgcn_ubfe(rs.x, 0u, x))) + rs.y;
   const uint32_t fb = *reinterpret_cast<lds_u32>(static_cast<uintptr_t>(index << 2));
@@ -725,11 +728,11 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
 #pragma unroll
       for (int j = 0; j < ILP; ++j) high[j] = st[j].coset_base + L::kHighBase;
       const uint32_t slot_base = MODE == kModeSym ? sym_slot_base(st[0]) : 0u;
+      const uint32_t rank_group = st[0].coset_base + rank_rs0;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
-          rank_step<PB, MASKED>(st[0], f, st[0].coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)),
-                                rank_val0, k, valid_lane);
+          rank_step<PB, MASKED>(st[0], f, rank_group, rank_val0, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
           sym_step<PB, MASKED>(st[0], f, slot_base, k, valid_lane);
         } else if constexpr (ILP == 2) {
@@ -845,8 +848,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
-          rank_step<PB, true>(s, f, s.coset_base + (rank_rs0 + static_cast<uint32_t>(2 * f) * ((L::kTable / 32u) * 8u)), rank_val0, k,
-                              valid_lane);
+          rank_step<PB, true>(s, f, s.coset_base + rank_rs0, rank_val0, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
           sym_step<PB, true>(s, f, slot_base, k, valid_lane);
         } else {
