@@ -410,82 +410,166 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
   const int frag_row = lane & 31;
   const int frag_k = (lane >> 5) * 16;
 
-  // Per operand tile: 256 rows of 8 chunks of 16 bytes; thread t moves chunks t, t + 512, ..., 4 per operand.
-  uint4 reg_a[4], reg_b[B_CHUNKS];
-  auto fetch = [&](int64_t kb) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int chunk = tid + kBigThreads * i;
-      const int r = chunk >> 3;
-      const int64_t at = kb + 16 * (chunk & 7);
-      reg_a[i] = make_uint4(0, 0, 0, 0);
-      if (!GUARD || (m0 + r < M && at < k_bytes)) reg_a[i] = *reinterpret_cast<const uint4*>(a + (m0 + r) * lda_bytes + at);
-    }
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      const int chunk = tid + kBigThreads * i;
-      const int r = chunk >> 3;
-      const int64_t at = kb + 16 * (chunk & 7);
-      reg_b[i] = make_uint4(0, 0, 0, 0);
-      if (!GUARD || (n0 + r < N && at < k_bytes)) reg_b[i] = *reinterpret_cast<const uint4*>(b + (n0 + r) * ldb_bytes + at);
-    }
+  // Per operand tile: rows of 8 pieces of 16 bytes; thread t moves pieces t, t + 512, ...: 4 of A, then B_CHUNKS of B.
+  constexpr int kMoves = 4 + B_CHUNKS;
+  uint4 staged[kMoves];
+  auto fetch_one = [&](int64_t kb, int c) {
+    const bool of_a = c < 4;
+    const int chunk = tid + kBigThreads * (of_a ? c : c - 4);
+    const int r = (of_a ? m0 : n0) + (chunk >> 3);
+    const int64_t at = kb + 16 * (chunk & 7);
+    const uint8_t* from = of_a ? a + r * lda_bytes + at : b + r * ldb_bytes + at;
+    staged[c] = make_uint4(0, 0, 0, 0);
+    if (!GUARD || (r < (of_a ? M : N) && at < k_bytes)) staged[c] = *reinterpret_cast<const uint4*>(from);
   };
-  auto stash = [&](int stage) {
-    uint8_t* tile_a = big_smem + stage * kStageBytes;
-    uint8_t* tile_b = tile_a + kBigM * kRowStride;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int chunk = tid + kBigThreads * i;
-      *reinterpret_cast<uint4*>(tile_a + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = reg_a[i];
-    }
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      const int chunk = tid + kBigThreads * i;
-      *reinterpret_cast<uint4*>(tile_b + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = reg_b[i];
-    }
+  auto stash_one = [&](int stage, int c) {
+    const bool of_a = c < 4;
+    const int chunk = tid + kBigThreads * (of_a ? c : c - 4);
+    uint8_t* tile = big_smem + stage * kStageBytes + (of_a ? 0 : kBigM * kRowStride);
+    *reinterpret_cast<uint4*>(tile + (chunk >> 3) * kRowStride + 16 * (chunk & 7)) = staged[c];
   };
 
   using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
+  using Frag = typename std::conditional<INT8, i32x4, bf16x8>::type;
   Acc acc[2][NJ] = {};
+  // Fragments of one 32-byte slice of K, held twice: while the matrix cores work through one set, the LDS reads of the
+  // next slice are under way, across the barrier between two K steps as well.
+  constexpr int kReads = 2 + NJ, kMultiplies = 2 * NJ;
+  Frag frag[2][kReads];
+  const uint32_t frag_a_at = static_cast<uint32_t>((wave_m * 64 + frag_row) * kRowStride + frag_k);
+  const uint32_t frag_b_at = static_cast<uint32_t>((kBigM + wave_n * WN + frag_row) * kRowStride + frag_k);
+  auto read_one = [&](int set, int stage, int kk, int t) {
+    const uint32_t at = stage * kStageBytes + kk * 32 + (t < 2 ? frag_a_at + t * 32 * kRowStride : frag_b_at + (t - 2) * 32 * kRowStride);
+    frag[set][t] = *reinterpret_cast<const Frag*>(big_smem + at);
+  };
+  auto multiply_one = [&](int set, int m) {
+    const int i = m / NJ, j = m % NJ;
+    if constexpr (INT8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+    else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+  };
+
   const int64_t steps = (k_bytes + kTileBytesK - 1) / kTileBytesK;
-  fetch(0);
-  stash(0);
+#pragma unroll
+  for (int c = 0; c < kMoves; ++c) fetch_one(0, c);
+#pragma unroll
+  for (int c = 0; c < kMoves; ++c) stash_one(0, c);
   __syncthreads();
-  if (steps > 1) fetch(kTileBytesK);
+  // Same order as in the loop (the pieces beyond one per multiply first): the stores there wait for the loads one by one.
+#pragma unroll
+  for (int c = kMultiplies; c < kMoves; ++c) fetch_one(steps > 1 ? kTileBytesK : 0, c);
+#pragma unroll
+  for (int c = 0; c < kMoves && c < kMultiplies; ++c) fetch_one(steps > 1 ? kTileBytesK : 0, c);
+#pragma unroll
+  for (int t = 0; t < kReads; ++t) read_one(0, 0, 0, t);
+  // One K step = four slices. Every multiply is followed by at most two memory operations and the order is pinned, so
+  // that the LDS port and the matrix cores work at the same time instead of taking turns: during slice 0 the tile held
+  // in registers goes to the other LDS stage, during slice 1 the loads of the tile after it are issued, and each slice
+  // reads the fragments of the next one. Past the last tile the stores and loads repeat work that nobody reads (the
+  // idle stage, the last tile again), which keeps the loop body one straight line.
   for (int64_t step = 0; step < steps; ++step) {
     const int stage = static_cast<int>(step & 1);
-    if (step + 1 < steps) stash(stage ^ 1);
-    if (step + 2 < steps) fetch((step + 2) * kTileBytesK);
-    const uint8_t* tile_a = big_smem + stage * kStageBytes + (wave_m * 64 + frag_row) * kRowStride + frag_k;
-    const uint8_t* tile_b = big_smem + stage * kStageBytes + (kBigM + wave_n * WN + frag_row) * kRowStride + frag_k;
+    const int64_t ahead = (step + 2 < steps ? step + 2 : steps - 1) * kTileBytesK;
 #pragma unroll
-    for (int kk = 0; kk < kTileBytesK / 32; ++kk) {
-      if constexpr (INT8) {
-        i32x4 fa[2], fb[NJ];
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(0, m);
+      if (kMultiplies + m < kMoves) stash_one(stage ^ 1, kMultiplies + m);
+      if (m < kMoves) stash_one(stage ^ 1, m);
+      if (m < kReads) read_one(1, stage, 1, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
-        for (int t = 0; t < 2; ++t) fa[t] = *reinterpret_cast<const i32x4*>(tile_a + t * 32 * kRowStride + kk * 32);
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(1, m);
+      if (kMultiplies + m < kMoves) fetch_one(ahead, kMultiplies + m);
+      if (m < kMoves) fetch_one(ahead, m);
+      if (m < kReads) read_one(0, stage, 2, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
-        for (int t = 0; t < NJ; ++t) fb[t] = *reinterpret_cast<const i32x4*>(tile_b + t * 32 * kRowStride + kk * 32);
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      } else {
-        bf16x8 fa[2], fb[NJ];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) fa[t] = *reinterpret_cast<const bf16x8*>(tile_a + t * 32 * kRowStride + kk * 32);
-#pragma unroll
-        for (int t = 0; t < NJ; ++t) fb[t] = *reinterpret_cast<const bf16x8*>(tile_b + t * 32 * kRowStride + kk * 32);
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      }
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(0, m);
+      if (m < kReads) read_one(1, stage, 3, m);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
+#pragma unroll
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(1, m);
+      if (m < kReads) read_one(0, stage ^ 1, 0, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 
   // Accumulator layout of a 32 x 32 tile: register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
+  // One lane therefore owns single elements of many rows. Written out as they lie that is 16 * NJ two-byte stores per
+  // lane and half tile, each instruction touching two 64-byte row pieces, and the stores then cost more than a fifth of
+  // a 4096 x 3072 x 3072 product. When the output allows 16-byte stores, each wave instead passes its half tile (32 rows
+  // x WN columns, as f32 after scales and bias) through a private slab of the LDS the tiles no longer need and stores
+  // whole row pieces, 16 bytes per lane. The arithmetic and the rounding are those of the element-wise path.
+  const int out_bytes = out_kind == kOutF32 ? 4 : 2;
+  const bool wide_rows = !GUARD && ((reinterpret_cast<uintptr_t>(y) | static_cast<uintptr_t>(ldy * out_bytes)) & 15u) == 0;
+  if (wide_rows) {
+    constexpr int kPitch = WN + 8;                          // dwords; rows 4 apart (the two lane halves) land on the other 32 banks
+    static_assert(8 * 32 * kPitch * 4 <= 2 * kStageBytes, "the eight slabs fit into the two tile stages");
+    float* slab = reinterpret_cast<float*>(big_smem) + wave * (32 * kPitch);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int n = n0 + wave_n * WN + j * 32 + (lane & 31);
+        const bool has_bias = bias != nullptr;
+        const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
+        float sb = 1.0f;
+        if constexpr (INT8) sb = scale_b[n];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+          float v;
+          if constexpr (INT8) {
+            v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[m0 + wave_m * 64 + i * 32 + row]), sb);
+            if (has_bias) v = __fadd_rn(v, bv);
+          } else {
+            v = acc[i][j][r] + bv;
+          }
+          slab[row * kPitch + j * 32 + (lane & 31)] = v;
+        }
+      }
+      const int64_t first = static_cast<int64_t>(m0 + wave_m * 64 + i * 32) * ldy + n0 + wave_n * WN;
+      if (out_kind == kOutF32) {
+        constexpr int kPieces = WN / 4;                     // 16-byte pieces per row
+        float* out = reinterpret_cast<float*>(y) + first;
+#pragma unroll
+        for (int at = 0; at < 32 * kPieces; at += 64) {
+          const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
+          *reinterpret_cast<uint4*>(out + row * ldy + 4 * piece) = *reinterpret_cast<const uint4*>(slab + row * kPitch + 4 * piece);
+        }
+      } else {
+        constexpr int kPieces = WN / 8;
+        uint16_t* out = reinterpret_cast<uint16_t*>(y) + first;
+#pragma unroll
+        for (int at = 0; at < 32 * kPieces; at += 64) {
+          const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
+          const float4 lo = *reinterpret_cast<const float4*>(slab + row * kPitch + 8 * piece);
+          const float4 hi = *reinterpret_cast<const float4*>(slab + row * kPitch + 8 * piece + 4);
+          uint4 packed;
+          if (out_kind == kOutBF16) {
+            packed.x = bf16_bits_of(lo.x) | bf16_bits_of(lo.y) << 16;
+            packed.y = bf16_bits_of(lo.z) | bf16_bits_of(lo.w) << 16;
+            packed.z = bf16_bits_of(hi.x) | bf16_bits_of(hi.y) << 16;
+            packed.w = bf16_bits_of(hi.z) | bf16_bits_of(hi.w) << 16;
+          } else {
+            auto half_bits = [](float v) { return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(v))); };
+            packed.x = half_bits(lo.x) | half_bits(lo.y) << 16;
+            packed.y = half_bits(lo.z) | half_bits(lo.w) << 16;
+            packed.z = half_bits(hi.x) | half_bits(hi.y) << 16;
+            packed.w = half_bits(hi.z) | half_bits(hi.w) << 16;
+          }
+          *reinterpret_cast<uint4*>(out + row * ldy + 8 * piece) = packed;
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
 #pragma unroll
