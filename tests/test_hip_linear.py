@@ -54,6 +54,32 @@ def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
         assert rel_l2(got, expect) <= REL_L2
     as_f32 = kernels.gemm_bf16(x, w, b, out_dtype=torch.float32)
     assert rel_l2(as_f32, expect) <= 1e-5
+    # Every output kind is one rounding of the same f32 sums, whichever way the kernel's epilogue writes them out.
+    assert torch.equal(got, as_f32.to(torch.bfloat16))
+    half_bias = None if b is None else b.to(torch.float16)
+    as_f16 = kernels.gemm_bf16(x, w, half_bias, out_dtype=torch.float16)
+    assert torch.equal(as_f16, kernels.gemm_bf16(x, w, half_bias, out_dtype=torch.float32).to(torch.float16))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_gemm_output_rows_that_are_not_16_byte_aligned(out_dtype):
+    """The 256-row kernel stores whole row pieces of 16 bytes when the output allows it; an output whose rows do not
+    start on 16-byte boundaries (here: a view with an odd row stride) takes the element-wise stores and must give the
+    same bits."""
+    from entropack_amd.backends import hip
+    m, n, k = 4096, 3072, 256
+    torch.manual_seed(6)
+    x = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(n, k, device="cuda") * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(n, device="cuda") * 0.01).to(out_dtype)
+    expect = kernels.gemm_bf16(x, w, bias, out_dtype=out_dtype)
+    padded = torch.full((m, n + 1), 7.0, dtype=out_dtype, device="cuda")
+    hip.check("ep_hip_gemm_bf16", hip.library().ep_hip_gemm_bf16(
+        x.data_ptr(), w.data_ptr(), bias.data_ptr(), padded.data_ptr(), m, n, k, x.stride(0), w.stride(0), padded.stride(0),
+        hip.FLOAT_KINDS[out_dtype], hip.current_stream(x.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(padded[:, :n], expect)
+    assert bool((padded[:, n] == 7.0).all())
 
 
 def test_gemm_bf16_takes_strided_rows_and_batches():
