@@ -381,6 +381,113 @@ __global__ __launch_bounds__(256) void rotate_quantize_rows_kernel(const void* _
 }
 
 
+// Writes one wave's 64 x 32 NJ accumulator tile: acc[i][j] is the 32 x 32 tile at rows 32 i, columns 32 j of it.
+// Accumulator layout of a 32 x 32 tile: register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
+// One lane therefore owns single elements of many rows. Written out as they lie that is 16 NJ two-byte stores per
+// lane and half tile, each instruction touching two 64-byte row pieces, and the stores then cost more than a fifth of
+// a 4096 x 3072 x 3072 product. When the output allows 16-byte stores, the wave instead passes each half tile (32 rows
+// x 32 NJ columns, as f32 after scales and bias) through `slab`, LDS private to it that the tiles no longer need, and
+// stores whole row pieces, 16 bytes per lane. In the slab, rows with bit 2 set keep their columns rotated by 32: the
+// two lane halves of an accumulator register (rows 4 apart) then write to different banks. The arithmetic and the
+// rounding are those of the element-wise path, which ragged products and outputs with unaligned rows take.
+template <bool INT8, bool GUARD, int NJ, typename Acc>
+__device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, const float* __restrict__ scale_a,
+                                                const float* __restrict__ scale_b, const void* __restrict__ bias,
+                                                void* __restrict__ y, int M, int N, int64_t ldy, int out_kind, int row0, int col0,
+                                                int lane) {
+  constexpr int WN = 32 * NJ;
+  auto slab_at = [](int row, int col) { const int c = col + ((row & 4) << 3); return row * WN + (c >= WN ? c - WN : c); };
+  const int out_bytes = out_kind == kOutF32 ? 4 : 2;
+  const bool wide_rows = !GUARD && ((reinterpret_cast<uintptr_t>(y) | static_cast<uintptr_t>(ldy * out_bytes)) & 15u) == 0;
+  if (wide_rows) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int n = col0 + j * 32 + (lane & 31);
+        const bool has_bias = bias != nullptr;
+        const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
+        float sb = 1.0f;
+        if constexpr (INT8) sb = scale_b[n];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+          float v;
+          if constexpr (INT8) {
+            v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[row0 + i * 32 + row]), sb);
+            if (has_bias) v = __fadd_rn(v, bv);
+          } else {
+            v = acc[i][j][r] + bv;
+          }
+          slab[slab_at(row, j * 32 + (lane & 31))] = v;
+        }
+      }
+      const int64_t first = static_cast<int64_t>(row0 + i * 32) * ldy + col0;
+      if (out_kind == kOutF32) {
+        constexpr int kPieces = WN / 4;                     // 16-byte pieces per row
+        float* out = reinterpret_cast<float*>(y) + first;
+#pragma unroll
+        for (int at = 0; at < 32 * kPieces; at += 64) {
+          const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
+          *reinterpret_cast<uint4*>(out + row * ldy + 4 * piece) =
+              *reinterpret_cast<const uint4*>(slab + slab_at(row, 4 * piece));
+        }
+      } else {
+        constexpr int kPieces = WN / 8;
+        uint16_t* out = reinterpret_cast<uint16_t*>(y) + first;
+#pragma unroll
+        for (int at = 0; at < 32 * kPieces; at += 64) {
+          const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
+          const float* from = slab + slab_at(row, 8 * piece);
+          const float4 lo = *reinterpret_cast<const float4*>(from);
+          const float4 hi = *reinterpret_cast<const float4*>(from + 4);
+          uint4 packed;
+          if (out_kind == kOutBF16) {
+            packed.x = bf16_bits_of(lo.x) | bf16_bits_of(lo.y) << 16;
+            packed.y = bf16_bits_of(lo.z) | bf16_bits_of(lo.w) << 16;
+            packed.z = bf16_bits_of(hi.x) | bf16_bits_of(hi.y) << 16;
+            packed.w = bf16_bits_of(hi.z) | bf16_bits_of(hi.w) << 16;
+          } else {
+            auto half_bits = [](float v) { return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(v))); };
+            packed.x = half_bits(lo.x) | half_bits(lo.y) << 16;
+            packed.y = half_bits(lo.z) | half_bits(lo.w) << 16;
+            packed.z = half_bits(hi.x) | half_bits(hi.y) << 16;
+            packed.w = half_bits(hi.z) | half_bits(hi.w) << 16;
+          }
+          *reinterpret_cast<uint4*>(out + row * ldy + 8 * piece) = packed;
+        }
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int n = col0 + j * 32 + (lane & 31);
+      if (n >= N) continue;
+      const bool has_bias = bias != nullptr;
+      const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
+      float sb = 1.0f;
+      if constexpr (INT8) sb = scale_b[n];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = row0 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+        if (m >= M) continue;
+        float v;
+        if constexpr (INT8) {
+          // int32 -> f32, times the activation row scale, times the weight row scale, plus bias: each one rounded operation.
+          v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[m]), sb);
+          if (has_bias) v = __fadd_rn(v, bv);
+        } else {
+          v = acc[i][j][r] + bv;
+        }
+        store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, v);
+      }
+    }
+  }
+}
+
 // ---- large products: 256 x 256 block tiles ----------------------------------------------------------------------------------
 //
 // With 64 x 64 per wave (above) every matrix-core instruction needs one 16-byte LDS read per lane and the LDS port, not
@@ -500,102 +607,129 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
     }
   }
 
-  // Accumulator layout of a 32 x 32 tile: register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
-  // One lane therefore owns single elements of many rows. Written out as they lie that is 16 * NJ two-byte stores per
-  // lane and half tile, each instruction touching two 64-byte row pieces, and the stores then cost more than a fifth of
-  // a 4096 x 3072 x 3072 product. When the output allows 16-byte stores, each wave instead passes its half tile (32 rows
-  // x WN columns, as f32 after scales and bias) through a private slab of the LDS the tiles no longer need and stores
-  // whole row pieces, 16 bytes per lane. The arithmetic and the rounding are those of the element-wise path.
-  const int out_bytes = out_kind == kOutF32 ? 4 : 2;
-  const bool wide_rows = !GUARD && ((reinterpret_cast<uintptr_t>(y) | static_cast<uintptr_t>(ldy * out_bytes)) & 15u) == 0;
-  if (wide_rows) {
-    constexpr int kPitch = WN + 8;                          // dwords; rows 4 apart (the two lane halves) land on the other 32 banks
-    static_assert(8 * 32 * kPitch * 4 <= 2 * kStageBytes, "the eight slabs fit into the two tile stages");
-    float* slab = reinterpret_cast<float*>(big_smem) + wave * (32 * kPitch);
+  static_assert(8 * 32 * WN * 4 <= 2 * kStageBytes, "the eight slabs fit into the two tile stages");
+  store_wave_tile<INT8, GUARD, NJ>(acc, reinterpret_cast<float*>(big_smem) + wave * (32 * WN), scale_a, scale_b, bias, y, M, N, ldy, out_kind,
+                                   m0 + wave_m * 64, n0 + wave_n * WN, lane);
+}
+
+// ---- the same block tile with the operand tiles loaded straight into LDS ----------------------------------------------------
+//
+// For whole tiles (M, N multiples of the block tile, K of one tile step). The kernel above moves every tile byte
+// memory -> registers -> LDS, and that round trip (seven 16-byte loads and seven LDS stores per wave and K step) is what
+// keeps it a third above the matrix cores' own time. Here `global_load_lds_dwordx4` writes the loaded bytes into LDS
+// itself: one instruction fills 1 KiB of consecutive LDS (lane l the 16 bytes at 16 l), i.e. eight tile rows of 128
+// bytes. Rows therefore cannot be padded; instead row r keeps its eight 16-byte pieces permuted, piece c at place
+// c ^ ((r >> 1) & 7), which each lane arranges by choosing the global address it loads from. Sixteen consecutive rows
+// read at the same logical piece then cover all 64 banks once. The two stages are two separate arrays and the K loop
+// is written out for both parities, so that every LDS access names its array: the compiler then waits for loads in
+// flight only where an access may touch the array they fill (before the barrier that publishes it), not before the
+// fragment reads of the other stage.
+template <bool INT8, int BN>
+__global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                             const float* __restrict__ scale_a, const float* __restrict__ scale_b,
+                                                             const void* __restrict__ bias, void* __restrict__ y, int M, int N,
+                                                             int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy,
+                                                             int out_kind) {
+  constexpr int kRowBytes = kTileBytesK;                    // 128, unpadded
+  constexpr int kStage = (kBigM + BN) * kRowBytes;
+  __shared__ __align__(1024) uint8_t stage0[kStage];
+  __shared__ __align__(1024) uint8_t stage1[kStage];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int WN = BN / 2, NJ = WN / 32;
+  constexpr int kLoadsA = kBigM / 64, kLoadsB = BN / 64, kLoads = kLoadsA + kLoadsB;   // 1 KiB pieces per wave and tile: 4 + 3 or 4
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int m0 = blockIdx.y * kBigM, n0 = blockIdx.x * BN;
+
+  // Load c of this wave fills tile rows 8 (wave + 8 c') .. + 8 of A (c < kLoadsA, c' = c) or of B (c' = c - kLoadsA).
+  const uint8_t* source[kLoads];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const int n = n0 + wave_n * WN + j * 32 + (lane & 31);
-        const bool has_bias = bias != nullptr;
-        const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
-        float sb = 1.0f;
-        if constexpr (INT8) sb = scale_b[n];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-          float v;
-          if constexpr (INT8) {
-            v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[m0 + wave_m * 64 + i * 32 + row]), sb);
-            if (has_bias) v = __fadd_rn(v, bv);
-          } else {
-            v = acc[i][j][r] + bv;
-          }
-          slab[row * kPitch + j * 32 + (lane & 31)] = v;
-        }
-      }
-      const int64_t first = static_cast<int64_t>(m0 + wave_m * 64 + i * 32) * ldy + n0 + wave_n * WN;
-      if (out_kind == kOutF32) {
-        constexpr int kPieces = WN / 4;                     // 16-byte pieces per row
-        float* out = reinterpret_cast<float*>(y) + first;
-#pragma unroll
-        for (int at = 0; at < 32 * kPieces; at += 64) {
-          const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
-          *reinterpret_cast<uint4*>(out + row * ldy + 4 * piece) = *reinterpret_cast<const uint4*>(slab + row * kPitch + 4 * piece);
-        }
-      } else {
-        constexpr int kPieces = WN / 8;
-        uint16_t* out = reinterpret_cast<uint16_t*>(y) + first;
-#pragma unroll
-        for (int at = 0; at < 32 * kPieces; at += 64) {
-          const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
-          const float4 lo = *reinterpret_cast<const float4*>(slab + row * kPitch + 8 * piece);
-          const float4 hi = *reinterpret_cast<const float4*>(slab + row * kPitch + 8 * piece + 4);
-          uint4 packed;
-          if (out_kind == kOutBF16) {
-            packed.x = bf16_bits_of(lo.x) | bf16_bits_of(lo.y) << 16;
-            packed.y = bf16_bits_of(lo.z) | bf16_bits_of(lo.w) << 16;
-            packed.z = bf16_bits_of(hi.x) | bf16_bits_of(hi.y) << 16;
-            packed.w = bf16_bits_of(hi.z) | bf16_bits_of(hi.w) << 16;
-          } else {
-            auto half_bits = [](float v) { return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(v))); };
-            packed.x = half_bits(lo.x) | half_bits(lo.y) << 16;
-            packed.y = half_bits(lo.z) | half_bits(lo.w) << 16;
-            packed.z = half_bits(hi.x) | half_bits(hi.y) << 16;
-            packed.w = half_bits(hi.z) | half_bits(hi.w) << 16;
-          }
-          *reinterpret_cast<uint4*>(out + row * ldy + 8 * piece) = packed;
-        }
-      }
-    }
-    return;
+  for (int c = 0; c < kLoads; ++c) {
+    const bool of_a = c < kLoadsA;
+    const int row = 8 * (wave + 8 * (of_a ? c : c - kLoadsA)) + (lane >> 3);
+    const int piece = (lane & 7) ^ ((row >> 1) & 7);
+    source[c] = of_a ? a + (m0 + row) * lda_bytes + 16 * piece : b + (n0 + row) * ldb_bytes + 16 * piece;
   }
+  auto load_one = [&](uint8_t* stage, int64_t kb, int c) {
+    const bool of_a = c < kLoadsA;
+    const int first_row = (of_a ? 0 : kBigM) + 8 * (wave + 8 * (of_a ? c : c - kLoadsA));
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(source[c] + kb),
+                                     (__attribute__((address_space(3))) void*)(stage + first_row * kRowBytes), 16, 0, 0);
+  };
+
+  using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
+  using Frag = typename std::conditional<INT8, i32x4, bf16x8>::type;
+  Acc acc[2][NJ] = {};
+  constexpr int kReads = 2 + NJ, kMultiplies = 2 * NJ;
+  Frag frag[2][kReads];
+  const int frag_row = lane & 31;
+  const int turn = (frag_row >> 1) & 7;                      // the same for rows 32 apart
+  const uint32_t frag_a_at = static_cast<uint32_t>((wave_m * 64 + frag_row) * kRowBytes);
+  const uint32_t frag_b_at = static_cast<uint32_t>((kBigM + wave_n * WN + frag_row) * kRowBytes);
+  auto read_one = [&](int set, const uint8_t* stage, int kk, int t) {
+    const uint32_t place = static_cast<uint32_t>(((2 * kk + (lane >> 5)) ^ turn) * 16);
+    const uint32_t at = place + (t < 2 ? frag_a_at + t * 32 * kRowBytes : frag_b_at + (t - 2) * 32 * kRowBytes);
+    frag[set][t] = *reinterpret_cast<const Frag*>(stage + at);
+  };
+  auto multiply_one = [&](int set, int m) {
+    const int i = m / NJ, j = m % NJ;
+    if constexpr (INT8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+    else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+  };
+
+  const int64_t steps = k_bytes / kTileBytesK;
+  auto tile_at = [&](int64_t t) { return (t < steps ? t : steps - 1) * kTileBytesK; };
+  // One K step on the stage `here` while `there` is filled. The A pieces of a tile are requested right after the barrier
+  // that frees their stage (the last slice of the step before), the B pieces during the first slice of this step, so
+  // every load has most of a step to land before the barrier that publishes the stage. Past the last tile the loads
+  // repeat the last one, which nobody reads.
+  auto k_step = [&](uint8_t* here, uint8_t* there, int64_t step) {
+    const int64_t next = tile_at(step + 1), second = tile_at(step + 2);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int n = n0 + wave_n * WN + j * 32 + (lane & 31);
-      if (n >= N) continue;
-      const bool has_bias = bias != nullptr;
-      const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
-      float sb = 1.0f;
-      if constexpr (INT8) sb = scale_b[n];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wave_m * 64 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-        if (m >= M) continue;
-        float v;
-        if constexpr (INT8) {
-          // int32 -> f32, times the activation row scale, times the weight row scale, plus bias: each one rounded operation.
-          v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[m]), sb);
-          if (has_bias) v = __fadd_rn(v, bv);
-        } else {
-          v = acc[i][j][r] + bv;
-        }
-        store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, v);
-      }
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(0, m);
+      if (m < kLoadsB) load_one(there, next, kLoadsA + m);
+      if (m < kReads) read_one(1, here, 1, m);
+      __builtin_amdgcn_sched_barrier(0);
     }
+#pragma unroll
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(1, m);
+      if (m < kReads) read_one(0, here, 2, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(0, m);
+      if (m < kReads) read_one(1, here, 3, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(1, m);
+      if (m < kLoadsA) load_one(here, second, m);
+      if (m < kReads) read_one(0, there, 0, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+#pragma unroll
+  for (int c = 0; c < kLoads; ++c) load_one(stage0, 0, c);
+#pragma unroll
+  for (int c = 0; c < kLoadsA; ++c) load_one(stage1, tile_at(1), c);
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < kReads; ++t) read_one(0, stage0, 0, t);
+  for (int64_t step = 0; step < steps; step += 2) {
+    k_step(stage0, stage1, step);
+    if (step + 1 < steps) k_step(stage1, stage0, step + 1);
   }
+  __syncthreads();     // every load has landed and every fragment is read before the slabs below reuse the stages
+
+  static_assert(4 * 32 * WN * 4 <= kStage, "four slabs fit into one stage");
+  float* slab = reinterpret_cast<float*>(wave < 4 ? stage0 : stage1) + (wave & 3) * (32 * WN);
+  store_wave_tile<INT8, false, NJ>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
 }
 
 template <bool INT8, bool GUARD, int BN>
@@ -622,6 +756,15 @@ template <bool INT8, int BN>
 static int launch_big(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                       int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
   const bool interior = M % kBigM == 0 && N % BN == 0 && k_bytes % kTileBytesK == 0;
+  if (interior) {
+    const dim3 grid(static_cast<unsigned>(N / BN), static_cast<unsigned>(M / kBigM));
+    if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
+    hipLaunchKernelGGL((gemm_direct_kernel<INT8, BN>), grid, dim3(kBigThreads), 0, stream, static_cast<const uint8_t*>(a),
+                       static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                       lda_bytes, ldb_bytes, ldy, out_kind);
+    EP_HIP_TRY(hipGetLastError());
+    return EP_HIP_OK;
+  }
   return interior ? launch_big_variant<INT8, false, BN>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream)
                   : launch_big_variant<INT8, true, BN>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream);
 }
