@@ -623,7 +623,8 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
 // read at the same logical piece then cover all 64 banks once. The two stages are two separate arrays and the K loop
 // is written out for both parities, so that every LDS access names its array: the compiler then waits for loads in
 // flight only where an access may touch the array they fill (before the barrier that publishes it), not before the
-// fragment reads of the other stage.
+// fragment reads of the other stage. (Requesting all pieces right after the barrier, a whole step ahead, measured the
+// same: the loads' latency is covered either way.)
 template <bool INT8, int BN>
 __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                              const float* __restrict__ scale_a, const float* __restrict__ scale_b,
@@ -705,6 +706,9 @@ __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __re
       if (m < kReads) read_one(1, here, 3, m);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // The barrier publishes `there`, which every wave has filled a part of: each waits for its own loads first. (Left
+    // to itself the compiler waits for them where this wave next reads that array, which may be after the barrier.)
+    __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
     __syncthreads();
 #pragma unroll
     for (int m = 0; m < kMultiplies; ++m) {
@@ -718,6 +722,7 @@ __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __re
   for (int c = 0; c < kLoads; ++c) load_one(stage0, 0, c);
 #pragma unroll
   for (int c = 0; c < kLoadsA; ++c) load_one(stage1, tile_at(1), c);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0), as before the barrier in k_step
   __syncthreads();
 #pragma unroll
   for (int t = 0; t < kReads; ++t) read_one(0, stage0, 0, t);
@@ -725,6 +730,7 @@ __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __re
     k_step(stage0, stage1, step);
     if (step + 1 < steps) k_step(stage1, stage0, step + 1);
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();     // every load has landed and every fragment is read before the slabs below reuse the stages
 
   static_assert(4 * 32 * WN * 4 <= kStage, "four slabs fit into one stage");
