@@ -776,13 +776,18 @@ static int launch_big(const void* a, const void* b, const float* scale_a, const 
 }
 
 // Which block tile a product takes: 256 x 256 once there is one for every CU (256 on MI355X); else 256 x 192 if that
-// shape gives at least nine tenths of the CUs a tile; else the 128 x 128 kernel, which spreads small products over
-// more CUs. Returns the tile's column count, 0 for the 128 x 128 kernel.
-static int big_tile_columns(int64_t M, int64_t N) {
+// shape gives enough CUs a tile; else the 128 x 128 kernel, which spreads small products over more CUs. "Enough" is 48
+// for products of whole tiles, which take the direct-load kernel (768 x 3072 x 3072, 48 tiles: 49 us against 56 us;
+// 3072 x 3072 x 3072, 192 tiles: 62 us against 105 us; with fewer tiles and a long K the smaller blocks win again:
+// 256 x 8192 x 28672, 43 tiles, 546 us against 496 us), and 150 for ragged ones, which take the register-staged kernel
+// (3072 x 3000 x 3072: 84 us against 102 us, but 512 x 3000 x 3072: 72 us against 55 us). Returns the tile's column
+// count, 0 for the 128 x 128 kernel.
+static int big_tile_columns(int64_t M, int64_t N, int64_t k_bytes) {
   if (M < kBigM) return 0;
   const int64_t rows = (M + kBigM - 1) / kBigM;
   if (N >= 256 && rows * ((N + 255) / 256) >= 256) return 256;
-  if (N >= 192 && rows * ((N + 191) / 192) >= 230) return 192;
+  const bool whole = M % kBigM == 0 && N % 192 == 0 && k_bytes % kTileBytesK == 0;
+  if (N >= 192 && rows * ((N + 191) / 192) >= (whole ? 48 : 150)) return 192;
   return 0;
 }
 
@@ -996,7 +1001,7 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  if (const int columns = big_tile_columns(M, N)) {
+  if (const int columns = big_tile_columns(M, N, K * 2)) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return columns == 256 ? launch_big<false, 256>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s)
                           : launch_big<false, 192>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s);
@@ -1056,7 +1061,7 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
   if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  if (const int columns = big_tile_columns(M, N)) {
+  if (const int columns = big_tile_columns(M, N, K)) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return columns == 256 ? launch_big<true, 256>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s)
                           : launch_big<true, 192>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s);
