@@ -1,4 +1,4 @@
-"""DecodeAhead: a layer sequence whose weights are decoded a group at a time on a second stream must compute exactly
+"""DecodeAhead: a layer sequence whose weights are decoded a group at a time (in line or on a second stream) must compute exactly
 what the same layers compute on their own, in any call order, pass after pass."""
 import pytest
 import torch
