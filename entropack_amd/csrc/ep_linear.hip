@@ -625,36 +625,38 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
 // flight only where an access may touch the array they fill (before the barrier that publishes it), not before the
 // fragment reads of the other stage. (Requesting all pieces right after the barrier, a whole step ahead, measured the
 // same: the loads' latency is covered either way.)
-template <bool INT8, int BN>
-__global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+template <bool INT8, int BM, int BN, int WAVES_M, int WAVES_N>      // wave tiles of 64 x (BN / WAVES_N); 256 x 192|256 with 4 x 2 waves, 128 x 128 with 2 x 2
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                              const float* __restrict__ scale_a, const float* __restrict__ scale_b,
                                                              const void* __restrict__ bias, void* __restrict__ y, int M, int N,
                                                              int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy,
                                                              int out_kind) {
+  constexpr int kWaves = WAVES_M * WAVES_N;
+  static_assert(BM == 64 * WAVES_M && BN % (32 * WAVES_N) == 0 && BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile shapes");
   constexpr int kRowBytes = kTileBytesK;                    // 128, unpadded
-  constexpr int kStage = (kBigM + BN) * kRowBytes;
+  constexpr int kStage = (BM + BN) * kRowBytes;
   __shared__ __align__(1024) uint8_t stage0[kStage];
   __shared__ __align__(1024) uint8_t stage1[kStage];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  constexpr int WN = BN / 2, NJ = WN / 32;
-  constexpr int kLoadsA = kBigM / 64, kLoadsB = BN / 64, kLoads = kLoadsA + kLoadsB;   // 1 KiB pieces per wave and tile: 4 + 3 or 4
-  const int wave_m = wave >> 1, wave_n = wave & 1;
-  const int m0 = blockIdx.y * kBigM, n0 = blockIdx.x * BN;
+  constexpr int WN = BN / WAVES_N, NJ = WN / 32;
+  constexpr int kLoadsA = BM / (8 * kWaves), kLoadsB = BN / (8 * kWaves), kLoads = kLoadsA + kLoadsB;   // 1 KiB pieces per wave and tile
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
 
-  // Load c of this wave fills tile rows 8 (wave + 8 c') .. + 8 of A (c < kLoadsA, c' = c) or of B (c' = c - kLoadsA).
+  // Load c of this wave fills tile rows 8 (wave + kWaves c') .. + 8 of A (c < kLoadsA, c' = c) or of B (c' = c - kLoadsA).
   const uint8_t* source[kLoads];
 #pragma unroll
   for (int c = 0; c < kLoads; ++c) {
     const bool of_a = c < kLoadsA;
-    const int row = 8 * (wave + 8 * (of_a ? c : c - kLoadsA)) + (lane >> 3);
+    const int row = 8 * (wave + kWaves * (of_a ? c : c - kLoadsA)) + (lane >> 3);
     const int piece = (lane & 7) ^ ((row >> 1) & 7);
     source[c] = of_a ? a + (m0 + row) * lda_bytes + 16 * piece : b + (n0 + row) * ldb_bytes + 16 * piece;
   }
   auto load_one = [&](uint8_t* stage, int64_t kb, int c) {
     const bool of_a = c < kLoadsA;
-    const int first_row = (of_a ? 0 : kBigM) + 8 * (wave + 8 * (of_a ? c : c - kLoadsA));
+    const int first_row = (of_a ? 0 : BM) + 8 * (wave + kWaves * (of_a ? c : c - kLoadsA));
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(source[c] + kb),
                                      (__attribute__((address_space(3))) void*)(stage + first_row * kRowBytes), 16, 0, 0);
   };
@@ -667,7 +669,7 @@ __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __re
   const int frag_row = lane & 31;
   const int turn = (frag_row >> 1) & 7;                      // the same for rows 32 apart
   const uint32_t frag_a_at = static_cast<uint32_t>((wave_m * 64 + frag_row) * kRowBytes);
-  const uint32_t frag_b_at = static_cast<uint32_t>((kBigM + wave_n * WN + frag_row) * kRowBytes);
+  const uint32_t frag_b_at = static_cast<uint32_t>((BM + wave_n * WN + frag_row) * kRowBytes);
   auto read_one = [&](int set, const uint8_t* stage, int kk, int t) {
     const uint32_t place = static_cast<uint32_t>(((2 * kk + (lane >> 5)) ^ turn) * 16);
     const uint32_t at = place + (t < 2 ? frag_a_at + t * 32 * kRowBytes : frag_b_at + (t - 2) * 32 * kRowBytes);
@@ -733,7 +735,7 @@ __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const uint8_t* __re
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();     // every load has landed and every fragment is read before the slabs below reuse the stages
 
-  static_assert(4 * 32 * WN * 4 <= kStage, "four slabs fit into one stage");
+  static_assert(4 * 32 * WN * 4 <= kStage && kWaves <= 8, "four slabs fit into one stage");
   float* slab = reinterpret_cast<float*>(wave < 4 ? stage0 : stage1) + (wave & 3) * (32 * WN);
   store_wave_tile<INT8, false, NJ>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
 }
@@ -765,7 +767,7 @@ static int launch_big(const void* a, const void* b, const float* scale_a, const 
   if (interior) {
     const dim3 grid(static_cast<unsigned>(N / BN), static_cast<unsigned>(M / kBigM));
     if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
-    hipLaunchKernelGGL((gemm_direct_kernel<INT8, BN>), grid, dim3(kBigThreads), 0, stream, static_cast<const uint8_t*>(a),
+    hipLaunchKernelGGL((gemm_direct_kernel<INT8, kBigM, BN, 4, 2>), grid, dim3(kBigThreads), 0, stream, static_cast<const uint8_t*>(a),
                        static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
                        lda_bytes, ldb_bytes, ldy, out_kind);
     EP_HIP_TRY(hipGetLastError());
@@ -775,8 +777,37 @@ static int launch_big(const void* a, const void* b, const float* scale_a, const 
                   : launch_big_variant<INT8, true, BN>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream);
 }
 
+// Products of whole 128 x 128 tiles: the direct-load kernel with four waves of 64 x 64 per block and two blocks per CU
+// (64 KB of LDS each). While all blocks are resident at once (at most 512 on the 256 CUs of an MI355X) this is the
+// fastest of the tiled kernels here: 256 x 3072 x 3072 bf16 24 us (the single-stage 128 x 128 kernel below 52 us, the
+// vendor library 25 us), 1024 x 3072 x 3072 35 us (256 x 192 tiles 49 us), 2560 x 3072 x 3072, 480 blocks, 51 us (57 us).
+// With more blocks than that a second round starts and the 256-row tiles win: 3072 x 3072 x 3072 80 us against 62 us.
+constexpr int64_t kSmallTileSlots = 512;
+
+template <bool INT8>
+static bool small_whole_tiles(int64_t M, int64_t N, int64_t k_bytes) {
+  return M % 128 == 0 && N % 128 == 0 && k_bytes % kTileBytesK == 0 && M / 128 <= 65535;
+}
+
+template <bool INT8>
+static bool small_tiles_in_one_round(int64_t M, int64_t N, int64_t k_bytes) {
+  return small_whole_tiles<INT8>(M, N, k_bytes) && (M / 128) * (N / 128) <= kSmallTileSlots;
+}
+
+template <bool INT8>
+static int launch_direct_small(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
+                               int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(N / 128), static_cast<unsigned>(M / 128));
+  hipLaunchKernelGGL((gemm_direct_kernel<INT8, 128, 128, 2, 2>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a),
+                     static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                     lda_bytes, ldb_bytes, ldy, out_kind);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
 // Which block tile a product takes: 256 x 256 once there is one for every CU (256 on MI355X); else 256 x 192 if that
-// shape gives enough CUs a tile; else the 128 x 128 kernel, which spreads small products over more CUs. "Enough" is 48
+// shape gives enough CUs a tile; else the 128 x 128 kernels, which spread small products over more CUs (products of
+// whole 128 x 128 tiles that fit the machine in one round never get here, see above). "Enough" is 48
 // for products of whole tiles, which take the direct-load kernel (768 x 3072 x 3072, 48 tiles: 49 us against 56 us;
 // 3072 x 3072 x 3072, 192 tiles: 62 us against 105 us; with fewer tiles and a long K the smaller blocks win again:
 // 256 x 8192 x 28672, 43 tiles, 546 us against 496 us), and 150 for ragged ones, which take the register-staged kernel
@@ -1001,11 +1032,15 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  if (small_tiles_in_one_round<false>(M, N, K * 2))
+    return launch_direct_small<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, static_cast<hipStream_t>(stream));
   if (const int columns = big_tile_columns(M, N, K * 2)) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return columns == 256 ? launch_big<false, 256>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s)
                           : launch_big<false, 192>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s);
   }
+  if (small_whole_tiles<false>(M, N, K * 2))
+    return launch_direct_small<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, static_cast<hipStream_t>(stream));
   const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
   hipLaunchKernelGGL(gemm_bf16_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
@@ -1061,11 +1096,15 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
   if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  if (small_tiles_in_one_round<true>(M, N, K))
+    return launch_direct_small<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, static_cast<hipStream_t>(stream));
   if (const int columns = big_tile_columns(M, N, K)) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return columns == 256 ? launch_big<true, 256>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s)
                           : launch_big<true, 192>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s);
   }
+  if (small_whole_tiles<true>(M, N, K))
+    return launch_direct_small<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, static_cast<hipStream_t>(stream));
   const dim3 grid(static_cast<unsigned>((N + kBlockN - 1) / kBlockN), static_cast<unsigned>((M + kBlockM - 1) / kBlockM));
   if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
   hipLaunchKernelGGL(gemm_i8_nt_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a_dev, b_dev, scale_a_dev,
