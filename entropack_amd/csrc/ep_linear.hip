@@ -390,7 +390,7 @@ __global__ __launch_bounds__(256) void rotate_quantize_rows_kernel(const void* _
 // stores whole row pieces, 16 bytes per lane. In the slab, rows with bit 2 set keep their columns rotated by 32: the
 // two lane halves of an accumulator register (rows 4 apart) then write to different banks. The arithmetic and the
 // rounding are those of the element-wise path, which ragged products and outputs with unaligned rows take.
-template <bool INT8, bool GUARD, int NJ, typename Acc>
+template <bool INT8, bool GUARD, int NJ, typename Acc, bool EDGE = false>    // EDGE: whole row pieces, but the tile may overhang M and N
 __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, const float* __restrict__ scale_a,
                                                 const float* __restrict__ scale_b, const void* __restrict__ bias,
                                                 void* __restrict__ y, int M, int N, int64_t ldy, int out_kind, int row0, int col0,
@@ -398,13 +398,15 @@ __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, 
   constexpr int WN = 32 * NJ;
   auto slab_at = [](int row, int col) { const int c = col + ((row & 4) << 3); return row * WN + (c >= WN ? c - WN : c); };
   const int out_bytes = out_kind == kOutF32 ? 4 : 2;
-  const bool wide_rows = !GUARD && ((reinterpret_cast<uintptr_t>(y) | static_cast<uintptr_t>(ldy * out_bytes)) & 15u) == 0;
+  const bool wide_rows = !GUARD && ((reinterpret_cast<uintptr_t>(y) | static_cast<uintptr_t>(ldy * out_bytes)) & 15u) == 0 &&
+                         (!EDGE || N % (16 / out_bytes) == 0);      // a 16-byte piece is then all inside the row or all outside
   if (wide_rows) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const int n = col0 + j * 32 + (lane & 31);
+        int n = col0 + j * 32 + (lane & 31);
+        if (EDGE && n >= N) n = N - 1;                        // overhanging columns are computed and dropped below
         const bool has_bias = bias != nullptr;
         const float bv = has_bias ? load_bias(bias, out_kind, n) : 0.0f;
         float sb = 1.0f;
@@ -414,7 +416,7 @@ __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, 
           const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
           float v;
           if constexpr (INT8) {
-            v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[row0 + i * 32 + row]), sb);
+            v = __fmul_rn(__fmul_rn(static_cast<float>(acc[i][j][r]), scale_a[EDGE && row0 + i * 32 + row >= M ? M - 1 : row0 + i * 32 + row]), sb);
             if (has_bias) v = __fadd_rn(v, bv);
           } else {
             v = acc[i][j][r] + bv;
@@ -429,6 +431,7 @@ __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, 
 #pragma unroll
         for (int at = 0; at < 32 * kPieces; at += 64) {
           const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
+          if (EDGE && (row0 + i * 32 + row >= M || col0 + 4 * piece >= N)) continue;
           *reinterpret_cast<uint4*>(out + row * ldy + 4 * piece) =
               *reinterpret_cast<const uint4*>(slab + slab_at(row, 4 * piece));
         }
@@ -438,6 +441,7 @@ __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, 
 #pragma unroll
         for (int at = 0; at < 32 * kPieces; at += 64) {
           const int row = (at + lane) / kPieces, piece = (at + lane) % kPieces;
+          if (EDGE && (row0 + i * 32 + row >= M || col0 + 8 * piece >= N)) continue;
           const float* from = slab + slab_at(row, 8 * piece);
           const float4 lo = *reinterpret_cast<const float4*>(from);
           const float4 hi = *reinterpret_cast<const float4*>(from + 4);
@@ -614,7 +618,7 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
 
 // ---- the same block tile with the operand tiles loaded straight into LDS ----------------------------------------------------
 //
-// For whole tiles (M, N multiples of the block tile, K of one tile step). The kernel above moves every tile byte
+// For K a multiple of one tile step (M and N may overhang the tiles with RAGGED). The kernel above moves every tile byte
 // memory -> registers -> LDS, and that round trip (seven 16-byte loads and seven LDS stores per wave and K step) is what
 // keeps it a third above the matrix cores' own time. Here `global_load_lds_dwordx4` writes the loaded bytes into LDS
 // itself: one instruction fills 1 KiB of consecutive LDS (lane l the 16 bytes at 16 l), i.e. eight tile rows of 128
@@ -625,7 +629,9 @@ __global__ __launch_bounds__(512, 2) void gemm_big_kernel(const uint8_t* __restr
 // flight only where an access may touch the array they fill (before the barrier that publishes it), not before the
 // fragment reads of the other stage. (Requesting all pieces right after the barrier, a whole step ahead, measured the
 // same: the loads' latency is covered either way.)
-template <bool INT8, int BM, int BN, int WAVES_M, int WAVES_N>      // wave tiles of 64 x (BN / WAVES_N); 256 x 192|256 with 4 x 2 waves, 128 x 128 with 2 x 2
+// RAGGED: M and N need not be multiples of the tile (K must be of a tile step): rows past the end load the last row
+// again and are dropped by the epilogue.
+template <bool INT8, int BM, int BN, int WAVES_M, int WAVES_N, bool RAGGED>   // wave tiles of 64 x (BN / WAVES_N); 256 x 192|256 with 4 x 2 waves, 128 x 128 with 2 x 2
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                              const float* __restrict__ scale_a, const float* __restrict__ scale_b,
                                                              const void* __restrict__ bias, void* __restrict__ y, int M, int N,
@@ -652,7 +658,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(
     const bool of_a = c < kLoadsA;
     const int row = 8 * (wave + kWaves * (of_a ? c : c - kLoadsA)) + (lane >> 3);
     const int piece = (lane & 7) ^ ((row >> 1) & 7);
-    source[c] = of_a ? a + (m0 + row) * lda_bytes + 16 * piece : b + (n0 + row) * ldb_bytes + 16 * piece;
+    int from_row = (of_a ? m0 : n0) + row;
+    if (RAGGED && from_row >= (of_a ? M : N)) from_row = (of_a ? M : N) - 1;
+    source[c] = of_a ? a + from_row * lda_bytes + 16 * piece : b + from_row * ldb_bytes + 16 * piece;
   }
   auto load_one = [&](uint8_t* stage, int64_t kb, int c) {
     const bool of_a = c < kLoadsA;
@@ -737,7 +745,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(
 
   static_assert(4 * 32 * WN * 4 <= kStage && kWaves <= 8, "four slabs fit into one stage");
   float* slab = reinterpret_cast<float*>(wave < 4 ? stage0 : stage1) + (wave & 3) * (32 * WN);
-  store_wave_tile<INT8, false, NJ>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
+  store_wave_tile<INT8, false, NJ, Acc, RAGGED>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
 }
 
 template <bool INT8, bool GUARD, int BN>
@@ -764,12 +772,17 @@ template <bool INT8, int BN>
 static int launch_big(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                       int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
   const bool interior = M % kBigM == 0 && N % BN == 0 && k_bytes % kTileBytesK == 0;
-  if (interior) {
-    const dim3 grid(static_cast<unsigned>(N / BN), static_cast<unsigned>(M / kBigM));
+  if (k_bytes % kTileBytesK == 0) {
+    const dim3 grid(static_cast<unsigned>((N + BN - 1) / BN), static_cast<unsigned>((M + kBigM - 1) / kBigM));
     if (grid.y > 65535) return EP_HIP_EUNSUPPORTED;
-    hipLaunchKernelGGL((gemm_direct_kernel<INT8, kBigM, BN, 4, 2>), grid, dim3(kBigThreads), 0, stream, static_cast<const uint8_t*>(a),
-                       static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
-                       lda_bytes, ldb_bytes, ldy, out_kind);
+    if (interior)
+      hipLaunchKernelGGL((gemm_direct_kernel<INT8, kBigM, BN, 4, 2, false>), grid, dim3(kBigThreads), 0, stream, static_cast<const uint8_t*>(a),
+                         static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                         lda_bytes, ldb_bytes, ldy, out_kind);
+    else
+      hipLaunchKernelGGL((gemm_direct_kernel<INT8, kBigM, BN, 4, 2, true>), grid, dim3(kBigThreads), 0, stream, static_cast<const uint8_t*>(a),
+                         static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                         lda_bytes, ldb_bytes, ldy, out_kind);
     EP_HIP_TRY(hipGetLastError());
     return EP_HIP_OK;
   }
@@ -785,22 +798,27 @@ static int launch_big(const void* a, const void* b, const float* scale_a, const 
 constexpr int64_t kSmallTileSlots = 512;
 
 template <bool INT8>
-static bool small_whole_tiles(int64_t M, int64_t N, int64_t k_bytes) {
-  return M % 128 == 0 && N % 128 == 0 && k_bytes % kTileBytesK == 0 && M / 128 <= 65535;
+static bool small_whole_tiles(int64_t M, int64_t N, int64_t k_bytes) {       // whole in K; M and N may overhang
+  return k_bytes % kTileBytesK == 0 && (M + 127) / 128 <= 65535;
 }
 
 template <bool INT8>
 static bool small_tiles_in_one_round(int64_t M, int64_t N, int64_t k_bytes) {
-  return small_whole_tiles<INT8>(M, N, k_bytes) && (M / 128) * (N / 128) <= kSmallTileSlots;
+  return small_whole_tiles<INT8>(M, N, k_bytes) && ((M + 127) / 128) * ((N + 127) / 128) <= kSmallTileSlots;
 }
 
 template <bool INT8>
 static int launch_direct_small(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                                int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
-  const dim3 grid(static_cast<unsigned>(N / 128), static_cast<unsigned>(M / 128));
-  hipLaunchKernelGGL((gemm_direct_kernel<INT8, 128, 128, 2, 2>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a),
-                     static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
-                     lda_bytes, ldb_bytes, ldy, out_kind);
+  const dim3 grid(static_cast<unsigned>((N + 127) / 128), static_cast<unsigned>((M + 127) / 128));
+  if (M % 128 == 0 && N % 128 == 0)
+    hipLaunchKernelGGL((gemm_direct_kernel<INT8, 128, 128, 2, 2, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a),
+                       static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                       lda_bytes, ldb_bytes, ldy, out_kind);
+  else
+    hipLaunchKernelGGL((gemm_direct_kernel<INT8, 128, 128, 2, 2, true>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a),
+                       static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
+                       lda_bytes, ldb_bytes, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }
@@ -817,7 +835,7 @@ static int big_tile_columns(int64_t M, int64_t N, int64_t k_bytes) {
   if (M < kBigM) return 0;
   const int64_t rows = (M + kBigM - 1) / kBigM;
   if (N >= 256 && rows * ((N + 255) / 256) >= 256) return 256;
-  const bool whole = M % kBigM == 0 && N % 192 == 0 && k_bytes % kTileBytesK == 0;
+  const bool whole = k_bytes % kTileBytesK == 0;            // the direct-load kernel takes it, overhanging tiles included
   if (N >= 192 && rows * ((N + 191) / 192) >= (whole ? 48 : 150)) return 192;
   return 0;
 }
