@@ -136,6 +136,18 @@ def linear_section(ep, steps):
         ms = _median_ms(lambda: layer(x), steps)
         out[mode] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2),
                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5), "rel_l2_vs_f32_reference": rel}
+    # Fewer activation rows than the configuration names, between the 128 of the streaming kernel and the 4096 above:
+    # the products of this library's tiled kernels (`fused`) beside the vendor library's (`decode_then_gemm`).
+    out["fewer_rows"] = {}
+    for rows in (256, 1024):
+        part = x[:rows].contiguous()
+        entry = {}
+        for mode in ("decode_then_gemm", "fused"):
+            layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
+            got = layer(part).double()
+            entry[mode] = {"ms": round(_median_ms(lambda: layer(part), steps), 5),
+                           "rel_l2_vs_f32_reference": ((got - reference[:rows]).norm() / reference[:rows].norm()).item()}
+        out["fewer_rows"][f"M={rows}"] = entry
     # The same layer encoded with tiles a quarter and an eighth of the default size (`tile_elements`, a field of the
     # reference's config): a tile's chain of dependent steps, which is all a single layer's decode waits for, shortens
     # in proportion, for a per-tile header that costs 1-3 % more stored bits.
