@@ -15,7 +15,8 @@ _PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(_
 LIBRARY_PATH = os.path.join(_PACKAGE_DIR, "libentropack_hip.so")
 ABI_VERSION = 1
 
-OK, EINVAL, EUNSUPPORTED, ERUNTIME, ENODEVICE = range(5)
+OK, EINVAL, EUNSUPPORTED, ERUNTIME, ENODEVICE, ETOOLARGE = range(6)
+STATIC_ACCUMULATOR_FLOATS = 1 << 18          # EP_HIP_STATIC_ACCUMULATOR_FLOATS
 TABLE_GLOBAL64, TABLE_LDS_BYTE, TABLE_LDS_WIDE, TABLE_LDS_RANK, TABLE_LDS_SYM = range(5)
 TABLE_KIND_NAMES = {TABLE_GLOBAL64: "global64", TABLE_LDS_BYTE: "lds_byte", TABLE_LDS_WIDE: "lds_wide", TABLE_LDS_RANK: "lds_rank",
                     TABLE_LDS_SYM: "lds_sym"}
@@ -91,6 +92,9 @@ _SIGNATURES = {
     "ep_hip_linear_fused_bf16": (ctypes.c_int, [
         ctypes.POINTER(DecodeJob), ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
         ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
+    "ep_hip_linear_fused_bf16_static": (ctypes.c_int, [
+        ctypes.POINTER(DecodeJob), ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
+        ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "ep_hip_gemm_bf16": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
         ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),

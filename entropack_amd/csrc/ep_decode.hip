@@ -12,6 +12,8 @@
 #include <hip/hip_fp16.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "ep_store.hpp"
 
 namespace ep {
@@ -431,13 +433,11 @@ __global__ __launch_bounds__(256) void finish_linear_kernel(const float* __restr
 
 }  // namespace ep
 
-extern "C" int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
-                                        const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, float* workspace_dev,
-                                        void* stream) {
-  using namespace ep;
-  if (weight == nullptr || x_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
-  if (out_kind < EP_FLOAT_BF16 || out_kind > EP_FLOAT_F32 || m_rows <= 0) return EP_HIP_EINVAL;
-  if (weight->desc == nullptr) return EP_HIP_EINVAL;
+namespace ep {
+
+// Decode-and-multiply for one to four activation rows with the f32 accumulator `y32` given by the caller.
+static int linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx, const void* bias_dev,
+                             void* y_dev, int64_t ldy, int out_kind, float* y32, hipStream_t s) {
   const int64_t outer = weight->rows, inner = weight->cols_padded;
   if (ldx < inner || ldy < outer || reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || ldx % 8 != 0) return EP_HIP_EINVAL;
   // The kernels carry at most four activation rows in registers, need whole weight rows of at least 32 vectors (a
@@ -452,17 +452,66 @@ extern "C" int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const v
   args.m_rows = static_cast<int>(m_rows);
   args.x = static_cast<const uint16_t*>(x_dev);
   args.ldx = ldx;
-  args.y32 = workspace_dev;
+  args.y32 = y32;
   args.ldy32 = outer;
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t cells = m_rows * outer;
+  // The accumulator is cleared by a kernel, never a memset node: the sequence may be captured into a graph.
   hipLaunchKernelGGL(zero_f32_kernel, dim3(static_cast<unsigned>((cells + 255) / 256 < 1024 ? (cells + 255) / 256 : 1024)), dim3(256), 0, s,
-                     workspace_dev, cells);
+                     y32, cells);
   EP_HIP_TRY(hipGetLastError());
   const int launched = launch_lds_decode(args, *weight->desc, m_rows == 1 ? -2 : -3, pairs, s);
   if (launched != EP_HIP_OK) return launched;
-  hipLaunchKernelGGL(finish_linear_kernel, dim3(static_cast<unsigned>((outer + 255) / 256)), dim3(256), 0, s, workspace_dev, bias_dev, y_dev,
+  hipLaunchKernelGGL(finish_linear_kernel, dim3(static_cast<unsigned>((outer + 255) / 256)), dim3(256), 0, s, y32, bias_dev, y_dev,
                      static_cast<int>(m_rows), outer, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
+}
+
+// The accumulator of ep_hip_linear_fused_bf16_static: one copy per GPU, held until the process ends. In host code the
+// array's name is only a handle; its device address comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) float scratch[EP_HIP_STATIC_ACCUMULATOR_FLOATS];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_lock;
+static float* g_scratch_of_device[kMaxDevices];      // device ordinal -> address of that device's `scratch`
+
+static int static_accumulator(float** address) {
+  int device = 0;
+  EP_HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return EP_HIP_EUNSUPPORTED;
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_scratch_of_device[device] == nullptr) {
+    float* found = nullptr;
+    EP_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&found), HIP_SYMBOL(scratch)));
+    if (found == nullptr) return EP_HIP_ERUNTIME;
+    g_scratch_of_device[device] = found;
+  }
+  *address = g_scratch_of_device[device];
+  return EP_HIP_OK;
+}
+
+}  // namespace ep
+
+extern "C" int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
+                                        const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, float* workspace_dev,
+                                        void* stream) {
+  using namespace ep;
+  if (weight == nullptr || x_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
+  if (out_kind < EP_FLOAT_BF16 || out_kind > EP_FLOAT_F32 || m_rows <= 0) return EP_HIP_EINVAL;
+  if (weight->desc == nullptr) return EP_HIP_EINVAL;
+  return linear_fused_bf16(weight, x_dev, m_rows, ldx, bias_dev, y_dev, ldy, out_kind, workspace_dev, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
+                                               const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* stream) {
+  using namespace ep;
+  if (weight == nullptr || x_dev == nullptr || y_dev == nullptr) return EP_HIP_EINVAL;
+  if (out_kind < EP_FLOAT_BF16 || out_kind > EP_FLOAT_F32 || m_rows <= 0) return EP_HIP_EINVAL;
+  if (weight->desc == nullptr || weight->rows <= 0) return EP_HIP_EINVAL;
+  if (m_rows > 4) return EP_HIP_EUNSUPPORTED;
+  if (m_rows * weight->rows > EP_HIP_STATIC_ACCUMULATOR_FLOATS) return EP_HIP_ETOOLARGE;
+  float* accumulator = nullptr;
+  const int status = static_accumulator(&accumulator);
+  if (status != EP_HIP_OK) return status;
+  return linear_fused_bf16(weight, x_dev, m_rows, ldx, bias_dev, y_dev, ldy, out_kind, accumulator, static_cast<hipStream_t>(stream));
 }

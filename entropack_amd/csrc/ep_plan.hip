@@ -178,6 +178,7 @@ const char* ep_hip_error_string(int status) {
     case EP_HIP_EUNSUPPORTED: return "unsupported by this build";
     case EP_HIP_ERUNTIME: return "HIP runtime call failed";
     case EP_HIP_ENODEVICE: return "no gfx950 device";
+    case EP_HIP_ETOOLARGE: return "request exceeds the library's fixed scratch buffer";
     default: return "unknown status";
   }
 }

@@ -25,7 +25,8 @@ enum ep_hip_status {
   EP_HIP_EINVAL = 1,        /* a size, alignment or enum argument is out of range */
   EP_HIP_EUNSUPPORTED = 2,  /* valid request this build has no kernel for */
   EP_HIP_ERUNTIME = 3,      /* a HIP runtime call failed; ep_hip_last_runtime_error() has the hipError_t */
-  EP_HIP_ENODEVICE = 4      /* no gfx950 device visible */
+  EP_HIP_ENODEVICE = 4,     /* no gfx950 device visible */
+  EP_HIP_ETOOLARGE = 5      /* the request needs more scratch memory than the library's fixed, statically allocated buffer holds */
 };
 
 /* Output container kinds. 0..12 keep the numbering of the reference's store kinds
@@ -245,6 +246,19 @@ int ep_hip_rotate_quantize_rows(const void* x_dev, int in_kind, int64_t rows, in
 int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
                              const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, float* workspace_dev,
                              void* stream);
+
+/* ep_hip_linear_fused_bf16 for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc): same arguments, results and errors, but the f32 accumulator is a fixed array inside
+ * the library's device image (EP_HIP_STATIC_ACCUMULATOR_FLOATS floats = 1 MiB on every GPU the library runs on, held
+ * until the process ends) instead of a caller's workspace. Nothing is allocated or freed, here or in any routine it
+ * calls. m_rows * weight->rows above EP_HIP_STATIC_ACCUMULATOR_FLOATS returns EP_HIP_ETOOLARGE. Every call on a GPU
+ * uses that GPU's one array (cleared by a kernel at the start of each call): calls that overlap on one GPU, from
+ * different streams or threads, race; calls on one stream, or otherwise ordered, are safe.
+ * No counterpart in the reference, whose lane allocates its outputs with torch.empty
+ * (entropack/schemes/lattice_rans/cuda.py:794). */
+#define EP_HIP_STATIC_ACCUMULATOR_FLOATS (1 << 18)
+int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
+                                    const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* stream);
 
 #ifdef __cplusplus
 }
