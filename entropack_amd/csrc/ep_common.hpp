@@ -61,11 +61,19 @@ inline size_t rank_table_bytes(int present, int prob_bits) {
   return rank_rs_offset(present, prob_bits) + kFieldStreams * rank_rs_stream_bytes(prob_bits);
 }
 
-// LDS_SYM section: FB u64[16][256] (indexed by value + 128) = {freq | (value & 0xFF) << 24, cdf + LDS address of the stream's slot table}, then
-// SLOT u8[16][2^pb] = value + 128. The kernel stages it at LDS offset 0.
+// LDS_SYM section, staged at LDS offset 0: FB u64[16][256], indexed by value + 128, then SLOT u8[16][2048] = value + 128
+// (the first 2^pb slots of each are used). An FB entry is
+//   word 0: freq | 0x3C000000 when the value is odd  (the multiply takes the low 24 bits; the high halves of seven such
+//           words XOR to the parity of z0..z6 as a half-precision 0.0 or 1.0)
+//   word 1: (cdf + 2048 * coset) | half(value) << 16  (the decode step forms slot | 2048 * coset, both as the slot
+//           table's address and as the number the low half is subtracted from; the high half is the value itself, which a
+//           mixed-precision multiply-add takes without a conversion).
+// A field's two cosets lie 2048 bytes apart in both parts, so one per-lane offset serves both lookups.
 constexpr int kSymFbStreamBytes = 256 * 8;
 constexpr int kSymFbBytes = kFieldStreams * kSymFbStreamBytes;
-inline int sym_table_bytes(int prob_bits) { return kSymFbBytes + (kFieldStreams << prob_bits); }
+constexpr int kSymSlotStreamBytes = 2048;
+static_assert(kSymSlotStreamBytes == kSymFbStreamBytes, "one coset offset addresses both parts");
+constexpr int sym_table_bytes(int /*prob_bits*/) { return kSymFbBytes + kFieldStreams * kSymSlotStreamBytes; }
 inline int lds_sym_decode_bytes(int prob_bits, int waves) { return sym_table_bytes(prob_bits) + waves * 2 * kRingBytes + 256; }
 
 // LDS bytes the LDS-table decode kernel needs for `waves` wavefronts each carrying `ilp` tile pairs.

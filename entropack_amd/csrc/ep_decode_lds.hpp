@@ -70,6 +70,7 @@ struct Pair {
   uint32_t coset_base;   // LDS byte offset of this lane's coset inside a field's table pair (0 or one table)
   uint64_t coset_mask;   // wave-uniform: the lanes whose current vector lies in coset 1
   uint32_t e[8];         // slot-table entries of the eight fields of the current vector
+  uint32_t ey[8];        // two-level tables only: the entries' second words (the value in half precision in the high half)
   int dot_row;           // multiply-on-the-fly only: the weight row `dot_acc` belongs to (same in all lanes of a half), -1 = none
   float dot_acc[kDotRows];
 };
@@ -342,22 +343,24 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_group,
 
 // ---- two-level tables (byte values, prob_bits <= 11) --------------------------------------------------------------------
 //
-// slot -> value + 128 (one byte) -> {freq | (value & 0xFF) << 24, cdf}. A quarter of the slot table of the byte form,
-// so two workgroups share a CU; one more dependent LDS read per step, one vector instruction less. The stored cdf
-// already contains the LDS address bits that `slot | table address` carries, and the first word has the layout of
-// a byte-form entry, so reconstruction is shared with it.
+// slot -> value + 128 (one byte) -> {freq | parity mark, cdf | half(value) << 16}. A quarter of the slot table of the
+// byte form, so two workgroups share a CU; one more dependent LDS read per step, one vector instruction less. The stored
+// cdf already contains the coset offset that `slot | coset offset` carries. The entry holds the value as a
+// half-precision number and its parity as a half-precision 0.0 / 1.0 pattern, so reconstruction needs no integer to
+// float conversion (see sym_point below).
 template <int PB, bool MASKED>
-__device__ __forceinline__ void sym_step(Pair& p, int field, uint32_t slot_cb, const StepConsts& k, bool valid_lane) {
+__device__ __forceinline__ void sym_step(Pair& p, int field, const StepConsts& k, bool valid_lane) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   typedef __attribute__((address_space(3))) const u32x2* lds_u2;
   typedef __attribute__((address_space(3))) const uint8_t* lds_u8;
   constexpr uint32_t kTable = 1u << PB;
   const uint32_t x = p.x;
-  const uint32_t at = (x & (kTable - 1u)) | slot_cb;
-  const uint32_t value = *reinterpret_cast<lds_u8>(static_cast<uintptr_t>(at + static_cast<uint32_t>(field) * 2u * kTable));
+  const uint32_t at = (x & (kTable - 1u)) | p.coset_base;
+  const uint32_t value = *reinterpret_cast<lds_u8>(static_cast<uintptr_t>(at + static_cast<uint32_t>(kSymFbBytes) + static_cast<uint32_t>(field) * 2u * kSymSlotStreamBytes));
   const u32x2 entry = *reinterpret_cast<lds_u2>(static_cast<uintptr_t>((value << 3) + p.coset_base + static_cast<uint32_t>(field) * 2u * kSymFbStreamBytes));
-  const uint32_t next = __umul24(entry.x, x >> PB) + at - entry.y;
+  const uint32_t next = __umul24(entry.x, x >> PB) + at - (entry.y & 0xFFFFu);
   p.e[field] = entry.x;
+  p.ey[field] = entry.y;
   p.x = (!MASKED || valid_lane) ? next : x;
   uint32_t t, d, na, nb;
   uint32_t pos = uniform(p.pos);
@@ -373,6 +376,20 @@ __device__ __forceinline__ void sym_step(Pair& p, int field, uint32_t slot_cb, c
                  : "vcc", "scc", "memory");
   }
   p.pos = pos;
+}
+
+// fma(half in the high 16 bits of `packed`, b, c) in float32 with one rounding: v_fma_mix_f32 reads the half-precision
+// operand where it lies, so a value the table holds in that form costs no conversion.
+__device__ __forceinline__ float fma_high_half(uint32_t packed, float b, float c) {
+  float r;
+  asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(b), "v"(c));
+  return r;
+}
+// fma(half in the high 16 bits of `packed`, 2, half in the high 16 bits of `addend`)
+__device__ __forceinline__ float twice_high_half_plus(uint32_t packed, uint32_t addend) {
+  float r;
+  asm("v_fma_mix_f32 %0, %1, 2.0, %2 op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "=v"(r) : "v"(packed), "v"(addend));
+  return r;
 }
 
 // ---- payload windows ---------------------------------------------------------------------------------------------------
@@ -471,7 +488,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   constexpr bool WIDE = MODE == kModeWide || MODE == kModeRank;    // symbols as integers, not as biased bytes in bits 24..31
   static_assert((MODE != kModeRank && MODE != kModeSym) || ILP == 1, "the rank/select and two-level steps are single-pair");
   const uint32_t lut_bytes = MODE == kModeRank ? (a.lut_bytes + 255u) / 256u * 256u
-                                               : (MODE == kModeSym ? static_cast<uint32_t>(kSymFbBytes + (kFieldStreams << PB)) : L::kLutBytes);
+                                               : (MODE == kModeSym ? static_cast<uint32_t>(sym_table_bytes(PB)) : L::kLutBytes);
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
 
   const int waves = blockDim.x >> 6;
@@ -561,7 +578,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
     // number rounded once, c * scale / 2 being exact, and costs one instruction per weight less. Any other scale
     // (zero, negative: the sign of a zero weight; subnormal; beyond 1e30: bf16 saturation) takes the literal form.
     auto lattice_point = [&](const Pair& s, float (&z)[8]) {
-      if constexpr (!WIDE) {
+      if constexpr (MODE == kModeSym) {
+        // The entries hold the values in half precision (second word, high half); the first words' high halves XOR to
+        // the parity of z0..z6 as a half-precision 0.0 or 1.0.
+        const uint32_t folded = xor3(xor3(s.e[0], s.e[1], s.e[2]), xor3(s.e[3], s.e[4], s.e[5]), s.e[6]);
+#pragma unroll
+        for (int f = 0; f < 7; ++f) z[f] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(s.ey[f] >> 16)));
+        z[7] = twice_high_half_plus(s.ey[7], folded);
+      } else if constexpr (!WIDE) {
         // Top byte = the value as a signed byte; the parity of z0..z6 is the parity of those bytes.
         const uint32_t folded = xor3(xor3(s.e[0], s.e[1], s.e[2]), xor3(s.e[3], s.e[4], s.e[5]), s.e[6]);
         const float parity = static_cast<float>((folded >> 24) & 1u);
@@ -583,17 +607,29 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         for (int f = 0; f < 8; ++f) z[f] = static_cast<float>(v[f]);
       }
     };
+    // w = fma(z, scale, shift) for an ordinary scale; with two-level tables straight from the half-precision values.
+    auto scaled_point = [&](const Pair& s, float scale, float shift, float (&w)[8]) {
+      if constexpr (MODE == kModeSym) {
+        const uint32_t folded = xor3(xor3(s.e[0], s.e[1], s.e[2]), xor3(s.e[3], s.e[4], s.e[5]), s.e[6]);
+#pragma unroll
+        for (int f = 0; f < 7; ++f) w[f] = fma_high_half(s.ey[f], scale, shift);
+        w[7] = __fmaf_rn(twice_high_half_plus(s.ey[7], folded), scale, shift);
+      } else {
+        float z[8];
+        lattice_point(s, z);
+#pragma unroll
+        for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], scale, shift);
+      }
+    };
     auto weights_of = [&](const Pair& s, float scale, float (&w)[8]) {
       const bool c = s.coset_base != 0;
-      float z[8];
-      lattice_point(s, z);
       // 1e-30 <= scale <= 1e30 as one unsigned comparison of the bit patterns (fails for negative values and NaN).
       const bool ordinary = __float_as_uint(scale) - 0x0DA24260u <= 0x7149F2CAu - 0x0DA24260u;
       if (__builtin_expect(ordinary, 1)) {
-        const float half = c ? __fmul_rn(scale, 0.5f) : 0.0f;
-#pragma unroll
-        for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], scale, half);
+        scaled_point(s, scale, c ? __fmul_rn(scale, 0.5f) : 0.0f, w);
       } else {
+        float z[8];
+        lattice_point(s, z);
         const float shift = c ? 0.5f : 0.0f;
 #pragma unroll
         for (int f = 0; f < 8; ++f) w[f] = __fmul_rn(__fadd_rn(z[f], shift), scale);
@@ -709,11 +745,6 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       s.dot_row = any ? low : -1;
     };
 
-    // Two-level tables: LDS address of the lane's coset's slot table of field 0.
-    auto sym_slot_base = [](const Pair& s) {
-      return __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? static_cast<uint32_t>(kSymFbBytes) + L::kTable : static_cast<uint32_t>(kSymFbBytes);
-    };
-
     using Masked = std::integral_constant<bool, true>;
     using Unmasked = std::integral_constant<bool, false>;
 
@@ -727,14 +758,13 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       uint32_t high[ILP];
 #pragma unroll
       for (int j = 0; j < ILP; ++j) high[j] = st[j].coset_base + L::kHighBase;
-      const uint32_t slot_base = MODE == kModeSym ? sym_slot_base(st[0]) : 0u;
       const uint32_t rank_group = st[0].coset_base + rank_rs0;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
           rank_step<PB, MASKED>(st[0], f, rank_group, rank_val0, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
-          sym_step<PB, MASKED>(st[0], f, slot_base, k, valid_lane);
+          sym_step<PB, MASKED>(st[0], f, k, valid_lane);
         } else if constexpr (ILP == 2) {
           field_step_dual<PB, MODE, MASKED>(st[0], st[ILP - 1], f, f & 3, f < 4 ? st[0].coset_base : high[0],
                                             f < 4 ? st[ILP - 1].coset_base : high[ILP - 1], k, valid);
@@ -810,11 +840,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         const Pair& s = st[j];
         float w[8];
         if (__builtin_expect(c.unusual == 0, 1)) {
-          float z[8];
-          lattice_point(s, z);
-          const float shift = __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? c.half_scale : 0.0f;
-#pragma unroll
-          for (int f = 0; f < 8; ++f) w[f] = __fmaf_rn(z[f], c.scale, shift);
+          scaled_point(s, c.scale, __builtin_amdgcn_inverse_ballot_w64(s.coset_mask) ? c.half_scale : 0.0f, w);
         } else {
           weights_of(s, c.scale, w);
         }
@@ -844,13 +870,12 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       if constexpr (DOT_ROWS > 0) dot_prefetch(vector, row, valid_lane, dot_in);
       coset_step_single<PB, MODE, true>(s, k, valid);
       const uint32_t high = s.coset_base + L::kHighBase;
-      const uint32_t slot_base = MODE == kModeSym ? sym_slot_base(s) : 0u;
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
           rank_step<PB, true>(s, f, s.coset_base + rank_rs0, rank_val0, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
-          sym_step<PB, true>(s, f, slot_base, k, valid_lane);
+          sym_step<PB, true>(s, f, k, valid_lane);
         } else {
           field_step_single<PB, MODE, true>(s, f, f & 3, f < 4 ? s.coset_base : high, k, valid);
         }

@@ -45,17 +45,19 @@ __global__ __launch_bounds__(256) void build_sym_tables_kernel(const int32_t* __
   }
   __syncthreads();
   uint32_t running = chunk_sum[tid];
-  // The decode step forms slot | (LDS address of this stream's slot table) and subtracts the second word from
-  // freq * (x >> pb) + that, so the address is folded into the stored cdf.
-  const uint32_t slot_table_at = static_cast<uint32_t>(kSymFbBytes) + (static_cast<uint32_t>(stream - 1) << prob_bits);
-  const uint32_t folded = static_cast<uint32_t>(kSymFbBytes) + ((static_cast<uint32_t>(stream - 1) & 1u) << prob_bits);
+  // The decode step forms slot | (2048 * coset), reads the slot table there, and subtracts the low half of the second
+  // word from freq * (x >> pb) + that, so the coset offset is folded into the stored cdf.
+  const uint32_t slot_table_at = static_cast<uint32_t>(kSymFbBytes) + static_cast<uint32_t>(stream - 1) * kSymSlotStreamBytes;
+  const uint32_t folded = (static_cast<uint32_t>(stream - 1) & 1u) * kSymSlotStreamBytes;
   uint2* fb = reinterpret_cast<uint2*>(section) + (stream - 1) * 256;
   uint8_t* slots = section + slot_table_at;
   for (int s = first; s < last; ++s) {
     const uint32_t f = freq[s];
     if (f == 0) continue;
-    const uint32_t value = static_cast<uint32_t>(s + sym_min + 128);
-    fb[value] = make_uint2(f | (static_cast<uint32_t>(s + sym_min) << 24), running + folded);     // top byte: the value, two's complement
+    const int z = s + sym_min;                                   // in [-128, 127]: exact in half precision
+    const uint32_t value = static_cast<uint32_t>(z + 128);
+    const uint32_t z_half = __builtin_bit_cast(uint16_t, static_cast<_Float16>(z));
+    fb[value] = make_uint2(f | ((z & 1) ? 0x3C000000u : 0u), (running + folded) | (z_half << 16));
     for (uint32_t d = 0; d < f && running + d < size; ++d) slots[running + d] = static_cast<uint8_t>(value);
     running += f;
   }

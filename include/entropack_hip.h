@@ -48,10 +48,12 @@ enum ep_hip_table_kind {
   EP_TABLE_LDS_WIDE = 2,    /* u32 per slot, LDS-resident; prob_bits <= 11, alphabets <= 1024, frequencies < 2048 */
   EP_TABLE_LDS_RANK = 3,    /* LDS-resident rank/select form: per 32 slots a bitmap of symbol ends + running symbol count,
                                per present symbol freq | cdf << 16 and an int16 value; any prob_bits whose tables fit LDS */
-  EP_TABLE_LDS_SYM = 4      /* two-level, LDS-resident: u8 per slot (the value + 128) and, per value, freq | (value & 0xFF) << 24
-                               and cdf; a quarter of LDS_BYTE's size, so two workgroups share a CU. Same conditions as
-                               LDS_BYTE. LDS_BYTE plans at prob_bits 11 carry it as a second section (sym_offset) that
-                               large launches use; as a plan's own kind (force_kind only) every launch uses it */
+  EP_TABLE_LDS_SYM = 4      /* two-level, LDS-resident: u8 per slot (the value + 128) and, per value, one 8-byte entry: freq plus a
+                               parity mark, and cdf plus the value as a half-precision number (the kernel multiplies it with
+                               the row scale without an integer conversion); a quarter of LDS_BYTE's size, so two workgroups
+                               share a CU. Same conditions as LDS_BYTE. LDS_BYTE plans at prob_bits 11 carry it as a second
+                               section (sym_offset) that large launches use; as a plan's own kind (force_kind only) every
+                               launch uses it */
 };
 
 /* Device-side error flag values written (first one wins) to *error_dev by the decode kernels; same meaning as the
