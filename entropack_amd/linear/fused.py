@@ -1,19 +1,41 @@
-"""Forward paths of the compressed linear layers that never call a library GEMM.
+"""`forward_mode="fused"` of the compressed linear layers: what runs for how many activation rows.
 
-One to four activation rows (the memory-bound regime): the decode kernel multiplies every decoded vector with the
-activations in registers, so the dense weight is neither written nor re-read. More rows: the weight is decoded once
-and multiplied on the matrix cores with this package's GEMM; at that size the serial rANS chain of a tile, not memory
-traffic, bounds the decode, and a multiply inside the decode kernel would only slow the GEMM down.
+  rows M            weight written to memory?   kernels
+  1 (and 2..4 on    no                          the decode kernel multiplies every decoded vector with the activations in
+  weights whose                                 registers (`ep_hip_linear_fused_bf16`): the memory-bound regime, where the
+  decode is chain-                              dense weight would be 16 / bpp times the bytes of the container
+  bound anyway)
+  up to 128         yes, once                   decode, then this package's split-K skinny product (`ep_hip_gemm_bf16_skinny`),
+                                                which streams the weight at 75 % of the memory bandwidth
+  more              yes, once                   decode, then a tiled product on the matrix cores: the vendor library's
+                                                (`TILED_PRODUCT = "library"`, the default) or this package's
+                                                (`"own"`, `ep_hip_gemm_bf16`)
+
+Beyond four rows nothing is multiplied inside the decode kernel: a tile is a chain of dependent rANS steps that lasts
+as long whatever is fused behind it, a wave's two tiles hold unrelated (row, k) ranges that form no matrix-core operand,
+and the vector ALU, which the decode saturates, would have to do the multiplying. The default for the tiled product is
+the library because its kernel is the faster one wherever the weight has just been decoded, i.e. is not in any cache:
+3072 x 3072 weight, 256 / 1024 / 4096 rows: 20 / 31 / 63 us against 46 / 46 / 67 us for this package's kernel, which
+keeps less than one K step of loads in flight (with both operands cache-resident the two are within 5 % of each
+other at 4096 rows). The reference has one path for every M: decode, then `F.linear` (entropack/linear/linear.py:163-165).
+
+The forward is differentiable with respect to the activations (like the reference's `F.linear` on a constant weight):
+under autograd the kernels run inside a `torch.autograd.Function` whose backward multiplies the output gradient with
+the decoded weight.
 """
 import torch
+from torch.nn import functional as F
 
 from ..schemes.base import packed_buffers
 from ..schemes.lattice_rans import hip as hip_lane
 from ..schemes.lattice_rans.format import LatticeBuffers
 from . import kernels
 
+#: Which tiled GEMM multiplies more than `kernels.SKINNY_MAX_ROWS` activation rows in fused mode: "library" or "own".
+TILED_PRODUCT = "library"
 
-def linear_forward(layer, x: torch.Tensor) -> torch.Tensor:
+
+def _forward_kernels(layer, x: torch.Tensor) -> torch.Tensor:
     container = layer._container()
     if container.compress_method == "lattice_rans" and container.encoded_dtype == torch.bfloat16:
         on_device = container.to(device=x.device)
@@ -23,7 +45,34 @@ def linear_forward(layer, x: torch.Tensor) -> torch.Tensor:
     weight = layer._decoded_for(x)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("the fused forward runs in bfloat16; use forward_mode='decode_then_gemm' for other dtypes")
+    rows = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    if rows > kernels.SKINNY_MAX_ROWS and TILED_PRODUCT == "library":
+        return F.linear(x, weight, layer._bias_on(x.device))
     return kernels.gemm_bf16(x, weight, layer._bias_on(x.device), out_dtype=x.dtype)
+
+
+class _FusedLinearFunction(torch.autograd.Function):
+    """The fused forward with the input gradient of y = x W^T: grad_x = grad_y W, W decoded again in the backward (the
+    compressed weight and the bias are frozen and get no gradient)."""
+
+    @staticmethod
+    def forward(ctx, x, layer):
+        ctx.layer = layer
+        ctx.input_shape = tuple(x.shape)
+        return _forward_kernels(layer, x.detach())
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        rows = grad_output.reshape(-1, grad_output.shape[-1])
+        dense = ctx.layer.dequantize(rows.device).to(rows.dtype)
+        return (rows @ dense).reshape(ctx.input_shape), None
+
+
+def linear_forward(layer, x: torch.Tensor) -> torch.Tensor:
+    if torch.is_grad_enabled() and x.requires_grad:
+        return _FusedLinearFunction.apply(x, layer)
+    return _forward_kernels(layer, x)
 
 
 def int8_linear_forward(layer, activation: torch.Tensor, activation_scale: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

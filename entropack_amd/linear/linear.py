@@ -8,8 +8,10 @@ the change of hardware forces:
   * decoding selects the `hip` backend (the reference hard-codes "cuda", linear.py:15,58-68); encoding, which the
     reference also runs on its CUDA lane, runs on this package's CPU encoder;
   * `forward` has two modes. "decode_then_gemm" materialises the dense weight with the decode kernel and multiplies
-    with the library GEMM, exactly the reference's data flow. "fused" hands the container to the fused
-    decode-to-GEMM kernel, which never writes the dense weight to HBM;
+    with the library GEMM, exactly the reference's data flow. "fused" picks by the number of activation rows
+    (`linear/fused.py`): for one row (up to four on weights whose decode is chain-bound) the decode kernel multiplies
+    in registers and the dense weight is never written; beyond that the weight is decoded to memory once and
+    multiplied by the split-K skinny product (up to 128 rows) or a tiled matrix-core product;
   * the W8A8 layer gates on a gfx950 device instead of a CUDA compute capability (linear.py:324-336) and its int8
     GEMM + row quantiser are HIP kernels with the semantics of the reference's Triton kernels
     (entropack/linear/quant_kernels.py:15-79).

@@ -68,12 +68,23 @@ def _plan_for(buffers: LatticeBuffers, info: dict) -> DecodePlan:
     return plan
 
 
+_C_INT_MAX = 2 ** 31 - 1
+
+
+def _check_abi_ranges(info: dict) -> None:
+    """The C ABI takes `tile_elements` as a C int. A container's layout holds it as int64, and ctypes would truncate a
+    larger value silently: the library would then derive other tiles than the ones the buffers were checked against."""
+    if not 0 < info["tile_elements"] <= _C_INT_MAX:
+        raise ValueError(f"lattice_rans tile_elements {info['tile_elements']} is outside what the hip lane takes (1 .. 2**31 - 1)")
+
+
 def _checked_geometry(buffers: LatticeBuffers, shape, dtype):
     """(geometry, dtype the kernel stores, decoded via float32?) of one container, after the lane's argument checks."""
     device = buffers.payload.device
     if device.type != "cuda":
         raise RuntimeError(f"the hip lane decodes device buffers only, got {device}")
     info = decode_geometry(buffers._asdict(), shape)
+    _check_abi_ranges(info)
     if buffers.scales.numel() != info["rows"] or buffers.states.numel() != max(1, info["total_tiles"]) * 32 \
             or buffers.offsets.numel() != max(1, info["total_tiles"]) + 1:
         raise ValueError("lattice_rans buffers do not match the container geometry")

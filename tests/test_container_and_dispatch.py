@@ -345,3 +345,31 @@ def test_entry_points_refuse_bad_arguments_before_touching_a_device():
     assert rotate(inner=2048, ldx=2048, group=1024) == EUNSUPPORTED            # a valid group, but not one this kernel rotates
     assert rotate(x=fake + 2) == EUNSUPPORTED                                  # rows it cannot load four elements at a time
     assert lib.ep_hip_quantize_rows(None, 0, 4, 256, 256, fake, fake, None) == EINVAL
+
+
+def test_static_accumulator_entry_point_checks_sizes_on_the_host():
+    """ep_hip_linear_fused_bf16_static refuses what its fixed array cannot hold before it touches a device."""
+    import ctypes
+    lib = hip_backend.library()
+    fake = 0x1000
+    desc = hip_backend.PlanDesc()
+    job = hip_backend.DecodeJob()
+    job.desc = ctypes.pointer(desc)
+    job.rows, job.cols_padded = hip_backend.STATIC_ACCUMULATOR_FLOATS // 4 + 1, 512
+    call = lambda m: lib.ep_hip_linear_fused_bf16_static(ctypes.byref(job), fake, m, 512, None, fake, job.rows, 0, None)
+    assert call(4) == hip_backend.ETOOLARGE
+    assert call(5) == hip_backend.EUNSUPPORTED
+    assert call(0) == hip_backend.EINVAL
+    assert lib.ep_hip_linear_fused_bf16_static(None, fake, 1, 512, None, fake, 512, 0, None) == hip_backend.EINVAL
+    assert lib.ep_hip_error_string(hip_backend.ETOOLARGE) == b"request exceeds the library's fixed scratch buffer"
+
+
+def test_hip_lane_refuses_tile_sizes_the_c_abi_would_truncate():
+    """`tile_elements` is an int64 in the container and a C int at the ABI: the lane must refuse what would not survive
+    the conversion instead of letting the library derive different tiles than the buffers were checked against."""
+    from entropack_amd.schemes.lattice_rans import hip as lane
+    lane._check_abi_ranges({"tile_elements": 16384})
+    lane._check_abi_ranges({"tile_elements": 2 ** 31 - 1})
+    for bad in (2 ** 31, 2 ** 32 + 16384, 2 ** 40):
+        with pytest.raises(ValueError, match="tile_elements"):
+            lane._check_abi_ranges({"tile_elements": bad})

@@ -210,6 +210,35 @@ def test_compressed_linear_small_m_both_modes_agree(m):
         assert rel_l2(y, expect) <= 3 * REL_L2          # few outputs: single final-ulp flips weigh more
 
 
+@pytest.mark.parametrize("m", [1, 4, 256])
+def test_fused_mode_is_differentiable_in_the_activations(m):
+    """The reference's forward is F.linear on a constant weight, so gradients flow to x (entropack/linear/linear.py:163-165).
+    The fused mode's kernels are outside autograd; under it they run in a Function whose backward is grad @ W_dec. The
+    input gradient must equal the decode_then_gemm layer's, which autograd derives from F.linear: the same bf16 product."""
+    print("case fused backward, M =", m, flush=True)
+    plain, _, _ = _c3_layer("decode_then_gemm", rows=512, cols=2048)
+    fused, _, _ = _c3_layer("fused", rows=512, cols=2048)
+    torch.manual_seed(21)
+    x = torch.randn(m, 2048).to(torch.bfloat16).cuda()
+    upstream = torch.randn(m, 512).to(torch.bfloat16).cuda()
+    grads, outputs = [], []
+    for layer in (plain, fused):
+        probe = x.clone().requires_grad_(True)
+        y = layer(probe)
+        assert y.requires_grad
+        y.backward(upstream)
+        grads.append(probe.grad)
+        outputs.append(y.detach())
+    torch.cuda.synchronize()
+    assert grads[1].shape == x.shape and grads[1].dtype == torch.bfloat16
+    want = upstream.float() @ plain.dequantize("cuda").float()
+    assert rel_l2(grads[0], want) <= REL_L2 and rel_l2(grads[1], want) <= REL_L2
+    assert within_one_ulp(grads[1], want.to(torch.bfloat16))
+    assert within_one_ulp(outputs[1], outputs[0])
+    with torch.no_grad():                                            # and without autograd nothing is recorded
+        assert not fused(x.clone().requires_grad_(True)).requires_grad
+
+
 @pytest.mark.parametrize("rows,cols,bpp", [(512, 2048, 4.0), (96, 256, 3.0), (300, 1032, 8.0), (64, 4104, 2.0), (1024, 3072, 5.0)])
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
 def test_fused_rows_never_materialise_the_weight_and_match(rows, cols, bpp, m):
