@@ -22,9 +22,40 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
-#: HBM bytes per decode launch measured with two rocprofv3 --pmc runs of this script (FETCH_SIZE, scaled by the 2.0
-#: a plain 512 MiB copy calibrates it to, plus WRITE_SIZE, factor 1.0): the default workload and the lossless one.
-MEASURED_TRAFFIC_BYTES = {"target": 600_700_000, "tile_ans": 818_700_000}
+#: HBM bytes per decode launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE, scaled by the factor a plain
+#: 512 MiB copy in the same run calibrates it to, plus WRITE_SIZE): a measurement of the kernels as they were when the
+#: named profile was taken. `csrc_sha16` names those sources; when the kernels have changed since, the figure is not
+#: reported (`traffic` is null and `traffic_source` says why) instead of going stale silently.
+MEASURED_TRAFFIC = {
+    "target": {"bytes": 600_700_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "unset"},
+    "tile_ans": {"bytes": 818_700_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "unset"},
+}
+#: The kernel sources a traffic figure depends on, per workload.
+TRAFFIC_SOURCES = {
+    "target": ("ep_common.hpp", "ep_store.hpp", "ep_decode_lds.hpp", "ep_decode_lds.hip", "ep_decode_sym.hip", "ep_plan.hip"),
+    "tile_ans": ("ep_common.hpp", "ep_decode_lds.hpp", "ep_tile_ans.hip"),
+}
+
+
+def csrc_sha16(workload):
+    import hashlib
+    digest = hashlib.sha256()
+    for name in TRAFFIC_SOURCES[workload]:
+        with open(os.path.join(ROOT, "entropack_amd", "csrc", name), "rb") as handle:
+            digest.update(handle.read())
+    return digest.hexdigest()[:16]
+
+
+def measured_traffic(workload, forced_kind=None):
+    """(`traffic`, `traffic_source`) of a roofline entry."""
+    entry = MEASURED_TRAFFIC.get(workload)
+    if entry is None or forced_kind is not None:
+        return None, "not measured for this workload"
+    now = csrc_sha16(workload)
+    if now != entry["csrc_sha16"]:
+        return None, f"{entry['profile']} holds {entry['bytes']} bytes for kernel sources {entry['csrc_sha16']}; they are {now} now"
+    return entry["bytes"], f"{entry['profile']} (kernel sources {now})"
+
 
 WORKLOADS = {
     # name: (rows, cols, sigma, seed, target_bpp, outliers)
@@ -123,9 +154,14 @@ def linear_section(ep, steps):
     x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
     flops = 2.0 * 4096 * 3072 * 3072
     out = {"workload": "CompressedLinear 3072x3072 @ 4.0 bpp + bias, X [4096, 3072] bf16, seed 2", "flops": flops}
+    from entropack_amd.linear import fused as fused_mode
     reference = None
-    for mode in ("decode_then_gemm", "fused"):
+    # `fused_own_gemm` = the fused mode made to multiply with this library's tiled kernel instead of the vendor library's
+    # (fused.TILED_PRODUCT = "own"); the mode's default is the faster of the two on a freshly decoded weight.
+    variants = (("decode_then_gemm", "decode_then_gemm", "library"), ("fused", "fused", "library"), ("fused_own_gemm", "fused", "own"))
+    for name, mode, product in variants:
         layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
+        fused_mode.TILED_PRODUCT = product
         y = layer(x)
         if reference is None:
             weight = layer.dequantize("cuda")
@@ -134,20 +170,21 @@ def linear_section(ep, steps):
             out["decode_ms"] = round(decode_ms, 5)
         rel = ((y.double() - reference).norm() / reference.norm()).item()
         ms = _median_ms(lambda: layer(x), steps)
-        out[mode] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2),
+        out[name] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2),
                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5), "rel_l2_vs_f32_reference": rel}
-    # Fewer activation rows than the configuration names, between the 128 of the streaming kernel and the 4096 above:
-    # the products of this library's tiled kernels (`fused`) beside the vendor library's (`decode_then_gemm`).
+    # Fewer activation rows than the configuration names, between the 128 of the streaming kernel and the 4096 above.
     out["fewer_rows"] = {}
     for rows in (256, 1024):
         part = x[:rows].contiguous()
         entry = {}
-        for mode in ("decode_then_gemm", "fused"):
+        for name, mode, product in variants:
             layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
+            fused_mode.TILED_PRODUCT = product
             got = layer(part).double()
-            entry[mode] = {"ms": round(_median_ms(lambda: layer(part), steps), 5),
+            entry[name] = {"ms": round(_median_ms(lambda: layer(part), steps), 5),
                            "rel_l2_vs_f32_reference": ((got - reference[:rows]).norm() / reference[:rows].norm()).item()}
         out["fewer_rows"][f"M={rows}"] = entry
+    fused_mode.TILED_PRODUCT = "library"
     # The same layer encoded with tiles a quarter and an eighth of the default size (`tile_elements`, a field of the
     # reference's config): a tile's chain of dependent steps, which is all a single layer's decode waits for, shortens
     # in proportion, for a per-tile header that costs 1-3 % more stored bits.
@@ -267,6 +304,10 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
     weights = [layer.dequantize("cuda") for layer in layers[:distinct]]
     out["dense_gemm_only"] = priced(_median_ms(lambda: [torch.nn.functional.linear(x, weights[i % distinct], layers[i].bias)
                                                         for i in range(layers_total)], max(3, steps // 5), warmup=2))
+    from entropack_amd.linear import fused as fused_mode
+    from entropack_amd.linear import kernels
+    out["dense_own_gemm_only"] = priced(_median_ms(lambda: [kernels.gemm_bf16(x, weights[i % distinct], layers[i].bias)
+                                                            for i in range(layers_total)], max(3, steps // 5), warmup=2))
     del weights
     # `beside`: groups decode on a second stream while the previous group multiplies (two arenas); `in_line`: on the
     # layers' own stream between two groups (one arena).
@@ -280,6 +321,24 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
             entry["dense_bytes_held"] = ahead.arena_bytes
             ahead.check_errors()
         out[f"decode_ahead_group_{group}" + ("" if overlap else "_in_line")] = entry
+    # The same stack multiplied by this library's tiled kernel (fused mode, TILED_PRODUCT = "own") instead of the vendor's.
+    for layer in layers:
+        layer.forward_mode = "fused"
+    fused_mode.TILED_PRODUCT = "own"
+    try:
+        own_reference = forward()
+        rel = ((own_reference.double() - reference.double()).norm() / reference.double().norm()).item()
+        with ep.DecodeAhead(layers, group_size=16, overlap=False) as ahead:
+            same = bool(torch.equal(forward(), own_reference))
+            entry = priced(_median_ms(forward, max(3, steps // 5), warmup=2))
+            entry["identical_to_layer_by_layer"] = same
+            entry["rel_l2_vs_library_product"] = rel
+            ahead.check_errors()
+        out["decode_ahead_group_16_in_line_own_gemm"] = entry
+    finally:
+        fused_mode.TILED_PRODUCT = "library"
+        for layer in layers:
+            layer.forward_mode = "decode_then_gemm"
     return out
 
 
@@ -415,7 +474,100 @@ def stack_workload(args, ep):
             "value": round(cpu_bytes / cpu_seconds / 1e9, 4), "unit": "GB/s", "cores": min(16, os.cpu_count() or 1), "kind": "port",
             "sample": f"the first 5 layers (one per rate), C port of the reference CPU decoder, OpenMP, {cpu_seconds:.2f} s"}
     print(json.dumps(result))
-    return 0
+    return 0 if parity_holds(result) else 1
+
+
+def decode_case(ep, name, steps, warmup, check):
+    """One decode-only configuration (a row of `decode_configs`): encode on the host, decode on the device, time the
+    launches with HIP events, compare the result with the C oracle bit for bit."""
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    from entropack_amd.schemes.lattice_rans.format import LatticeBuffers
+    rows, cols, sigma, seed, bpp, outliers = WORKLOADS[name]
+    container = ep.compress(make_weight(rows, cols, sigma, seed, outliers), ep.EntroPackLossyConfig(target_bpp=bpp, execution_backend="eager"))
+    on_gpu = container.to("cuda")
+    lattice = LatticeBuffers(**{key: on_gpu.buffers[key] for key in LatticeBuffers._fields})
+    cols_padded = int(container.buffers["layout"][0])
+    alg_bytes = algorithmic_bytes(container.buffers, rows, cols_padded, 2)
+
+    def step():
+        return hip_lane.decode(lattice, shape=(rows, cols), dtype=torch.bfloat16)
+
+    for _ in range(max(warmup, 1)):
+        dense = step()
+    torch.cuda.synchronize()
+    hip_lane.check_errors(lattice)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for begin, end in events:
+        begin.record()
+        dense = step()
+        end.record()
+    torch.cuda.synchronize()
+    kernel_ms = sorted(begin.elapsed_time(end) for begin, end in events)
+    avg_ms = sum(kernel_ms) / len(kernel_ms)
+    entry = {
+        "workload": f"{rows}x{cols} N(0,{sigma}) seed {seed}{' +0.1% x20 outliers' if outliers else ''} @ {bpp} bpp -> bf16",
+        "tiles": int(lattice.states.shape[0]), "prob_bits": int(container.buffers["layout"][1]),
+        "table_kind": hip_lane.launch_table_kind(lattice, shape=(rows, cols), dtype=torch.bfloat16),
+        "algorithmic_bytes": alg_bytes, "kernel_ms_avg": round(avg_ms, 5), "GBps": round(alg_bytes / avg_ms / 1e6, 1),
+        "frac_of_hbm_peak": round(alg_bytes / avg_ms / 1e6 / HBM_PEAK_GBPS, 5), "params_per_s": round(rows * cols / (avg_ms * 1e-3), 1),
+    }
+    if check:
+        from oracle import c_oracle
+        c_oracle.load()
+        expect = c_oracle.decode(host_arrays(container.buffers), (rows, cols_padded), "bfloat16", threads=min(16, os.cpu_count() or 1))
+        entry["bit_exact_vs_oracle"] = bool(np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), expect[:, :cols]))
+    return entry
+
+
+def stack_case(ep, steps, check):
+    """Configuration 4 inside the default run: 120 layers, rates round-robin, one batched pass. The 20 distinct
+    (shape, rate) pairs are encoded once from one N(0, 0.02) weight per shape and every pair is placed on the device six
+    times, as six layers with buffers and plans of their own: the decode work of the configuration without 120 encodes
+    (`--workload c4` encodes 120 different weights)."""
+    torch.manual_seed(3)
+    weights = [(torch.randn(rows, cols) * 0.02).to(torch.bfloat16) for rows, cols in STACK_SHAPES]
+    distinct = {}
+    for index in range(20):
+        distinct[index % 4, index % 5] = ep.compress(weights[index % 4], ep.EntroPackLossyConfig(target_bpp=STACK_RATES[index % 5],
+                                                                                                 execution_backend="eager"))
+    del weights
+    keys = [(index % 4, index % 5) for index in range(120)]
+    containers = [distinct[key].to("cuda") for key in keys]
+    params = sum(STACK_SHAPES[key[0]][0] * STACK_SHAPES[key[0]][1] for key in keys)
+    alg_bytes = sum(algorithmic_bytes(distinct[key].buffers, STACK_SHAPES[key[0]][0], int(distinct[key].buffers["layout"][0]), 2) for key in keys)
+    config = ep.EntroPackLossyConfig(execution_backend="hip")
+    torch.cuda.synchronize()
+    plan_started = time.perf_counter()
+    batch = ep.BatchDecompressor(containers, config)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - plan_started) * 1e3
+    arena = torch.empty(batch.arena_bytes, dtype=torch.uint8, device="cuda")
+    dense = batch(arena)
+    torch.cuda.synchronize()
+    batch.check_errors()
+    ms = _median_ms(lambda: batch(arena), max(5, steps // 5), warmup=2)
+    entry = {
+        "workload": "120 layers {11520x3840, 3840x3840, 10240x3840, 3840x10240} N(0,0.02) seed 3, rates [2.3, 4, 5, 6, 8] round-robin, "
+                    "one batched pass (20 distinct containers, six device copies each)",
+        "layers": len(containers), "params": params, "algorithmic_bytes": alg_bytes, "ms_per_pass": round(ms, 4),
+        "GBps": round(alg_bytes / ms / 1e6, 1), "frac_of_hbm_peak": round(alg_bytes / ms / 1e6 / HBM_PEAK_GBPS, 5),
+        "params_per_s": round(params / (ms * 1e-3), 1), "plan_build_ms_once": round(plan_ms, 2),
+    }
+    if check:
+        from oracle import c_oracle
+        c_oracle.load()
+        exact = True
+        for index in range(20):
+            key = keys[index]
+            rows, cols = STACK_SHAPES[key[0]]
+            expect = c_oracle.decode(host_arrays(distinct[key].buffers), (rows, int(distinct[key].buffers["layout"][0])), "bfloat16",
+                                     threads=min(16, os.cpu_count() or 1))
+            got = dense[index].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+            exact = exact and bool(np.array_equal(got, expect[:, :cols]))
+        for index in range(20, 120):                                  # the other copies against the checked ones
+            exact = exact and bool(torch.equal(dense[index].view(torch.int16), dense[index % 20].view(torch.int16)))
+        entry["bit_exact_vs_oracle"] = exact
+    return entry
 
 
 def lossless_workload(args, ep):
@@ -466,7 +618,8 @@ def lossless_workload(args, ep):
         },
         "roofline": {
             "bound": "hbm", "achieved": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9, 3), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": MEASURED_TRAFFIC_BYTES["tile_ans"],
+            "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5), "traffic": measured_traffic("tile_ans")[0],
+            "traffic_source": measured_traffic("tile_ans")[1],
             "kernel_ms_avg": round(kernel_avg_ms, 5), "kernel_ms_median": round(kernel_ms[len(kernel_ms) // 2], 5),
         },
     }
@@ -485,7 +638,7 @@ def lossless_workload(args, ep):
             "sample": f"whole container, C port of the reference CPU decoder, {threads} OpenMP threads, best of 2, {best:.3f} s"}
         result["config"]["bit_exact_vs_oracle"] = bool(np.array_equal(dense.view(torch.uint8).cpu().numpy().reshape(-1), expect))
     print(json.dumps(result))
-    return 0
+    return 0 if parity_holds(result) else 1
 
 
 def main():
@@ -497,6 +650,7 @@ def main():
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
+    parser.add_argument("--no-configs", action="store_true", help="skip the decode_configs section (c2, c5a, c5b, c4) of the default run")
     parser.add_argument("--copy-probe-mib", type=int, default=0,
                         help="also run one plain device copy of this many MiB (calibrates FETCH_SIZE / WRITE_SIZE counters)")
     parser.add_argument("--prob-bits", type=int, default=None, help="encode with this prob_bits instead of the rate's default")
@@ -576,7 +730,7 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9, 3), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.table_kind is None else None,
+            "traffic": measured_traffic(args.workload, args.table_kind)[0], "traffic_source": measured_traffic(args.workload, args.table_kind)[1],
             "kernel_ms_avg": round(kernel_avg_ms, 5), "kernel_ms_median": round(kernel_ms[len(kernel_ms) // 2], 5),
         },
     }
@@ -596,8 +750,32 @@ def main():
         result["cpu_python_loop"] = python_loop_baseline(host, rows, cols_padded, alg_bytes)
         got = dense.view(torch.int16).cpu().numpy().view(np.uint16)
         result["config"]["bit_exact_vs_oracle"] = bool(np.array_equal(got, expect[:, :cols]))
+        del host, expect, got
+    del dense
+    if args.workload == "target" and not args.no_configs:
+        # The other decode configurations of the benchmark, each on its own container, checked like the headline.
+        del on_gpu, lattice, container
+        torch.cuda.empty_cache()
+        configs = {}
+        for name in ("c2", "c5a", "c5b"):
+            configs[name] = decode_case(ep, name, max(10, args.steps // 2), args.warmup, not args.no_cpu)
+            torch.cuda.empty_cache()
+        configs["c4"] = stack_case(ep, args.steps, not args.no_cpu)
+        result["decode_configs"] = configs
     print(json.dumps(result))
-    return 0
+    return 0 if parity_holds(result) else 1
+
+
+def parity_holds(node):
+    """False when any `bit_exact...` / `identical...` / `lossless` flag anywhere in a result is false."""
+    if isinstance(node, dict):
+        for key, value in node.items():
+            if isinstance(value, bool) and (key.startswith("bit_exact") or key.startswith("identical") or key == "lossless") and not value:
+                print(f"bench.py: parity check failed: {key}", file=sys.stderr)
+                return False
+            if not parity_holds(value):
+                return False
+    return True
 
 
 if __name__ == "__main__":
