@@ -501,21 +501,42 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   const uint32_t rings0 = lds0 + lut_bytes;
   const uint32_t minima0 = rings0 + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes;
 
-  {
-    const uint4* src = reinterpret_cast<const uint4*>(MODE == kModeSym ? a.sym_tables : reinterpret_cast<const uint8_t*>(a.plan) + kHeaderBytes);
-    uint4* dst = reinterpret_cast<uint4*>(smem);
-    const uint32_t quads = (MODE == kModeRank ? a.lut_bytes : lut_bytes) / 16;
-    for (uint32_t i = threadIdx.x; i < quads; i += blockDim.x) dst[i] = src[i];
-    if (threadIdx.x < kStreams) {
-      reinterpret_cast<int32_t*>(smem + lut_bytes + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes)[threadIdx.x] =
-          static_cast<int32_t>(a.plan[kHdrSymMin + threadIdx.x]);
-    }
-  }
-  __syncthreads();
   if (lds0 != 0) {      // the steps address the tables from LDS offset 0 and OR table bases into slot offsets
     if (threadIdx.x == 0) flag_error(a.error, EP_DECODE_BAD_OFFSETS);
     return;
   }
+  // Staging the tables. The slot-table forms are whole KiB: they are loaded straight into LDS (one wave instruction
+  // moves 1 KiB, lane l the 16 bytes at 16 l, no registers in between), and the loads are left in flight while the
+  // wave sets its first tiles up (offsets, states and payload chunks: two dependent trips to memory); the wait and the
+  // barrier that publish the tables come after that set-up, inside the loop below. The rank/select tables have any
+  // multiple of 16 bytes and are copied through registers.
+  constexpr bool kStageDirect = MODE != kModeRank;
+  {
+    const uint8_t* src = MODE == kModeSym ? a.sym_tables : reinterpret_cast<const uint8_t*>(a.plan) + kHeaderBytes;
+    if (threadIdx.x < kStreams) {
+      reinterpret_cast<int32_t*>(smem + lut_bytes + static_cast<uint32_t>(waves) * ILP * 2 * kRingBytes)[threadIdx.x] =
+          static_cast<int32_t>(a.plan[kHdrSymMin + threadIdx.x]);
+    }
+    if constexpr (kStageDirect) {
+      static_assert(L::kLutBytes % 1024 == 0 && sym_table_bytes(PB) % 1024 == 0, "slot tables are whole KiB");
+      for (uint32_t kib = static_cast<uint32_t>(wave); kib < lut_bytes / 1024u; kib += static_cast<uint32_t>(waves)) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + kib * 1024u + static_cast<uint32_t>(lane) * 16u),
+                                         (__attribute__((address_space(3))) void*)(smem + kib * 1024u), 16, 0, 0);
+      }
+    } else {
+      const uint4* from = reinterpret_cast<const uint4*>(src);
+      uint4* dst = reinterpret_cast<uint4*>(smem);
+      for (uint32_t i = threadIdx.x; i < a.lut_bytes / 16; i += blockDim.x) dst[i] = from[i];
+    }
+  }
+  bool tables_published = false;
+  auto publish_tables = [&]() {
+    if (!tables_published) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): this wave's part of the tables has landed
+      __syncthreads();
+      tables_published = true;
+    }
+  };
 
   StepConsts k;
   k.f0s = uniform(a.plan[kHdrCosetFreq0]);
@@ -567,6 +588,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       open_window(s, window_at, word_begin, word_end, s.count > 0, a.payload, a.payload_words, a.offsets, l32);
     }
     const bool all_full = __builtin_amdgcn_readfirstlane(__all(full) ? 1 : 0) != 0;
+    publish_tables();
 
     // After a step: a half whose position fell below 64 slides its window down by 64 words. All 32 lanes of the half
     // (voting or not) move their dword of the lower chunk up, drop their prefetched dword in its place and ask for
@@ -944,6 +966,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       }
     }
   }
+  publish_tables();      // a wave without tiles still takes part in the workgroup's barrier
 }
 
 // One container spread over the whole grid.

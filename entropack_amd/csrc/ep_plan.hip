@@ -10,56 +10,78 @@ static thread_local int g_last_runtime_error = 0;
 
 void set_runtime_error(hipError_t e) { g_last_runtime_error = static_cast<int>(e); }
 
-// One block per stream. Threads split the alphabet into contiguous chunks, scan the chunk sums, then each
-// thread writes the slot entries of its own symbols, so slot ranges are disjoint and no atomics are needed.
 __global__ __launch_bounds__(256) void zero_fill_kernel(uint4* __restrict__ p, size_t quads) {
   for (size_t i = blockIdx.x * size_t{256} + threadIdx.x; i < quads; i += gridDim.x * size_t{256}) p[i] = make_uint4(0, 0, 0, 0);
 }
 
-// LDS_SYM section of a byte-valued plan: one block per field stream, same chunked scan as below.
+// The table builders run one block of 256 threads per stream. Threads split the alphabet into contiguous chunks and
+// scan the chunk sums, which gives every symbol its cumulative frequency; the slots are then filled slot by slot (thread
+// t takes slots t, t + 256, ...), each finding its symbol by bisection of the cumulative frequencies kept in LDS, so the
+// work is even however skewed the frequencies are. (Filling symbol by symbol left one thread writing the hundreds of
+// slots of the likeliest symbol while the others idled: 55 us per container against 6 us.)
+constexpr int kScanThreads = 256;
+constexpr int kCdfInLds = 4096;          // alphabets up to this size keep their cumulative frequencies in LDS
+
+// Exclusive prefix sums of one value per thread over the block, in place in `values` (256 entries of LDS).
+__device__ __forceinline__ void block_exclusive_scan(uint32_t* values, int tid) {
+  __syncthreads();
+  const uint32_t own = values[tid];
+  uint32_t sum = own;
+  for (int step = 1; step < kScanThreads; step <<= 1) {
+    const uint32_t below = tid >= step ? values[tid - step] : 0u;
+    __syncthreads();
+    sum += below;
+    values[tid] = sum;
+    __syncthreads();
+  }
+  values[tid] = sum - own;
+  __syncthreads();
+}
+
+// Symbol of `slot`: the last symbol whose cumulative frequency is at most `slot`; cdf[0 .. alphabet] ascending, cdf[0] = 0,
+// cdf[alphabet] = table size. Symbols of frequency zero share their neighbour's value and are never the answer.
+__device__ __forceinline__ int symbol_of_slot(const uint32_t* cdf, int alphabet, uint32_t slot) {
+  int low = 0, high = alphabet;          // cdf[low] <= slot < cdf[high]
+  while (high - low > 1) {
+    const int mid = (low + high) >> 1;
+    if (cdf[mid] <= slot) low = mid; else high = mid;
+  }
+  return low;
+}
+
+// LDS_SYM section of a byte-valued plan: one block per field stream.
 __global__ __launch_bounds__(256) void build_sym_tables_kernel(const int32_t* __restrict__ meta, const uint16_t* __restrict__ freq_tables,
                                                                int prob_bits, uint8_t* __restrict__ section) {
-  __shared__ uint32_t chunk_sum[256];
+  __shared__ uint32_t chunk_sum[kScanThreads];
+  __shared__ uint32_t cdf[256 + 1];
   const int stream = blockIdx.x + 1;
   const int tid = threadIdx.x;
   const uint32_t size = 1u << prob_bits;
   const int sym_min = meta[stream * kMetaWidth + 1];
   const int freq_off = meta[stream * kMetaWidth + 2];
   const int alphabet = meta[stream * kMetaWidth + 3];
-  if (alphabet <= 0) return;
+  if (alphabet <= 0 || alphabet > 256) return;            // byte-valued plans have alphabets of at most 256 symbols
   const uint16_t* freq = freq_tables + freq_off;
-  const int per = (alphabet + 255) / 256;
-  const int first = tid * per;
-  const int last = first + per < alphabet ? first + per : alphabet;
-  uint32_t local = 0;
-  for (int s = first; s < last; ++s) local += freq[s];
-  chunk_sum[tid] = local;
-  __syncthreads();
-  if (tid == 0) {
-    uint32_t running = 0;
-    for (int i = 0; i < 256; ++i) {
-      const uint32_t v = chunk_sum[i];
-      chunk_sum[i] = running;
-      running += v;
-    }
-  }
-  __syncthreads();
-  uint32_t running = chunk_sum[tid];
+  const uint32_t f = tid < alphabet ? freq[tid] : 0u;     // one symbol per thread
+  chunk_sum[tid] = f;
+  block_exclusive_scan(chunk_sum, tid);
+  const uint32_t begin = chunk_sum[tid];
+  if (tid < alphabet) cdf[tid] = begin;
+  if (tid == 0) cdf[alphabet] = size;
   // The decode step forms slot | (2048 * coset), reads the slot table there, and subtracts the low half of the second
   // word from freq * (x >> pb) + that, so the coset offset is folded into the stored cdf.
   const uint32_t slot_table_at = static_cast<uint32_t>(kSymFbBytes) + static_cast<uint32_t>(stream - 1) * kSymSlotStreamBytes;
   const uint32_t folded = (static_cast<uint32_t>(stream - 1) & 1u) * kSymSlotStreamBytes;
   uint2* fb = reinterpret_cast<uint2*>(section) + (stream - 1) * 256;
   uint8_t* slots = section + slot_table_at;
-  for (int s = first; s < last; ++s) {
-    const uint32_t f = freq[s];
-    if (f == 0) continue;
-    const int z = s + sym_min;                                   // in [-128, 127]: exact in half precision
-    const uint32_t value = static_cast<uint32_t>(z + 128);
+  if (tid < alphabet && f != 0) {
+    const int z = tid + sym_min;                                 // in [-128, 127]: exact in half precision
     const uint32_t z_half = __builtin_bit_cast(uint16_t, static_cast<_Float16>(z));
-    fb[value] = make_uint2(f | ((z & 1) ? 0x3C000000u : 0u), (running + folded) | (z_half << 16));
-    for (uint32_t d = 0; d < f && running + d < size; ++d) slots[running + d] = static_cast<uint8_t>(value);
-    running += f;
+    fb[z + 128] = make_uint2(f | ((z & 1) ? 0x3C000000u : 0u), (begin + folded) | (z_half << 16));
+  }
+  __syncthreads();
+  for (uint32_t slot = tid; slot < size; slot += kScanThreads) {
+    slots[slot] = static_cast<uint8_t>(symbol_of_slot(cdf, alphabet, slot) + sym_min + 128);
   }
 }
 
@@ -72,8 +94,9 @@ struct RankLayout {
 __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __restrict__ meta,
                                                            const uint16_t* __restrict__ freq_tables, int kind,
                                                            int prob_bits, uint32_t* __restrict__ plan, RankLayout rank) {
-  __shared__ uint32_t chunk_sum[256];
-  __shared__ uint32_t chunk_present[256];
+  __shared__ uint32_t chunk_sum[kScanThreads];
+  __shared__ uint32_t chunk_present[kScanThreads];
+  __shared__ uint32_t cdf[kCdfInLds + 1];
   const int stream = blockIdx.x;
   const int tid = threadIdx.x;
   const uint32_t size = 1u << prob_bits;
@@ -96,7 +119,7 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
   if (alphabet <= 0) return;
 
   const uint16_t* freq = freq_tables + freq_off;
-  const int per = (alphabet + 255) / 256;
+  const int per = (alphabet + kScanThreads - 1) / kScanThreads;
   const int first = tid * per;
   const int last = first + per < alphabet ? first + per : alphabet;
   uint32_t local = 0, local_present = 0;
@@ -106,18 +129,8 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
   }
   chunk_sum[tid] = local;
   chunk_present[tid] = local_present;
-  __syncthreads();
-  if (tid == 0) {
-    uint32_t running = 0, seen = 0;
-    for (int i = 0; i < 256; ++i) {
-      const uint32_t v = chunk_sum[i], n = chunk_present[i];
-      chunk_sum[i] = running;
-      chunk_present[i] = seen;
-      running += v;
-      seen += n;
-    }
-  }
-  __syncthreads();
+  block_exclusive_scan(chunk_sum, tid);
+  block_exclusive_scan(chunk_present, tid);
   uint32_t running = chunk_sum[tid];
   uint8_t* tables = reinterpret_cast<uint8_t*>(plan) + kHeaderBytes;
   if (kind == EP_TABLE_LDS_RANK) {
@@ -138,31 +151,52 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
     }
     __threadfence_block();
     __syncthreads();
-    if (tid == 0) {
-      uint32_t before = static_cast<uint32_t>(rank.present_offset[stream]);
-      for (uint32_t w = 0; w < size / 32; ++w) {
-        rs[w * 2 + 1] = before;
-        before += __popc(rs[w * 2]);
-      }
+    // Symbols that end before each word: a scan of the words' bit counts, 256 words at a time.
+    uint32_t carried = static_cast<uint32_t>(rank.present_offset[stream]);
+    for (uint32_t base = 0; base < size / 32; base += kScanThreads) {
+      const uint32_t w = base + static_cast<uint32_t>(tid);
+      const uint32_t bits = w < size / 32 ? static_cast<uint32_t>(__popc(rs[w * 2])) : 0u;
+      chunk_sum[tid] = bits;
+      block_exclusive_scan(chunk_sum, tid);
+      if (w < size / 32) rs[w * 2 + 1] = carried + chunk_sum[tid];
+      const uint32_t total = chunk_sum[kScanThreads - 1] + __shfl(bits, 63);      // meaningful in the last wave only
+      __syncthreads();
+      if (tid == kScanThreads - 1) chunk_present[0] = total;
+      __syncthreads();
+      carried += chunk_present[0];
+      __syncthreads();
     }
     return;
   }
-  for (int s = first; s < last; ++s) {
-    const uint32_t f = freq[s];
-    for (uint32_t d = 0; d < f && running + d < size; ++d) {
-      const uint32_t slot = running + d;
-      if (kind == EP_TABLE_GLOBAL64) {
-        uint64_t* lut = reinterpret_cast<uint64_t*>(tables) + (static_cast<size_t>(stream) << prob_bits);
-        lut[slot] = (static_cast<uint64_t>(d) << 32) | (static_cast<uint64_t>(f) << 16) | static_cast<uint64_t>(s);
+  auto entry_of = [&](uint32_t slot, uint32_t s, uint32_t f, uint32_t d) {
+    if (kind == EP_TABLE_GLOBAL64) {
+      uint64_t* lut = reinterpret_cast<uint64_t*>(tables) + (static_cast<size_t>(stream) << prob_bits);
+      lut[slot] = (static_cast<uint64_t>(d) << 32) | (static_cast<uint64_t>(f) << 16) | static_cast<uint64_t>(s);
+    } else {
+      uint32_t* lut = reinterpret_cast<uint32_t*>(tables) + (static_cast<size_t>(stream - 1) << prob_bits);
+      if (kind == EP_TABLE_LDS_BYTE) {
+        lut[slot] = f | (d << 12) | (static_cast<uint32_t>(static_cast<int>(s) + sym_min) << 24);     // top byte: the value, two's complement
       } else {
-        uint32_t* lut = reinterpret_cast<uint32_t*>(tables) + (static_cast<size_t>(stream - 1) << prob_bits);
-        if (kind == EP_TABLE_LDS_BYTE) {
-          lut[slot] = f | (d << 12) | (static_cast<uint32_t>(s + sym_min) << 24);     // top byte: the value, two's complement
-        } else {
-          lut[slot] = f | (d << 11) | (static_cast<uint32_t>(s) << 22);
-        }
+        lut[slot] = f | (d << 11) | (s << 22);
       }
     }
+  };
+  if (alphabet <= kCdfInLds) {
+    for (int s = first; s < last; ++s) {
+      cdf[s] = running;
+      running += freq[s];
+    }
+    if (tid == 0) cdf[alphabet] = size;
+    __syncthreads();
+    for (uint32_t slot = tid; slot < size; slot += kScanThreads) {
+      const uint32_t s = static_cast<uint32_t>(symbol_of_slot(cdf, alphabet, slot));
+      entry_of(slot, s, cdf[s + 1] - cdf[s], slot - cdf[s]);
+    }
+    return;
+  }
+  for (int s = first; s < last; ++s) {      // very large alphabets (global tables only): symbol by symbol
+    const uint32_t f = freq[s];
+    for (uint32_t d = 0; d < f && running + d < size; ++d) entry_of(running + d, static_cast<uint32_t>(s), f, d);
     running += f;
   }
 }

@@ -111,6 +111,15 @@ def _rules(config_class: type) -> tuple:
     return _compiled[config_class]
 
 
+_last_valid: list = [None, None]      # the config object validated last and the field values it had then
+
+
 def validate_config(config) -> None:
+    # A layer validates the same config object on every forward: skip the rules while its fields are unchanged.
+    fields = getattr(config, "__dict__", None)
+    if fields is not None and _last_valid[0] is config and _last_valid[1] == fields:
+        return
     for rule in _rules(type(config)):
         rule.apply(getattr(config, rule.name))
+    if fields is not None:
+        _last_valid[0], _last_valid[1] = config, dict(fields)
