@@ -1,6 +1,6 @@
 """Headline benchmark: lossy (lattice_rans) decode throughput on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm]
 
 One "step" = one decode of the whole container (entropy decode + E8 reconstruction + BF16 store) from buffers
 already resident in HBM. Prints ONE JSON line. `value` = algorithmic bytes (container bytes read + dense bytes
@@ -570,6 +570,69 @@ def stack_case(ep, steps, check):
     return entry
 
 
+def gemm_workload(args, ep):
+    """The tiled bf16 products on their own: this library's kernel and the vendor library's on the config-3 layer shape
+    (N = K = 3072) at 256, 1024 and 4096 activation rows, once with one weight used over and over (operands resident in
+    the caches) and once rotating through enough different weights that each one comes from memory, as a weight fresh from
+    the decoder does; then the same product at M = 4096 against K, which separates the per-launch cost from the cost of
+    a K step. Device times from events around each launch with the queue kept busy by a spin kernel in front."""
+    from torch.nn import functional as F
+    from entropack_amd.linear import kernels
+    torch.manual_seed(0)
+
+    def timed(fn, count=30):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(count):
+            torch.cuda._sleep(200000)                  # the launch below is queued behind this: no host latency in the events
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            fn()
+            end.record()
+            torch.cuda.synchronize()
+            times.append(begin.elapsed_time(end) * 1e3)
+        times.sort()
+        return round(times[len(times) // 2], 2)
+
+    n = k = 3072
+    weights = [(torch.randn(n, k, device="cuda") * 0.02).to(torch.bfloat16) for _ in range(24)]      # 453 MB: more than the 256 MB last-level cache
+    rows_out = {}
+    for m in (256, 1024, 4096):
+        x = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+        entry = {}
+        for name, product in (("own", lambda w: kernels.gemm_bf16(x, w, None)), ("library", lambda w: F.linear(x, w))):
+            turn = [0]
+
+            def rotating():
+                turn[0] = (turn[0] + 1) % len(weights)
+                return product(weights[turn[0]])
+
+            entry[name] = {"same_weight_us": timed(lambda: product(weights[0])), "rotating_weights_us": timed(rotating)}
+        entry["bit_identical_products"] = bool(torch.equal(kernels.gemm_bf16(x, weights[0], None), F.linear(x, weights[0])))
+        rows_out[f"M={m}"] = entry
+    del weights
+    sweep = {}
+    for inner in (64, 256, 1024, 2048, 3072, 6144):
+        x = torch.randn(4096, inner, device="cuda").to(torch.bfloat16)
+        w = (torch.randn(n, inner, device="cuda") * 0.02).to(torch.bfloat16)
+        sweep[f"K={inner}"] = {"own_us": timed(lambda: kernels.gemm_bf16(x, w, None)), "library_us": timed(lambda: F.linear(x, w))}
+    flops = 2.0 * 4096 * n * k
+    own = rows_out["M=4096"]["own"]["rotating_weights_us"]
+    result = {
+        "metric": "bf16 GEMM TFLOP/s, 4096 x 3072 x 3072, weight from memory", "value": round(flops / own / 1e6, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": 30, "warmup": 3, "ms_per_step": round(own / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "y = x W^T, N = K = 3072, bf16, f32 accumulation; own kernel (ep_hip_gemm_bf16) beside the vendor library's",
+                   "by_rows": rows_out, "by_inner_size_at_M_4096": sweep},
+        "roofline": {"bound": "mfma", "achieved": round(flops / own / 1e6, 2), "peak": MFMA_PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / own / 1e6 / MFMA_PEAK_BF16_TFLOPS, 5), "traffic": None},
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def lossless_workload(args, ep):
     """The lossless neighbour of the target: tile_ans decode of 8192 x 28672 bf16 N(0, 0.015) seed 4 (the reference's
     default options for bfloat16: 8192-element tiles, 10-bit tables; low byte raw, high byte coded)."""
@@ -646,7 +709,7 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans"])
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm"])
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
@@ -668,6 +731,8 @@ def main():
         return stack_workload(args, ep)
     if args.workload == "tile_ans":
         return lossless_workload(args, ep)
+    if args.workload == "gemm":
+        return gemm_workload(args, ep)
     rows, cols, sigma, seed, bpp, outliers = WORKLOADS[args.workload]
     started = time.perf_counter()
     weight = make_weight(rows, cols, sigma, seed, outliers)

@@ -37,6 +37,21 @@ class DecodePlan:
         return _hip.TABLE_KIND_NAMES[self.desc.table_kind]
 
 
+_ERROR_WORDS_PER_POOL = 1024
+_error_pools: dict = {}        # device -> [int32 tensor of zeros, words handed out]
+
+
+def _error_word(device: torch.device) -> torch.Tensor:
+    """A zeroed int32[1] for one plan's decode errors, cut from a pool per device: one fill kernel per 1024 plans instead
+    of one per plan (a model's containers are planned in a burst when it is first decoded)."""
+    pool = _error_pools.get(device)
+    if pool is None or pool[1] == _ERROR_WORDS_PER_POOL:
+        pool = _error_pools[device] = [torch.zeros(_ERROR_WORDS_PER_POOL, dtype=torch.int32, device=device), 0]
+    word = pool[0][pool[1]:pool[1] + 1]
+    pool[1] += 1
+    return word
+
+
 def _plan_for(buffers: LatticeBuffers, info: dict) -> DecodePlan:
     layout, meta, freq = buffers.layout, buffers.stream_meta, buffers.freq_tables
     device = meta.device
@@ -60,7 +75,7 @@ def _plan_for(buffers: LatticeBuffers, info: dict) -> DecodePlan:
         raise ValueError("lattice_rans stream_meta / freq_tables are inconsistent (ranges, sums or coset stream)")
     _hip.check("ep_hip_plan_describe", status)
     tables = torch.empty(desc.table_bytes, dtype=torch.uint8, device=device)
-    error = torch.zeros(1, dtype=torch.int32, device=device)
+    error = _error_word(device)
     _hip.check("ep_hip_plan_build", lib.ep_hip_plan_build(
         meta.data_ptr(), _hip.pointer(freq), ctypes.byref(desc), tables.data_ptr(), _hip.current_stream(device)))
     plan = DecodePlan(desc=desc, tables=tables, error=error, key=key)
