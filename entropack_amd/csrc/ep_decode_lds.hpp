@@ -730,12 +730,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       float dot[DOT_ROWS > 0 ? DOT_ROWS : 1];
 #pragma unroll
       for (int m = 0; m < DOT_ROWS; ++m) {
+        // Two bf16 products and the running sum per instruction (v_dot2_f32_bf16): the operands are used as they lie,
+        // packed in pairs, instead of being widened to float32 one by one.
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
         const uint32_t xw[4] = {in.x[m].x, in.x[m].y, in.x[m].z, in.x[m].w};
         float sum = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          sum = __fmaf_rn(__uint_as_float(packed[i] << 16), __uint_as_float(xw[i] << 16), sum);
-          sum = __fmaf_rn(__uint_as_float(packed[i] & 0xFFFF0000u), __uint_as_float(xw[i] & 0xFFFF0000u), sum);
+          sum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed[i]), __builtin_bit_cast(bf16x2, xw[i]), sum, false);
         }
         dot[m] = valid_lane ? sum : 0.0f;
       }

@@ -2,9 +2,10 @@
 
   rows M            weight written to memory?   kernels
   1 (and 2..4 on    no                          the decode kernel multiplies every decoded vector with the activations in
-  weights whose                                 registers (`ep_hip_linear_fused_bf16`): the memory-bound regime, where the
-  decode is chain-                              dense weight would be 16 / bpp times the bytes of the container
-  bound anyway)
+  weights large                                 registers (`ep_hip_linear_fused_bf16`, two bf16 products per instruction):
+  enough that their                             the memory-bound regime, where the dense weight would be 16 / bpp times the
+  decode is bound by                            bytes of the container
+  throughput)
   up to 128         yes, once                   decode, then this package's split-K skinny product (`ep_hip_gemm_bf16_skinny`),
                                                 which streams the weight at 75 % of the memory bandwidth
   more              yes, once                   decode, then a tiled product on the matrix cores: the vendor library's

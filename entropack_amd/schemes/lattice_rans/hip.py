@@ -200,8 +200,12 @@ def fused_linear_usable(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool
 def fused_linear_pays(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
     """Usable, and measured faster than decoding and multiplying separately.
 
-    One row always pays. With rank/select tables the four-row kernel needs more registers than two resident blocks
-    per CU allow and loses to decode + the split-K product.
+    One row always pays (8192 x 28672 @ 4 bpp: 175 us against 233 us; on a 3072 x 3072 weight the two are level and
+    this one never writes the weight). Two to four rows pay on weights whose decode is bound by throughput (more tile
+    pairs than 16 waves on every CU hold): the extra products ride along in issue slots the decode leaves free
+    (8192 x 28672: 217 us against 224 us at 4 bpp, 275 against 290 at 8 bpp). On a smaller weight the launch lasts as
+    long as one tile's chain of dependent steps, the products lengthen every link of it, and decoding first is faster
+    (3072 x 3072, four rows: 103 us against 84 us).
     """
     if not fused_linear_usable(buffers, shape, x):
         return False
@@ -213,15 +217,10 @@ def fused_linear_pays(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
     rows = x.numel() // x.shape[-1]
     if rows == 1:
         return True
-    if plan.desc.table_kind == _hip.TABLE_LDS_RANK:
-        return False
-    # Two to four rows: the four-row kernel costs a third more than a plain decode. A weight small enough that its
-    # decode lasts as long as one tile's chain anyway (at most 16 tile pairs per CU) hides that; a large one is decoded
-    # at full rate and multiplied by the split-K product faster (8192 x 28672 @ 4 bpp: 239 us against 270 us).
     device = buffers.payload.device
     caps = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device())
     pairs = (int(buffers.states.shape[0]) + 1) // 2
-    return pairs <= 16 * caps.compute_units
+    return pairs > 16 * caps.compute_units
 
 
 def linear_rows(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
