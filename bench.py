@@ -633,6 +633,16 @@ def gemm_workload(args, ep):
     return 0
 
 
+def copy_probe(args, device):
+    """One plain device copy of `--copy-probe-mib` MiB: the calibration of the FETCH_SIZE / WRITE_SIZE counters."""
+    if args.copy_probe_mib:
+        probe = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=device)
+        probe.zero_()
+        torch.empty_like(probe).copy_(probe)          # reads and writes exactly copy_probe_mib MiB
+        torch.cuda.synchronize()
+        del probe
+
+
 def lossless_workload(args, ep):
     """The lossless neighbour of the target: tile_ans decode of 8192 x 28672 bf16 N(0, 0.015) seed 4 (the reference's
     default options for bfloat16: 8192-element tiles, 10-bit tables; low byte raw, high byte coded)."""
@@ -653,6 +663,7 @@ def lossless_workload(args, ep):
     def step():
         return tile_lane.decode(buffers, dtype=torch.bfloat16)
 
+    copy_probe(args, device)
     for _ in range(max(args.warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
@@ -752,12 +763,7 @@ def main():
     def step():
         return hip_lane.decode(lattice, shape=(rows, cols), dtype=torch.bfloat16)
 
-    if args.copy_probe_mib:
-        probe = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=device)
-        probe.zero_()
-        torch.empty_like(probe).copy_(probe)          # reads and writes exactly copy_probe_mib MiB
-        torch.cuda.synchronize()
-        del probe
+    copy_probe(args, device)
 
     for _ in range(max(args.warmup, 1)):
         dense = step()
