@@ -130,7 +130,24 @@ def python_loop_baseline(host, rows, cols_padded, alg_bytes, tiles_sampled=8):
 MFMA_PEAK_BF16_TFLOPS = 2500.0
 
 
+#: Seconds of untimed launches in front of every timed region. From idle the card's clock governor needs about 30 ms of
+#: load before launch times settle (8192x28672 @ 4 bpp decode: launches 5..25 after idle take 142-165 us, from the 200th
+#: on 130 us, steady for as long as the load lasts); measurements taken inside that ramp describe the governor.
+SETTLE_SECONDS = 0.2
+
+
+def settle(fn, seconds=None):
+    """Keeps the device busy with `fn` for `seconds` (queue kept full, one synchronisation per 32 calls)."""
+    seconds = SETTLE_SECONDS if seconds is None else seconds
+    started = time.perf_counter()
+    while time.perf_counter() - started < seconds:
+        for _ in range(32):
+            fn()
+        torch.cuda.synchronize()
+
+
 def _median_ms(fn, steps, warmup=5):
+    settle(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -418,19 +435,19 @@ def stack_workload(args, ep):
         kinds[kind] = kinds.get(kind, 0) + 1
 
     def timed(fn, steps, warmup):
+        settle(fn)
         for _ in range(max(warmup, 1)):
             out = fn()
         torch.cuda.synchronize()
-        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         wall = time.perf_counter()
-        for begin, end in events:
-            begin.record()
+        first.record()
+        for _ in range(steps):
             out = fn()
-            end.record()
+        last.record()
         torch.cuda.synchronize()
         wall = (time.perf_counter() - wall) / steps
-        device_ms = sorted(begin.elapsed_time(end) for begin, end in events)
-        return out, wall, sum(device_ms) / len(device_ms)
+        return out, wall, first.elapsed_time(last) / steps
 
     steps = min(args.steps, 20)
     dense, wall, device_ms = timed(lambda: batch(arena), steps, args.warmup)
@@ -492,18 +509,19 @@ def decode_case(ep, name, steps, warmup, check):
     def step():
         return hip_lane.decode(lattice, shape=(rows, cols), dtype=torch.bfloat16)
 
+    dense = step()
+    settle(step)
     for _ in range(max(warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
     hip_lane.check_errors(lattice)
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for begin, end in events:
-        begin.record()
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    first.record()
+    for _ in range(steps):
         dense = step()
-        end.record()
+    last.record()
     torch.cuda.synchronize()
-    kernel_ms = sorted(begin.elapsed_time(end) for begin, end in events)
-    avg_ms = sum(kernel_ms) / len(kernel_ms)
+    avg_ms = first.elapsed_time(last) / steps
     entry = {
         "workload": f"{rows}x{cols} N(0,{sigma}) seed {seed}{' +0.1% x20 outliers' if outliers else ''} @ {bpp} bpp -> bf16",
         "tiles": int(lattice.states.shape[0]), "prob_bits": int(container.buffers["layout"][1]),
@@ -575,26 +593,20 @@ def gemm_workload(args, ep):
     (N = K = 3072) at 256, 1024 and 4096 activation rows, once with one weight used over and over (operands resident in
     the caches) and once rotating through enough different weights that each one comes from memory, as a weight fresh from
     the decoder does; then the same product at M = 4096 against K, which separates the per-launch cost from the cost of
-    a K step. Device times from events around each launch with the queue kept busy by a spin kernel in front."""
+    a K step. Device times: 200 launches back to back between one pair of events, after the clocks have settled."""
     from torch.nn import functional as F
     from entropack_amd.linear import kernels
     torch.manual_seed(0)
 
-    def timed(fn, count=30):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
-        times = []
+    def timed(fn, count=200):
+        settle(fn)
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record()
         for _ in range(count):
-            torch.cuda._sleep(200000)                  # the launch below is queued behind this: no host latency in the events
-            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            begin.record()
             fn()
-            end.record()
-            torch.cuda.synchronize()
-            times.append(begin.elapsed_time(end) * 1e3)
-        times.sort()
-        return round(times[len(times) // 2], 2)
+        last.record()
+        torch.cuda.synchronize()
+        return round(first.elapsed_time(last) / count * 1e3, 2)
 
     n = k = 3072
     weights = [(torch.randn(n, k, device="cuda") * 0.02).to(torch.bfloat16) for _ in range(24)]      # 453 MB: more than the 256 MB last-level cache
@@ -622,7 +634,7 @@ def gemm_workload(args, ep):
     own = rows_out["M=4096"]["own"]["rotating_weights_us"]
     result = {
         "metric": "bf16 GEMM TFLOP/s, 4096 x 3072 x 3072, weight from memory", "value": round(flops / own / 1e6, 2), "unit": "TFLOP/s", "n_gpus": 1,
-        "steps": 30, "warmup": 3, "ms_per_step": round(own / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "steps": 200, "warmup": 0, "ms_per_step": round(own / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "y = x W^T, N = K = 3072, bf16, f32 accumulation; own kernel (ep_hip_gemm_bf16) beside the vendor library's",
                    "by_rows": rows_out, "by_inner_size_at_M_4096": sweep},
@@ -664,20 +676,28 @@ def lossless_workload(args, ep):
         return tile_lane.decode(buffers, dtype=torch.bfloat16)
 
     copy_probe(args, device)
+    dense = step()
+    settle(step)
     for _ in range(max(args.warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
     tile_lane.check_errors(buffers)
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     wall = time.perf_counter()
+    first.record()
+    for _ in range(args.steps):
+        dense = step()
+    last.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall) / args.steps
+    kernel_avg_ms = first.elapsed_time(last) / args.steps
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     for begin, end in events:
         begin.record()
         dense = step()
         end.record()
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - wall) / args.steps
     kernel_ms = sorted(begin.elapsed_time(end) for begin, end in events)
-    kernel_avg_ms = sum(kernel_ms) / len(kernel_ms)
     tile_elements, prob_bits, lanes, elements = (int(v) for v in container.buffers["layout"].tolist())
     result = {
         "metric": "lossless decode GB/s (+% HBM roofline)", "value": round(alg_bytes / wall / 1e9, 3), "unit": "GB/s", "n_gpus": 1,
@@ -765,23 +785,49 @@ def main():
 
     copy_probe(args, device)
 
+    # From idle first (the device has done nothing while the host encoded): `warmup` + `steps` launches as they come.
+    dense = step()                                    # builds the plan
+    torch.cuda.synchronize()
+    hip_lane.check_errors(lattice)
+    time.sleep(0.2)
+    for _ in range(max(args.warmup, 1)):
+        dense = step()
+    idle_first, idle_last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    idle_first.record()
+    for _ in range(args.steps):
+        dense = step()
+    idle_last.record()
+    torch.cuda.synchronize()
+    from_idle_ms = idle_first.elapsed_time(idle_last) / args.steps
+    # Then with the clocks settled: SETTLE_SECONDS of the same launches, the warm-up steps, the timed steps.
+    settle(step)
     for _ in range(max(args.warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
     hip_lane.check_errors(lattice)
 
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    # The timed region: exactly `steps` launches back to back between two synchronisations, with one pair of HIP events
+    # on the launch stream around all of them (average launch duration = their distance / steps; events between the
+    # launches would put a marker packet, and a few microseconds, between every two kernels).
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     wall = time.perf_counter()
+    first.record()
+    for _ in range(args.steps):
+        dense = step()
+    last.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall
+    kernel_avg_ms = first.elapsed_time(last) / args.steps
+    ms_per_step = wall * 1e3 / args.steps
+    # Outside the timed region: the same launches bracketed one by one, for the spread.
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     for begin, end in events:
         begin.record()
         dense = step()
         end.record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - wall
     kernel_ms = sorted(begin.elapsed_time(end) for begin, end in events)
-    kernel_avg_ms = sum(kernel_ms) / len(kernel_ms)
-    ms_per_step = wall * 1e3 / args.steps
 
     result = {
         "metric": "lossy decode GB/s (+% HBM roofline); CompressedLinear TFLOPS @ M=4096, 4 bpp",
@@ -803,6 +849,11 @@ def main():
             "unit": "GB/s", "frac": round(alg_bytes / (kernel_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
             "traffic": measured_traffic(args.workload, args.table_kind)[0], "traffic_source": measured_traffic(args.workload, args.table_kind)[1],
             "kernel_ms_avg": round(kernel_avg_ms, 5), "kernel_ms_median": round(kernel_ms[len(kernel_ms) // 2], 5),
+            "kernel_ms_min": round(kernel_ms[0], 5),
+            "kernel_ms_avg_from_idle": round(from_idle_ms, 5),
+            "frac_from_idle": round(alg_bytes / (from_idle_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
+            "clocks": f"settled: {SETTLE_SECONDS} s of untimed launches of the same kernel before the warm-up steps; "
+                      f"from idle = the first {args.warmup} + {args.steps} launches after 0.2 s without work",
         },
     }
 
