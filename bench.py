@@ -27,8 +27,8 @@ HBM_PEAK_GBPS = 8000.0
 #: named profile was taken. `csrc_sha16` names those sources; when the kernels have changed since, the figure is not
 #: reported (`traffic` is null and `traffic_source` says why) instead of going stale silently.
 MEASURED_TRAFFIC = {
-    "target": {"bytes": 600_700_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "unset"},
-    "tile_ans": {"bytes": 818_700_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "unset"},
+    "target": {"bytes": 600_600_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "de8d4dbbfb1a2f18"},
+    "tile_ans": {"bytes": 818_700_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "2f34e254db80ae6b"},
 }
 #: The kernel sources a traffic figure depends on, per workload.
 TRAFFIC_SOURCES = {
@@ -146,8 +146,15 @@ def settle(fn, seconds=None):
         torch.cuda.synchronize()
 
 
-def _median_ms(fn, steps, warmup=5):
-    settle(fn)
+def _median_ms(fn, steps, warmup=5, from_idle=False):
+    """Median duration of `fn` over `steps` calls bracketed one by one, with the clocks settled; `from_idle`: after half a
+    second without work instead (the first few tens of milliseconds of load run at other clocks: a decode slower, a
+    matrix-core product faster, than they do in a loop that lasts)."""
+    if from_idle:
+        torch.cuda.synchronize()
+        time.sleep(0.5)
+    else:
+        settle(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -310,21 +317,28 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
             out = layer(x)
         return out
 
-    def priced(ms_stack):
+    def priced(ms_stack, ms_stack_from_idle=None):
         per_layer = ms_stack / layers_total
-        return {"ms_per_layer": round(per_layer, 5), "tflops": round(flops / per_layer / 1e9, 2),
-                "frac_of_mfma_peak": round(flops / per_layer / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5)}
+        entry = {"ms_per_layer": round(per_layer, 5), "tflops": round(flops / per_layer / 1e9, 2),
+                 "frac_of_mfma_peak": round(flops / per_layer / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5)}
+        if ms_stack_from_idle is not None:
+            entry["ms_per_layer_from_idle"] = round(ms_stack_from_idle / layers_total, 5)
+        return entry
+
+    def both(fn):
+        count = max(3, steps // 5)
+        return priced(_median_ms(fn, count, warmup=2), _median_ms(fn, count, warmup=2, from_idle=True))
 
     out = {"workload": f"{layers_total} x CompressedLinear 3072x3072 @ 4.0 bpp + bias, X [4096, 3072] bf16, decode_then_gemm"}
     reference = forward()
-    out["layer_by_layer"] = priced(_median_ms(forward, max(3, steps // 5), warmup=2))
+    out["clocks"] = (f"ms_per_layer: after {SETTLE_SECONDS} s of the same forward passes (the card then runs at its 1400 W limit); "
+                     "ms_per_layer_from_idle: the first passes after half a second without work")
+    out["layer_by_layer"] = both(forward)
     weights = [layer.dequantize("cuda") for layer in layers[:distinct]]
-    out["dense_gemm_only"] = priced(_median_ms(lambda: [torch.nn.functional.linear(x, weights[i % distinct], layers[i].bias)
-                                                        for i in range(layers_total)], max(3, steps // 5), warmup=2))
+    out["dense_gemm_only"] = both(lambda: [torch.nn.functional.linear(x, weights[i % distinct], layers[i].bias) for i in range(layers_total)])
     from entropack_amd.linear import fused as fused_mode
     from entropack_amd.linear import kernels
-    out["dense_own_gemm_only"] = priced(_median_ms(lambda: [kernels.gemm_bf16(x, weights[i % distinct], layers[i].bias)
-                                                            for i in range(layers_total)], max(3, steps // 5), warmup=2))
+    out["dense_own_gemm_only"] = both(lambda: [kernels.gemm_bf16(x, weights[i % distinct], layers[i].bias) for i in range(layers_total)])
     del weights
     # `beside`: groups decode on a second stream while the previous group multiplies (two arenas); `in_line`: on the
     # layers' own stream between two groups (one arena).
@@ -333,7 +347,7 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
             continue
         with ep.DecodeAhead(layers, group_size=group, overlap=overlap) as ahead:
             same = bool(torch.equal(forward(), reference))
-            entry = priced(_median_ms(forward, max(3, steps // 5), warmup=2))
+            entry = both(forward)
             entry["identical_to_layer_by_layer"] = same
             entry["dense_bytes_held"] = ahead.arena_bytes
             ahead.check_errors()
@@ -347,7 +361,7 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
         rel = ((own_reference.double() - reference.double()).norm() / reference.double().norm()).item()
         with ep.DecodeAhead(layers, group_size=16, overlap=False) as ahead:
             same = bool(torch.equal(forward(), own_reference))
-            entry = priced(_median_ms(forward, max(3, steps // 5), warmup=2))
+            entry = both(forward)
             entry["identical_to_layer_by_layer"] = same
             entry["rel_l2_vs_library_product"] = rel
             ahead.check_errors()
