@@ -65,8 +65,9 @@ inline size_t rank_table_bytes(int present, int prob_bits) {
 // (the first 2^pb slots of each are used). An FB entry is
 //   word 0: freq | 0x3C000000 when the value is odd  (the multiply takes the low 24 bits; the high halves of seven such
 //           words XOR to the parity of z0..z6 as a half-precision 0.0 or 1.0)
-//   word 1: (cdf + 2048 * coset) | half(value) << 16  (the decode step forms slot | 2048 * coset, both as the slot
-//           table's address and as the number the low half is subtracted from; the high half is the value itself, which a
+//   word 1: (cdf + 2048 * coset) | half(coordinate) << 16  (the decode step forms slot | 2048 * coset, both as the slot
+//           table's address and as the number the low half is subtracted from; the high half is the lattice coordinate
+//           value + coset / 2 (for the last field, whose coordinate is 2 m + parity + coset / 2: m + coset / 4), which a
 //           mixed-precision multiply-add takes without a conversion).
 // A field's two cosets lie 2048 bytes apart in both parts, so one per-lane offset serves both lookups.
 constexpr int kSymFbStreamBytes = 256 * 8;

@@ -378,11 +378,11 @@ __device__ __forceinline__ void sym_step(Pair& p, int field, const StepConsts& k
   p.pos = pos;
 }
 
-// fma(half in the high 16 bits of `packed`, b, c) in float32 with one rounding: v_fma_mix_f32 reads the half-precision
+// (half in the high 16 bits of `packed`) * b in float32 with one rounding: v_fma_mix_f32 reads the half-precision
 // operand where it lies, so a value the table holds in that form costs no conversion.
-__device__ __forceinline__ float fma_high_half(uint32_t packed, float b, float c) {
+__device__ __forceinline__ float mul_high_half(uint32_t packed, float b) {
   float r;
-  asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(b), "v"(c));
+  asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(b));
   return r;
 }
 // fma(half in the high 16 bits of `packed`, 2, half in the high 16 bits of `addend`)
@@ -601,8 +601,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
     // (zero, negative: the sign of a zero weight; subnormal; beyond 1e30: bf16 saturation) takes the literal form.
     auto lattice_point = [&](const Pair& s, float (&z)[8]) {
       if constexpr (MODE == kModeSym) {
-        // The entries hold the values in half precision (second word, high half); the first words' high halves XOR to
-        // the parity of z0..z6 as a half-precision 0.0 or 1.0.
+        // The entries hold the coordinates, coset shift included, in half precision (second word, high half); the first
+        // words' high halves XOR to the parity of z0..z6 as a half-precision 0.0 or 1.0.
         const uint32_t folded = xor3(xor3(s.e[0], s.e[1], s.e[2]), xor3(s.e[3], s.e[4], s.e[5]), s.e[6]);
 #pragma unroll
         for (int f = 0; f < 7; ++f) z[f] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(s.ey[f] >> 16)));
@@ -629,13 +629,14 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         for (int f = 0; f < 8; ++f) z[f] = static_cast<float>(v[f]);
       }
     };
-    // w = fma(z, scale, shift) for an ordinary scale; with two-level tables straight from the half-precision values.
+    // w = fma(z, scale, shift) for an ordinary scale. The two-level tables hold z + c / 2 itself in half precision, so
+    // there the weight is one product, literally the reference's (z + c / 2) * scale, and `shift` is not used.
     auto scaled_point = [&](const Pair& s, float scale, float shift, float (&w)[8]) {
       if constexpr (MODE == kModeSym) {
         const uint32_t folded = xor3(xor3(s.e[0], s.e[1], s.e[2]), xor3(s.e[3], s.e[4], s.e[5]), s.e[6]);
 #pragma unroll
-        for (int f = 0; f < 7; ++f) w[f] = fma_high_half(s.ey[f], scale, shift);
-        w[7] = __fmaf_rn(twice_high_half_plus(s.ey[7], folded), scale, shift);
+        for (int f = 0; f < 7; ++f) w[f] = mul_high_half(s.ey[f], scale);
+        w[7] = __fmul_rn(twice_high_half_plus(s.ey[7], folded), scale);
       } else {
         float z[8];
         lattice_point(s, z);
@@ -652,7 +653,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       } else {
         float z[8];
         lattice_point(s, z);
-        const float shift = c ? 0.5f : 0.0f;
+        const float shift = MODE != kModeSym && c ? 0.5f : 0.0f;       // the two-level tables' values include it
 #pragma unroll
         for (int f = 0; f < 8; ++f) w[f] = __fmul_rn(__fadd_rn(z[f], shift), scale);
       }

@@ -75,8 +75,12 @@ __global__ __launch_bounds__(256) void build_sym_tables_kernel(const int32_t* __
   uint2* fb = reinterpret_cast<uint2*>(section) + (stream - 1) * 256;
   uint8_t* slots = section + slot_table_at;
   if (tid < alphabet && f != 0) {
-    const int z = tid + sym_min;                                 // in [-128, 127]: exact in half precision
-    const uint32_t z_half = __builtin_bit_cast(uint16_t, static_cast<_Float16>(z));
+    // The half-precision value is the lattice coordinate itself, coset shift included: z + c / 2, and for the last field,
+    // whose z7 = 2 m + parity the kernel forms with one multiply-add, m + c / 4. |z| <= 128, so quarters are exact.
+    const int z = tid + sym_min;
+    const int coset = (stream - 1) & 1, field = (stream - 1) >> 1;
+    const float coordinate = static_cast<float>(z) + (field == kFields - 1 ? 0.25f : 0.5f) * static_cast<float>(coset);
+    const uint32_t z_half = __builtin_bit_cast(uint16_t, static_cast<_Float16>(coordinate));
     fb[z + 128] = make_uint2(f | ((z & 1) ? 0x3C000000u : 0u), (begin + folded) | (z_half << 16));
   }
   __syncthreads();
