@@ -481,6 +481,12 @@ __device__ __forceinline__ int window_pointer_b(const Pair& s) {
 
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
+// A wave alternates between a chain of dependent symbol steps, where every instruction waits for the one before, and a
+// burst of independent work (reconstruction, products, the store). The chain runs at the higher wave priority: the
+// bursts of a SIMD's other waves then fill the issue slots that its chains leave open instead of delaying them.
+__device__ __forceinline__ void chain_priority() { __builtin_amdgcn_s_setprio(1); }
+__device__ __forceinline__ void emit_priority() { __builtin_amdgcn_s_setprio(0); }
+
 template <int PB, int MODE, int ILP, int KIND>
 __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_begin, int pair_end, int pair_stride) {
   extern __shared__ __align__(16) uint8_t smem[];
@@ -826,7 +832,9 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         scale[j] = valid_lane ? a.scales[row] : 0.0f;
         if constexpr (DOT_ROWS > 0) dot_prefetch(vector[j], row, valid_lane, dot_in[j]);
       }
+      chain_priority();
       group_steps(masked_tag, valid_lane, valid);
+      emit_priority();
       if constexpr (DOT_ROWS > 0) {
 #pragma unroll
         for (int j = 0; j < ILP; ++j) dot_emit(st[j], scale[j], valid_lane, dot_in[j]);
@@ -858,7 +866,9 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
           cursor[j].unusual = __builtin_amdgcn_ballot_w64(!(__float_as_uint(scale) - 0x0DA24260u <= 0x7149F2CAu - 0x0DA24260u));
         }
       }
+      chain_priority();
       group_steps(Unmasked{}, true, all_lanes);
+      emit_priority();
 #pragma unroll
       for (int j = 0; j < ILP; ++j) {
         const RowCursor& c = cursor[j];
@@ -893,6 +903,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       const float scale = valid_lane ? a.scales[row] : 0.0f;
       DotInput dot_in;
       if constexpr (DOT_ROWS > 0) dot_prefetch(vector, row, valid_lane, dot_in);
+      chain_priority();
       coset_step_single<PB, MODE, true>(s, k, valid);
       const uint32_t high = s.coset_base + L::kHighBase;
 #pragma unroll
@@ -906,6 +917,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         }
         if ((f & 1) == 0 || f == kFields - 1) top_up(s);
       }
+      emit_priority();
       if constexpr (DOT_ROWS > 0) dot_emit(s, scale, valid_lane, dot_in);
       else if (valid_lane) emit(s, vector, scale);
     };

@@ -334,6 +334,7 @@ __global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) voi
 #pragma unroll
           for (int r = 0; r < RAW; ++r) __builtin_memcpy(&raw[j][r], payload8 + (raw_at[j][r] + static_cast<uint32_t>(at) + mine), 8);
         }
+        __builtin_amdgcn_s_setprio(1);      // the dependent steps go before other waves' independent work (below)
 #pragma unroll
         for (int g = kTileChunk / 32 - 1; g >= 0; --g) {
           auto leave = [&](int k, uint32_t symbol) {
@@ -356,6 +357,7 @@ __global__ __launch_bounds__(1024, tile_kernel_waves_per_simd(BYTES, CODED)) voi
             if ((g & 1) == 0) slide_window(st[k]);
           }
         }
+        __builtin_amdgcn_s_setprio(0);
         if constexpr (CODED > 0) {
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
