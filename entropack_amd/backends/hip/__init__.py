@@ -13,7 +13,7 @@ import torch
 
 _PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 LIBRARY_PATH = os.path.join(_PACKAGE_DIR, "libentropack_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 OK, EINVAL, EUNSUPPORTED, ERUNTIME, ENODEVICE, ETOOLARGE = range(6)
 STATIC_ACCUMULATOR_FLOATS = 1 << 18          # EP_HIP_STATIC_ACCUMULATOR_FLOATS
@@ -45,7 +45,7 @@ class PlanDesc(ctypes.Structure):
     _fields_ = [
         ("table_kind", ctypes.c_int), ("prob_bits", ctypes.c_int), ("table_bytes", ctypes.c_size_t),
         ("lds_bytes", ctypes.c_int), ("max_alphabet", ctypes.c_int), ("alphabet_sum", ctypes.c_int),
-        ("sym_offset", ctypes.c_int), ("present_offset", ctypes.c_int * 18),
+        ("sym_offset", ctypes.c_int), ("present_offset", ctypes.c_int * 18), ("rank_values_half", ctypes.c_int),
     ]
 
 

@@ -146,7 +146,7 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
   args.tile_vectors = tv;
   args.num_tiles = static_cast<int>(tiles);
   args.error = error_dev;
-  args.lut_bytes = args.rank_val_offset = args.rank_rs_offset = 0;
+  args.lut_bytes = args.rank_val_offset = args.rank_rs_offset = args.rank_half = 0;
   args.sym_tables = nullptr;
   args.m_rows = 0;
   args.x = nullptr;
@@ -178,6 +178,8 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
       args.lut_bytes = static_cast<uint32_t>(desc->lds_bytes);
       args.rank_val_offset = static_cast<uint32_t>(rank_fb_bytes(present));
       args.rank_rs_offset = static_cast<uint32_t>(rank_rs_offset(present, desc->prob_bits));
+      if (desc->rank_values_half != 0 && desc->prob_bits > 14) return EP_HIP_EINVAL;
+      args.rank_half = desc->rank_values_half != 0;
       return EP_HIP_OK;
     }
     case EP_TABLE_LDS_SYM:

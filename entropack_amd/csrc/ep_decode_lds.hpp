@@ -302,15 +302,16 @@ __device__ __forceinline__ void coset_step_dual(Pair& p0, Pair& p1, const StepCo
 // 32 slots the table keeps {bits, count}: bit b is set when slot 32 w + b is the last slot of its symbol, count is the
 // number of symbols (of all field streams before this one, plus this stream's) that end before slot 32 w. The symbol
 // of a slot is then count + popcount(bits below the slot): one 8-byte read, and a second read fetches that symbol's
-// freq | cdf << 16; its value (symbol + minimum, int16) is read off the critical path. The lookups are ordinary C++;
-// renormalisation is the same scalar vote as above.
+// cdf | freq << 16 (the subtraction takes the low half where it lies; with half-precision values bit 31 marks an odd
+// value and the frequency is the 15 bits below it, `freq_width`); its 16-bit value is read off the critical path. The
+// lookups are ordinary C++; renormalisation is the same scalar vote as above.
 template <int PB, bool MASKED>
-__device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_group, uint32_t val0, const StepConsts& k,
-                                          bool valid_lane) {
+__device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_group, uint32_t val0, uint32_t freq_width,
+                                          const StepConsts& k, bool valid_lane) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   typedef __attribute__((address_space(3))) const u32x2* lds_u2;
   typedef __attribute__((address_space(3))) const uint32_t* lds_u32;
-  typedef __attribute__((address_space(3))) const int16_t* lds_i16;
+  typedef __attribute__((address_space(3))) const uint16_t* lds_u16;
   constexpr uint32_t kTable = 1u << PB;
   const uint32_t x = p.x;
   const uint32_t slot = x & (kTable - 1u);
@@ -322,8 +323,9 @@ __device__ __forceinline__ void rank_step(Pair& p, int field, uint32_t rs_group,
   // The bit-field extract takes its width from the low five bits of x: the bits of rs.x below slot % 32.
   const uint32_t index = static_cast<uint32_t>(__builtin_popcount(__builtin_amdgcn_ubfe(rs.x, 0u, x))) + rs.y;
   const uint32_t fb = *reinterpret_cast<lds_u32>(static_cast<uintptr_t>(index << 2));
-  p.e[field] = static_cast<uint32_t>(static_cast<int32_t>(*reinterpret_cast<lds_i16>(static_cast<uintptr_t>((index << 1) + val0))));
-  const uint32_t next = __umul24(fb & 0xFFFFu, x >> PB) + slot - (fb >> 16);
+  p.e[field] = *reinterpret_cast<lds_u16>(static_cast<uintptr_t>((index << 1) + val0));      // 16 bits, not extended
+  p.ey[field] = fb;
+  const uint32_t next = __umul24(__builtin_amdgcn_ubfe(fb, 16u, freq_width), x >> PB) + (slot - (fb & 0xFFFFu));
   p.x = (!MASKED || valid_lane) ? next : x;
   uint32_t t, d, na, nb;
   uint32_t pos = uniform(p.pos);
@@ -383,6 +385,18 @@ __device__ __forceinline__ void sym_step(Pair& p, int field, const StepConsts& k
 __device__ __forceinline__ float mul_high_half(uint32_t packed, float b) {
   float r;
   asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(b));
+  return r;
+}
+// The same for a half in the low 16 bits.
+__device__ __forceinline__ float mul_low_half(uint32_t packed, float b) {
+  float r;
+  asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(b));
+  return r;
+}
+// fma(half in the low 16 bits of `packed`, 2, addend)
+__device__ __forceinline__ float twice_low_half_plus(uint32_t packed, float addend) {
+  float r;
+  asm("v_fma_mix_f32 %0, %1, 2.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(addend));
   return r;
 }
 // fma(half in the high 16 bits of `packed`, 2, half in the high 16 bits of `addend`)
@@ -551,6 +565,9 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
   // Byte distance between a field's two cosets, in the table the coset offset is added to.
   k.ktab = MODE == kModeRank ? (L::kTable / 32u) * 8u : (MODE == kModeSym ? static_cast<uint32_t>(kSymFbStreamBytes) : L::kTableBytes);
   const uint32_t rank_val0 = uniform(a.rank_val_offset), rank_rs0 = uniform(a.rank_rs_offset);
+  // Rank/select tables with half-precision values (the usual case): reconstruction as for the two-level tables.
+  const bool rank_half = MODE == kModeRank && uniform(a.rank_half) != 0;
+  const uint32_t rank_freq_width = rank_half ? 15u : 16u;
   k.shv = half ? 16u : 0u;
   // Keep the per-lane constants in vector registers (the steps name them as VGPR operands).
   asm volatile("" : "+v"(k.f0v), "+v"(k.f1v), "+v"(k.ktab), "+v"(k.shv));
@@ -620,13 +637,19 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
 #pragma unroll
         for (int f = 0; f < 8; ++f) z[f] = static_cast<float>(static_cast<int32_t>(s.e[f]) >> 24);
         z[7] = __fmaf_rn(z[7], 2.0f, parity);
+      } else if (MODE == kModeRank && rank_half) {
+        // The values are the coordinates, coset shift included, in half precision; bit 31 of an entry marks an odd value.
+        const uint32_t folded = xor3(xor3(s.ey[0], s.ey[1], s.ey[2]), xor3(s.ey[3], s.ey[4], s.ey[5]), s.ey[6]);
+#pragma unroll
+        for (int f = 0; f < 7; ++f) z[f] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(s.e[f])));
+        z[7] = twice_low_half_plus(s.e[7], static_cast<float>(folded >> 31));
       } else {
         const bool c = s.coset_base != 0;
         const int32_t* minima = reinterpret_cast<const int32_t*>(smem + (minima0 - lds0)) + 1 + (c ? 1 : 0);
         int v[8];
 #pragma unroll
         for (int f = 0; f < 8; ++f) {
-          if constexpr (MODE == kModeRank) v[f] = static_cast<int>(s.e[f]);
+          if constexpr (MODE == kModeRank) v[f] = static_cast<int16_t>(s.e[f]);
           else v[f] = static_cast<int>(s.e[f] >> L::kSymShift) + minima[2 * f];
         }
         const int parity = (v[0] + v[1] + v[2] + v[3] + v[4] + v[5] + v[6]) & 1;
@@ -643,6 +666,11 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
 #pragma unroll
         for (int f = 0; f < 7; ++f) w[f] = mul_high_half(s.ey[f], scale);
         w[7] = __fmul_rn(twice_high_half_plus(s.ey[7], folded), scale);
+      } else if (MODE == kModeRank && rank_half) {
+        const uint32_t folded = xor3(xor3(s.ey[0], s.ey[1], s.ey[2]), xor3(s.ey[3], s.ey[4], s.ey[5]), s.ey[6]);
+#pragma unroll
+        for (int f = 0; f < 7; ++f) w[f] = mul_low_half(s.e[f], scale);
+        w[7] = __fmul_rn(twice_low_half_plus(s.e[7], static_cast<float>(folded >> 31)), scale);
       } else {
         float z[8];
         lattice_point(s, z);
@@ -659,7 +687,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
       } else {
         float z[8];
         lattice_point(s, z);
-        const float shift = MODE != kModeSym && c ? 0.5f : 0.0f;       // the two-level tables' values include it
+        const float shift = MODE != kModeSym && !rank_half && c ? 0.5f : 0.0f;       // half-precision table values include it
 #pragma unroll
         for (int f = 0; f < 8; ++f) w[f] = __fmul_rn(__fadd_rn(z[f], shift), scale);
       }
@@ -793,7 +821,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
-          rank_step<PB, MASKED>(st[0], f, rank_group, rank_val0, k, valid_lane);
+          rank_step<PB, MASKED>(st[0], f, rank_group, rank_val0, rank_freq_width, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
           sym_step<PB, MASKED>(st[0], f, k, valid_lane);
         } else if constexpr (ILP == 2) {
@@ -909,7 +937,7 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
 #pragma unroll
       for (int f = 0; f < kFields; ++f) {
         if constexpr (MODE == kModeRank) {
-          rank_step<PB, true>(s, f, s.coset_base + rank_rs0, rank_val0, k, valid_lane);
+          rank_step<PB, true>(s, f, s.coset_base + rank_rs0, rank_val0, rank_freq_width, k, valid_lane);
         } else if constexpr (MODE == kModeSym) {
           sym_step<PB, true>(s, f, k, valid_lane);
         } else {

@@ -93,6 +93,7 @@ struct RankLayout {
   int present_offset[18];
   uint32_t val_offset;     // byte offsets inside the table area
   uint32_t rs_offset;
+  int values_half;         // values as half-precision coordinates (coset shift included) instead of 16-bit integers
 };
 
 __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __restrict__ meta,
@@ -138,7 +139,9 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
   uint32_t running = chunk_sum[tid];
   uint8_t* tables = reinterpret_cast<uint8_t*>(plan) + kHeaderBytes;
   if (kind == EP_TABLE_LDS_RANK) {
-    // Symbol-end bitmap + running symbol count per 32 slots, and per present symbol freq | cdf << 16 and its value.
+    // Symbol-end bitmap + running symbol count per 32 slots, and per present symbol cdf | freq << 16 | (value odd) << 31
+    // and its value: a 16-bit integer, or the lattice coordinate in half precision (z + c / 2; m + c / 4 for the last
+    // field, whose z7 = 2 m + parity the kernel forms with one multiply-add).
     uint32_t* fb = reinterpret_cast<uint32_t*>(tables);
     int16_t* val = reinterpret_cast<int16_t*>(tables + rank.val_offset);
     uint32_t* rs = reinterpret_cast<uint32_t*>(tables + rank.rs_offset) + (static_cast<size_t>(stream - 1) << prob_bits) / 32 * 2;
@@ -146,8 +149,15 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const int32_t* __rest
     for (int s = first; s < last; ++s) {
       const uint32_t f = freq[s];
       if (f == 0) continue;
-      fb[index] = f | (running << 16);
-      val[index] = static_cast<int16_t>(s + sym_min);
+      const int z = s + sym_min;
+      fb[index] = running | (f << 16) | (rank.values_half ? static_cast<uint32_t>(z & 1) << 31 : 0u);
+      if (rank.values_half) {
+        const int coset = (stream - 1) & 1, field = (stream - 1) >> 1;
+        const float coordinate = static_cast<float>(z) + (field == kFields - 1 ? 0.25f : 0.5f) * static_cast<float>(coset);
+        val[index] = __builtin_bit_cast(int16_t, static_cast<_Float16>(coordinate));
+      } else {
+        val[index] = static_cast<int16_t>(z);
+      }
       const uint32_t end = running + f - 1;
       if (end < size) atomicOr(&rs[(end >> 5) * 2], 1u << (end & 31));
       running += f;
@@ -254,6 +264,8 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
   int64_t cursor = 0;
   int max_alphabet = 0;
   bool byte_ok = true, wide_ok = true, rank_ok = true;
+  // Half precision holds z + 1/2 exactly for |z| < 1024 and m + 1/4 for |m| < 512; its entry keeps one bit beside a 15-bit frequency.
+  bool half_ok = prob_bits <= 14;
   int64_t present = 0;       // symbols with non-zero frequency in the field streams so far
   for (int s = 0; s < ep::kStreams; ++s) {
     const int64_t sym_min = meta[s * 4 + 1], off = meta[s * 4 + 2], alphabet = meta[s * 4 + 3];
@@ -272,6 +284,8 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
         if (sym_min < -128 || sym_min + alphabet - 1 > 127) byte_ok = false;
         if (alphabet > 1024 || top > 2047) wide_ok = false;
         if (sym_min < -32768 || sym_min + alphabet - 1 > 32767) rank_ok = false;
+        const int64_t exact = s >= ep::kStreams - 2 ? 511 : 1023;       // the last field's two streams code m, z7 = 2 m + parity
+        if (sym_min < -exact || sym_min + alphabet - 1 > exact) half_ok = false;
         for (int64_t i = 0; i < alphabet; ++i) present += freq[off + i] != 0;
       }
     }
@@ -309,6 +323,7 @@ int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_fre
     desc->lds_bytes = 0;
   } else if (kind == EP_TABLE_LDS_RANK) {
     desc->lds_bytes = static_cast<int>(ep::rank_table_bytes(static_cast<int>(present), prob_bits));
+    desc->rank_values_half = half_ok ? 1 : 0;
     desc->table_bytes = ep::kHeaderBytes + static_cast<size_t>(desc->lds_bytes);
   } else {
     desc->table_bytes = ep::kHeaderBytes + (static_cast<size_t>(ep::kFieldStreams) << prob_bits) * 4;
@@ -344,6 +359,8 @@ int ep_hip_plan_build(const int32_t* stream_meta_dev, const uint16_t* freq_table
     }
     rank.val_offset = static_cast<uint32_t>(ep::rank_fb_bytes(present));
     rank.rs_offset = static_cast<uint32_t>(ep::rank_rs_offset(present, desc->prob_bits));
+    rank.values_half = desc->rank_values_half != 0;
+    if (rank.values_half && desc->prob_bits > 14) return EP_HIP_EINVAL;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   // Slots of empty streams are never read, but keep the buffer deterministic; the rank form ORs into zeroed bitmaps.

@@ -25,6 +25,7 @@ struct DecodeArgs {
   uint32_t lut_bytes;       // LDS_RANK: bytes of tables to stage, and where the value and rank/select parts start
   uint32_t rank_val_offset;
   uint32_t rank_rs_offset;
+  uint32_t rank_half;       // LDS_RANK: the value table holds half-precision coordinates
   const uint8_t* sym_tables;   // the plan's two-level (LDS_SYM) section, or null
   // Multiply-on-the-fly kernels only: activations x[m_rows][ldx] (bf16) and the f32 accumulator y32[m_rows][ldy32].
   int m_rows;

@@ -18,7 +18,7 @@
 extern "C" {
 #endif
 
-#define EP_HIP_ABI_VERSION 1
+#define EP_HIP_ABI_VERSION 2
 
 enum ep_hip_status {
   EP_HIP_OK = 0,
@@ -84,6 +84,8 @@ typedef struct ep_hip_plan_desc {
   int sym_offset;             /* byte offset of the LDS_SYM section inside the plan buffer, 0 = none */
   int present_offset[18];     /* LDS_RANK: symbols with non-zero frequency in field streams before stream s (index s),
                                  [17] = their total; zero for the other kinds */
+  int rank_values_half;       /* LDS_RANK: 1 = the value table holds lattice coordinates in half precision (every value is
+                                 small enough to be exact there), 0 = 16-bit integers */
 } ep_hip_plan_desc;
 
 /* Library / device ------------------------------------------------------------------------------------------ */

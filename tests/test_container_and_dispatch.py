@@ -248,6 +248,15 @@ def test_plan_describe_rejects_inconsistent_tables():
     assert _describe(shifted, freq, 11)[0] == hip_backend.EINVAL               # offsets not contiguous
     assert _describe(meta, freq[:-1], 11)[0] == hip_backend.EINVAL
     assert _describe(meta, freq, 11, lds=64 * 1024)[1].table_kind == hip_backend.TABLE_LDS_RANK
+    # The rank/select form keeps its values in half precision while every coordinate is exact there: |z| < 1024, and
+    # |m| < 512 in the last field's two streams (z7 = 2 m + parity); a minimum beyond that keeps 16-bit integers.
+    assert _describe(meta, freq, 11, lds=64 * 1024)[1].rank_values_half == 1
+    assert _describe(meta, freq, 11)[1].rank_values_half == 0                  # only the rank/select form has the field set
+    for stream, minimum, expect in ((3, -1023, 1), (3, -1024, 0), (16, -511, 1), (16, -512, 0)):
+        far = meta.copy()
+        far[stream, 1] = minimum
+        status, desc = _describe(far, freq, 11, force=hip_backend.TABLE_LDS_RANK)
+        assert status == hip_backend.OK and desc.rank_values_half == expect, (stream, minimum)
     assert _describe(meta, freq, 11, lds=2 * 1024)[1].table_kind == hip_backend.TABLE_GLOBAL64
     assert _describe(meta, freq, 11, force=hip_backend.TABLE_GLOBAL64)[1].table_kind == hip_backend.TABLE_GLOBAL64
     assert _describe(meta, freq, 11, tile_elements=0)[0] == hip_backend.EINVAL

@@ -86,6 +86,34 @@ def test_dit_like_layer_at_each_rate(bpp):
     container, used = decode_and_check(gauss(3, 3840, 3840), kinds=(None, hip_backend.TABLE_GLOBAL64), target_bpp=bpp)
     assert abs(container.actual_bpp - bpp) < 0.12
     assert used[0] == ("lds_rank" if bpp > 7.0 else "lds_byte")
+    if bpp > 7.0:
+        # Values this small are exact in half precision: the rank/select tables hold the coordinates in that form.
+        on_gpu = container.to("cuda")
+        ep.decompress(on_gpu, ep.EntroPackLossyConfig(execution_backend="hip"))
+        lattice = LatticeBuffers(**{k: on_gpu.buffers[k] for k in LatticeBuffers._fields})
+        assert hip_lane.plan_of(lattice).desc.rank_values_half == 1
+
+
+def test_rank_tables_with_values_beyond_half_precision():
+    """One column a thousand times the rest: alphabets thousands of values wide with few of them present. The rank/select
+    tables then keep 16-bit integers (z + 1/2 is not exact in half precision beyond 1023) and the kernel its integer
+    reconstruction; the general kernel decodes the same container too."""
+    torch.manual_seed(26)
+    weight = torch.randn(32, 32768) * 0.02
+    weight[:, 100] *= 1000.0
+    container, used = decode_and_check(weight.to(torch.bfloat16), kinds=(hip_backend.TABLE_LDS_RANK, None, hip_backend.TABLE_GLOBAL64), target_bpp=4.0)
+    assert used[0] == "lds_rank"
+    on_gpu = container.to("cuda")
+    hip_lane.FORCE_TABLE_KIND = hip_backend.TABLE_LDS_RANK
+    try:
+        ep.decompress(on_gpu, ep.EntroPackLossyConfig(execution_backend="hip"))
+    finally:
+        hip_lane.FORCE_TABLE_KIND = None
+    lattice = LatticeBuffers(**{k: on_gpu.buffers[k] for k in LatticeBuffers._fields})
+    plan = hip_lane.plan_of(lattice)
+    assert plan.table_kind == "lds_rank" and plan.desc.rank_values_half == 0
+    meta = container.buffers["stream_meta"]
+    assert int(meta[1:, 1].min()) < -1023 or int((meta[1:, 1] + meta[1:, 3]).max()) > 1024
 
 
 @pytest.mark.parametrize("shape", [(3840, 11520), (10240, 3840)])
