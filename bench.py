@@ -27,8 +27,8 @@ HBM_PEAK_GBPS = 8000.0
 #: named profile was taken. `csrc_sha16` names those sources; when the kernels have changed since, the figure is not
 #: reported (`traffic` is null and `traffic_source` says why) instead of going stale silently.
 MEASURED_TRAFFIC = {
-    "target": {"bytes": 600_600_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "de8d4dbbfb1a2f18"},
-    "tile_ans": {"bytes": 818_700_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "2f34e254db80ae6b"},
+    "target": {"bytes": 599_800_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "c15e64bcd7fec39f"},
+    "tile_ans": {"bytes": 819_000_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "0f34596f8f8863b4"},
 }
 #: The kernel sources a traffic figure depends on, per workload.
 TRAFFIC_SOURCES = {
