@@ -115,6 +115,7 @@ _SIGNATURES = {
     "ep_hip_rotate_quantize_rows": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p,
         ctypes.c_void_p, ctypes.c_void_p]),
+    "ep_hip_probe_store_pattern": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 FLOAT_KINDS = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}

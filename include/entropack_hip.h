@@ -264,6 +264,15 @@ int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev,
 int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
                                     const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* stream);
 
+/* Measurement aid --------------------------------------------------------------------------------------------- */
+
+/* Writes `vectors` 16-byte vectors to `out_dev` (16-byte aligned) in the order and shape a bf16 lattice decode of tiles
+ * of `tile_vectors` vectors writes them (one tile per 32-lane half of a persistent grid, top-down in groups of 32
+ * vectors, 16 bytes per lane), with streaming stores like the decode kernels or, `through_cache` != 0, plain ones, and
+ * decodes nothing: the time of this launch is what the decode kernels' output side costs on its own.
+ * No counterpart in the reference; `bench.py --workload store_pattern` is its caller. */
+int ep_hip_probe_store_pattern(void* out_dev, int64_t vectors, int tile_vectors, int through_cache, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
