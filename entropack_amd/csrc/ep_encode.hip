@@ -1,0 +1,422 @@
+// The lattice_rans encoder on the device: nearest-E8 quantisation, stream statistics, row-scale refit and the tiled
+// 32-way interleaved rANS encode. Every kernel produces, from the same inputs, exactly what the CPU encoder
+// (csrc/host_codec.c) produces: the float work is single IEEE operations in the same order (this file is compiled
+// without contraction), the rest is integer work. The one exception is the row-scale refit, whose float32 row sums are
+// added in this kernel's own fixed order (the CPU lane adds them in torch's).
+//
+// Counterparts in the reference (entropack/schemes/lattice_rans/): the quantise kernels lattice_rans.cu:224, the refit
+// kernels :313, e8_minmax_fields_kernel :334, e8_histogram_kernel :376, e8_rans_encode_vector_kernel :400 and
+// e8_compact_kernel :467, launched from cuda.py:115-221 and :520-558. The algorithms followed are the eager lane's
+// (eager.py:18-58, rans.py:133-186), with which the reference states its kernels agree bit for bit
+// (lattice_rans.cu:3-18).
+#include <hip/hip_runtime.h>
+#include <limits.h>
+
+#include "entropack_hip.h"
+#include "ep_common.hpp"
+
+namespace ep {
+
+constexpr int kSummaryMinMax = 2 * kFieldStreams;       // summary[2 k], [2 k + 1]: least and greatest value of field stream k
+constexpr int kSummaryOnes = kSummaryMinMax;            // summary[32]: vectors of coset 1
+constexpr int kSummaryWords = kSummaryOnes + 1;
+static_assert(kSummaryWords == EP_HIP_ENCODE_SUMMARY_WORDS, "header and kernels agree on the summary's size");
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4v __attribute__((ext_vector_type(4)));
+
+__global__ void summary_init_kernel(long long* __restrict__ summary) {
+  const int k = threadIdx.x;
+  if (k < kSummaryMinMax) summary[k] = (k & 1) ? LLONG_MIN : LLONG_MAX;
+  else if (k == kSummaryOnes) summary[k] = 0;
+}
+
+// Nearest point of D8 (integer vectors with an even sum): round every coordinate to nearest-even; when the sum is odd,
+// move the coordinate that was rounded furthest (the first of equals) one step to its other side (up when its residual
+// is zero).
+__device__ __forceinline__ void nearest_d8(const float (&y)[8], float (&out)[8]) {
+  float total = 0.0f, best = -1.0f, residual_at_best = 0.0f;
+  int at = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    out[j] = __builtin_rintf(y[j]);
+    const float r = y[j] - out[j];
+    total += out[j];                          // small integers: exact
+    const float a = __builtin_fabsf(r);
+    if (a > best) { best = a; at = j; residual_at_best = r; }
+  }
+  const float halved = total * 0.5f;          // exact; a whole number exactly when the sum is even
+  const bool odd = halved != __builtin_rintf(halved);
+  const float step = residual_at_best < 0.0f ? -1.0f : 1.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) out[j] = (odd && j == at) ? out[j] + step : out[j];
+}
+
+// Squared distance in float64, added as ((0+4)+(2+6)) + ((1+5)+(3+7)): the order that decides exact ties between the
+// two cosets in the CPU encoder.
+__device__ __forceinline__ double distance2(const float (&y)[8], const float (&p)[8]) {
+  double s[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const double d = static_cast<double>(y[j]) - static_cast<double>(p[j]);
+    s[j] = d * d;
+  }
+  return ((s[0] + s[4]) + (s[2] + s[6])) + ((s[1] + s[5]) + (s[3] + s[7]));
+}
+
+// One thread per vector (grid-stride). y = (x / rms[row]) / scale, nearest E8 point = the nearer of the nearest D8 point
+// and the nearest point of D8 + 1/2 (the first on a tie), written as the coset bit and the fields z0..z6, m with
+// 2 m + parity(z0..z6) = z7. Every block folds the least and greatest field values it saw, per stream, into `summary`.
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, const float* __restrict__ rms, int64_t cols, float scale,
+                                                       const int64_t* __restrict__ row_index, int64_t vectors, int64_t vectors_per_row,
+                                                       int8_t* __restrict__ coset, int32_t* __restrict__ fields,
+                                                       long long* __restrict__ summary) {
+  __shared__ int lo_shared[kFieldStreams], hi_shared[kFieldStreams];
+  __shared__ unsigned ones_shared;
+  if (threadIdx.x < kFieldStreams) { lo_shared[threadIdx.x] = INT_MAX; hi_shared[threadIdx.x] = INT_MIN; }
+  if (threadIdx.x == 0) ones_shared = 0;
+  __syncthreads();
+
+  int lo[kFieldStreams], hi[kFieldStreams];
+#pragma unroll
+  for (int k = 0; k < kFieldStreams; ++k) { lo[k] = INT_MAX; hi[k] = INT_MIN; }
+  unsigned ones = 0;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t at = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; at < vectors; at += stride) {
+    const int64_t picked = at / vectors_per_row, v = at - picked * vectors_per_row;
+    const int64_t row = row_index != nullptr ? row_index[picked] : picked;
+    const f32x4* source = reinterpret_cast<const f32x4*>(x + row * cols + v * 8);
+    const f32x4 first = source[0], second = source[1];
+    const float raw[8] = {first.x, first.y, first.z, first.w, second.x, second.y, second.z, second.w};
+    const float norm = rms[row];
+    float y[8], shifted[8], p0[8], p1[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      y[j] = (raw[j] / norm) / scale;
+      shifted[j] = y[j] - 0.5f;
+    }
+    nearest_d8(y, p0);
+    nearest_d8(shifted, p1);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p1[j] += 0.5f;
+    const int c = !(distance2(y, p0) <= distance2(y, p1));
+    int z[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) z[j] = static_cast<int>(__builtin_rintf(c ? p1[j] - 0.5f : p0[j] - 0.0f));
+    const int parity = (z[0] + z[1] + z[2] + z[3] + z[4] + z[5] + z[6]) & 1;
+    z[7] = (z[7] - parity) >> 1;              // even for a lattice point; floor otherwise
+    coset[at] = static_cast<int8_t>(c);
+    i32x4v* to = reinterpret_cast<i32x4v*>(fields + at * 8);
+    to[0] = i32x4v{z[0], z[1], z[2], z[3]};
+    to[1] = i32x4v{z[4], z[5], z[6], z[7]};
+    ones += static_cast<unsigned>(c);
+#pragma unroll
+    for (int f = 0; f < kFields; ++f) {
+      const int k0 = 2 * f, k1 = 2 * f + 1;
+      lo[k0] = c ? lo[k0] : min(lo[k0], z[f]);
+      hi[k0] = c ? hi[k0] : max(hi[k0], z[f]);
+      lo[k1] = c ? min(lo[k1], z[f]) : lo[k1];
+      hi[k1] = c ? max(hi[k1], z[f]) : hi[k1];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kFieldStreams; ++k) {
+    if (lo[k] != INT_MAX) { atomicMin(&lo_shared[k], lo[k]); atomicMax(&hi_shared[k], hi[k]); }
+  }
+  if (ones != 0) atomicAdd(&ones_shared, ones);
+  __syncthreads();
+  if (threadIdx.x < kFieldStreams && lo_shared[threadIdx.x] != INT_MAX) {
+    atomicMin(&summary[2 * threadIdx.x], static_cast<long long>(lo_shared[threadIdx.x]));
+    atomicMax(&summary[2 * threadIdx.x + 1], static_cast<long long>(hi_shared[threadIdx.x]));
+  }
+  if (threadIdx.x == 0 && ones_shared != 0)
+    atomicAdd(reinterpret_cast<unsigned long long*>(&summary[kSummaryOnes]), static_cast<unsigned long long>(ones_shared));
+}
+
+// Counts of every symbol of every stream. bin_rel[s] = first bin of stream s - least value of stream s (stream 0 = the
+// coset bits, stream 1 + 2 f + c = field f of the vectors of coset c). STAGED: the block counts in LDS and adds what it
+// counted to the global bins at its end. A value whose bin lies outside [0, total_bins) is not counted (the caller
+// compares the bins' sum with the number of symbols).
+template <bool STAGED>
+__global__ __launch_bounds__(256) void histogram_kernel(const int8_t* __restrict__ coset, const int32_t* __restrict__ fields, int64_t vectors,
+                                                        const int32_t* __restrict__ bin_rel, int total_bins,
+                                                        unsigned long long* __restrict__ bins) {
+  extern __shared__ unsigned staged[];
+  __shared__ int rel[kStreams];
+  if (threadIdx.x < kStreams) rel[threadIdx.x] = bin_rel[threadIdx.x];
+  if (STAGED)
+    for (int b = threadIdx.x; b < total_bins; b += blockDim.x) staged[b] = 0;
+  __syncthreads();
+  auto count = [&](int bin) {
+    if (static_cast<unsigned>(bin) >= static_cast<unsigned>(total_bins)) return;
+    if (STAGED) atomicAdd(&staged[bin], 1u);
+    else atomicAdd(&bins[bin], 1ull);
+  };
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t at = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; at < vectors; at += stride) {
+    const int c = coset[at] != 0;
+    const i32x4v* from = reinterpret_cast<const i32x4v*>(fields + at * 8);
+    const i32x4v a = from[0], b = from[1];
+    const int z[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    count(rel[0] + c);
+#pragma unroll
+    for (int f = 0; f < kFields; ++f) count(rel[1 + 2 * f + c] + z[f]);
+  }
+  if (STAGED) {
+    __syncthreads();
+    for (int b = threadIdx.x; b < total_bins; b += blockDim.x)
+      if (staged[b] != 0) atomicAdd(&bins[b], static_cast<unsigned long long>(staged[b]));
+  }
+}
+
+__global__ void zero_words_kernel(unsigned long long* __restrict__ words, int64_t count) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride) words[i] = 0;
+}
+
+// Least-squares scale of a row against the lattice points chosen for it: sum(x p) / sum(p p) in float32, at least
+// 1e-12; scale * rms[row] for a row of zeros. One block per row; every thread adds its vectors (t, t + 256, ...) in
+// order, coordinate 0 to 7, and the 256 partial sums are added pairwise (t with t + 128, then + 64, ...).
+__global__ __launch_bounds__(256) void row_scales_kernel(const float* __restrict__ x, const float* __restrict__ rms, int64_t cols, float scale,
+                                                         const int8_t* __restrict__ coset, const int32_t* __restrict__ fields,
+                                                         float* __restrict__ scales) {
+  __shared__ float numerators[256], denominators[256];
+  const int64_t row = blockIdx.x, vectors_per_row = cols / 8;
+  float numerator = 0.0f, denominator = 0.0f;
+  for (int64_t v = threadIdx.x; v < vectors_per_row; v += 256) {
+    const int64_t at = row * vectors_per_row + v;
+    const f32x4* source = reinterpret_cast<const f32x4*>(x + row * cols + v * 8);
+    const f32x4 first = source[0], second = source[1];
+    const float raw[8] = {first.x, first.y, first.z, first.w, second.x, second.y, second.z, second.w};
+    const i32x4v* from = reinterpret_cast<const i32x4v*>(fields + at * 8);
+    const i32x4v a = from[0], b = from[1];
+    const int z[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const float half = coset[at] != 0 ? 0.5f : 0.0f;
+    const int parity = (z[0] + z[1] + z[2] + z[3] + z[4] + z[5] + z[6]) & 1;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float level = static_cast<float>(j < 7 ? z[j] : 2 * z[7] + parity) + half;
+      numerator += raw[j] * level;
+      denominator += level * level;
+    }
+  }
+  numerators[threadIdx.x] = numerator;
+  denominators[threadIdx.x] = denominator;
+  __syncthreads();
+  for (int width = 128; width > 0; width >>= 1) {
+    if (threadIdx.x < width) {
+      numerators[threadIdx.x] += numerators[threadIdx.x + width];
+      denominators[threadIdx.x] += denominators[threadIdx.x + width];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const float fitted = numerators[0] / denominators[0];
+    scales[row] = denominators[0] > 0.0f ? (fitted > 1.0e-12f ? fitted : 1.0e-12f) : scale * rms[row];
+  }
+}
+
+// One tile per 32-lane half of a wavefront, lane l carrying state l. A group of 32 vectors is one vector per lane; its
+// symbols go in last to first (field 7 ... field 0, then the coset bit), and the words the lanes push out in one step
+// are appended in lane order, as the sequential encoder appends them. entries[i] = freq | cdf << 16 of table position
+// i; table_rel[s] = first position of stream s - least value of stream s. A symbol outside the tables, or one of
+// frequency 0, raises *error and is coded with frequency 1 so that the launch still ends.
+__global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restrict__ coset, const int32_t* __restrict__ fields, int64_t vectors,
+                                                          int tile_vectors, int64_t tiles, const uint32_t* __restrict__ entries,
+                                                          const int32_t* __restrict__ table_rel, int total_entries, int prob_bits,
+                                                          uint32_t* __restrict__ states, uint32_t* __restrict__ tile_words,
+                                                          uint16_t* __restrict__ scratch, int* __restrict__ error) {
+  __shared__ int rel[kStreams];
+  if (threadIdx.x < kStreams) rel[threadIdx.x] = table_rel[threadIdx.x];
+  __syncthreads();
+  const int lane = threadIdx.x & 63, half = lane >> 5, l = lane & 31;
+  const int64_t tile = (static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2 + half;
+  if (tile >= tiles) return;
+  const int64_t begin = tile * tile_vectors;
+  const int64_t end = begin + tile_vectors < vectors ? begin + tile_vectors : vectors;
+  uint16_t* out = scratch + tile * (static_cast<int64_t>(tile_vectors) * 9);
+  const uint32_t below = (1u << l) - 1u;
+  const int renorm_shift = 31 - prob_bits;
+  uint32_t state = kStateMin, cursor = 0;
+  bool bad = false;
+  for (int64_t base = begin; base < end; base += kStatesPerTile) {
+    const bool valid = base + l < end;
+    int c = 0;
+    int z[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (valid) {
+      c = coset[base + l] != 0;
+      const i32x4v* from = reinterpret_cast<const i32x4v*>(fields + (base + l) * 8);
+      const i32x4v a = from[0], b = from[1];
+      z[0] = a.x; z[1] = a.y; z[2] = a.z; z[3] = a.w; z[4] = b.x; z[5] = b.y; z[6] = b.z; z[7] = b.w;
+    }
+#pragma unroll
+    for (int step = 0; step < 9; ++step) {
+      const int f = 7 - step;
+      const int position = step < 8 ? rel[1 + 2 * f + c] + z[f] : rel[0] + c;
+      uint32_t entry = 1u;
+      if (valid) {
+        if (static_cast<unsigned>(position) < static_cast<unsigned>(total_entries)) entry = entries[position];
+        else bad = true;
+      }
+      uint32_t freq = entry & 0xFFFFu;
+      const uint32_t cdf = entry >> 16;
+      if (freq == 0) { bad = true; freq = 1; }
+      const bool push = valid && state >= (freq << renorm_shift);
+      const uint32_t pushing = static_cast<uint32_t>(__ballot(push) >> (32 * half));
+      if (push) {
+        out[cursor + __popc(pushing & below)] = static_cast<uint16_t>(state & 0xFFFFu);
+        state >>= 16;
+      }
+      cursor += __popc(pushing);
+      if (valid) {
+        const uint32_t quotient = state / freq;
+        state = (quotient << prob_bits) + (state - quotient * freq) + cdf;
+      }
+    }
+  }
+  states[tile * kStatesPerTile + l] = state;
+  if (l == 0) tile_words[tile] = cursor;
+  if (bad) *error = 1;
+}
+
+// offsets[0] = 0, offsets[t + 1] = words of tiles 0..t (modulo 2^32; *total holds the full sum). One block.
+__global__ __launch_bounds__(1024) void offsets_kernel(const uint32_t* __restrict__ tile_words, int64_t tiles, uint32_t* __restrict__ offsets,
+                                                       unsigned long long* __restrict__ total) {
+  __shared__ unsigned long long sums[1024];
+  const int t = threadIdx.x;
+  const int64_t share = (tiles + 1023) / 1024;
+  const int64_t first = t * share, last = first + share < tiles ? first + share : tiles;
+  unsigned long long mine = 0;
+  for (int64_t i = first; i < last; ++i) mine += tile_words[i];
+  sums[t] = mine;
+  __syncthreads();
+  for (int distance = 1; distance < 1024; distance <<= 1) {
+    const unsigned long long before = t >= distance ? sums[t - distance] : 0;
+    __syncthreads();
+    sums[t] += before;
+    __syncthreads();
+  }
+  unsigned long long running = sums[t] - mine;
+  if (t == 0) offsets[0] = 0;
+  for (int64_t i = first; i < last; ++i) {
+    running += tile_words[i];
+    offsets[i + 1] = static_cast<uint32_t>(running);
+  }
+  if (t == 1023) *total = sums[1023];
+}
+
+// payload[offsets[t] ..) = the words tile t left at the start of its part of the scratch.
+__global__ __launch_bounds__(256) void gather_kernel(const uint16_t* __restrict__ scratch, const uint32_t* __restrict__ offsets, int64_t tiles,
+                                                     int tile_vectors, uint16_t* __restrict__ payload) {
+  const int64_t stride = static_cast<int64_t>(tile_vectors) * 9;
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const uint32_t from = offsets[tile], words = offsets[tile + 1] - from;
+    const uint16_t* source = scratch + tile * stride;
+    for (uint32_t i = threadIdx.x; i < words && i < stride; i += blockDim.x) payload[static_cast<uint64_t>(from) + i] = source[i];
+  }
+}
+
+static int grid_for(int64_t items, int per_block, int* blocks) {
+  int device = 0, cus = 0;
+  EP_HIP_TRY(hipGetDevice(&device));
+  EP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+  const int64_t wanted = (items + per_block - 1) / per_block, most = static_cast<int64_t>(cus > 0 ? cus : 256) * 8;
+  *blocks = static_cast<int>(wanted < 1 ? 1 : (wanted < most ? wanted : most));
+  return EP_HIP_OK;
+}
+
+}  // namespace ep
+
+extern "C" int ep_hip_encode_quantize(const float* x_dev, const float* rms_dev, int64_t cols, float scale, const int64_t* row_index_dev,
+                                      int64_t rows, int8_t* coset_dev, int32_t* fields_dev, int64_t* summary_dev, void* stream) {
+  if (x_dev == nullptr || rms_dev == nullptr || coset_dev == nullptr || fields_dev == nullptr || summary_dev == nullptr) return EP_HIP_EINVAL;
+  if (rows <= 0 || cols <= 0 || cols % 8 != 0 || !(scale > 0.0f)) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(summary_dev) % 8 != 0)
+    return EP_HIP_EINVAL;
+  const int64_t vectors_per_row = cols / 8, vectors = rows * vectors_per_row;
+  int blocks = 0;
+  const int status = ep::grid_for(vectors, 256, &blocks);
+  if (status != EP_HIP_OK) return status;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(ep::summary_init_kernel, dim3(1), dim3(64), 0, s, reinterpret_cast<long long*>(summary_dev));
+  hipLaunchKernelGGL(ep::quantize_kernel, dim3(blocks), dim3(256), 0, s, x_dev, rms_dev, cols, scale, row_index_dev, vectors, vectors_per_row,
+                     coset_dev, fields_dev, reinterpret_cast<long long*>(summary_dev));
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_encode_histogram(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const int32_t* bin_rel_dev,
+                                       int32_t total_bins, uint64_t* bins_dev, void* stream) {
+  if (coset_dev == nullptr || fields_dev == nullptr || bin_rel_dev == nullptr || bins_dev == nullptr) return EP_HIP_EINVAL;
+  if (vectors <= 0 || total_bins <= 0 || reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(bins_dev) % 8 != 0)
+    return EP_HIP_EINVAL;
+  int blocks = 0;
+  const int status = ep::grid_for(vectors, 256 * 8, &blocks);
+  if (status != EP_HIP_OK) return status;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(ep::zero_words_kernel, dim3((total_bins + 255) / 256), dim3(256), 0, s, reinterpret_cast<unsigned long long*>(bins_dev),
+                     static_cast<int64_t>(total_bins));
+  constexpr int kMostStagedBins = 15360;      // 60 KiB of LDS
+  if (total_bins <= kMostStagedBins)
+    hipLaunchKernelGGL(ep::histogram_kernel<true>, dim3(blocks), dim3(256), static_cast<size_t>(total_bins) * 4, s, coset_dev, fields_dev, vectors,
+                       bin_rel_dev, total_bins, reinterpret_cast<unsigned long long*>(bins_dev));
+  else
+    hipLaunchKernelGGL(ep::histogram_kernel<false>, dim3(blocks), dim3(256), 0, s, coset_dev, fields_dev, vectors, bin_rel_dev, total_bins,
+                       reinterpret_cast<unsigned long long*>(bins_dev));
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_encode_row_scales(const float* x_dev, const float* rms_dev, int64_t cols, float scale, int64_t rows,
+                                        const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, void* stream) {
+  if (x_dev == nullptr || rms_dev == nullptr || coset_dev == nullptr || fields_dev == nullptr || scales_dev == nullptr) return EP_HIP_EINVAL;
+  if (rows <= 0 || cols <= 0 || cols % 8 != 0) return EP_HIP_EINVAL;
+  if (rows > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0) return EP_HIP_EINVAL;
+  hipLaunchKernelGGL(ep::row_scales_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream), x_dev, rms_dev,
+                     cols, scale, coset_dev, fields_dev, scales_dev);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const uint32_t* entries_dev,
+                                  const int32_t* table_rel_dev, int32_t total_entries, int prob_bits, int tile_vectors,
+                                  uint32_t* states_dev, uint32_t* tile_words_dev, uint16_t* scratch_dev, int32_t* error_dev, void* stream) {
+  if (coset_dev == nullptr || fields_dev == nullptr || entries_dev == nullptr || table_rel_dev == nullptr || states_dev == nullptr ||
+      tile_words_dev == nullptr || scratch_dev == nullptr || error_dev == nullptr)
+    return EP_HIP_EINVAL;
+  if (vectors <= 0 || total_entries <= 0 || prob_bits < 1 || prob_bits > 15 || tile_vectors < ep::kStatesPerTile) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0) return EP_HIP_EINVAL;
+  const int64_t tiles = (vectors + tile_vectors - 1) / tile_vectors;
+  const int64_t blocks = (tiles + 7) / 8;                 // 4 wavefronts of two tiles each
+  if (blocks > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
+  hipLaunchKernelGGL(ep::rans_encode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), coset_dev,
+                     fields_dev, vectors, tile_vectors, tiles, entries_dev, table_rel_dev, total_entries, prob_bits, states_dev, tile_words_dev,
+                     scratch_dev, error_dev);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_encode_offsets(const uint32_t* tile_words_dev, int64_t tiles, uint32_t* offsets_dev, uint64_t* total_words_dev,
+                                     void* stream) {
+  if (tile_words_dev == nullptr || offsets_dev == nullptr || total_words_dev == nullptr || tiles <= 0) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(total_words_dev) % 8 != 0) return EP_HIP_EINVAL;
+  hipLaunchKernelGGL(ep::offsets_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), tile_words_dev, tiles, offsets_dev,
+                     reinterpret_cast<unsigned long long*>(total_words_dev));
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int tile_vectors,
+                                    uint16_t* payload_dev, void* stream) {
+  if (scratch_dev == nullptr || offsets_dev == nullptr || payload_dev == nullptr || tiles <= 0 || tile_vectors < ep::kStatesPerTile)
+    return EP_HIP_EINVAL;
+  int blocks = 0;
+  const int status = ep::grid_for(tiles, 1, &blocks);
+  if (status != EP_HIP_OK) return status;
+  hipLaunchKernelGGL(ep::gather_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), scratch_dev, offsets_dev, tiles,
+                     tile_vectors, payload_dev);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}

@@ -1,6 +1,6 @@
 /* libentropack_host.so: CPU encoder kernels of the lattice_rans scheme (plain C + OpenMP, no GPU).
  *
- * The MI355X path only decodes. Containers still have to come from somewhere, so the package carries its own
+ * Tensors on the CPU are encoded on the CPU: the package carries its own
  * CPU restatement of the reference encoder; the heavy loops live here and the orchestration (scale search,
  * Hamilton normalisation, row-scale refit) in schemes/lattice_rans/eager.py. Algorithms followed, in the
  * reference tree:

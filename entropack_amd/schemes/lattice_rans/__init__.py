@@ -2,7 +2,7 @@
 
 Public behaviour of the reference scheme (entropack/schemes/lattice_rans/__init__.py:13-58): 2-D inputs of the
 supported dtypes, columns padded to whole 8-vectors for the lane and cut back after decoding, buffers returned on the
-device the input came from. Lanes here: `hip` decodes on an MI355X, `eager` encodes on the CPU.
+device the input came from. Lanes here: `hip` decodes and encodes on an MI355X, `eager` encodes on the CPU.
 """
 import torch
 

@@ -1,6 +1,6 @@
 """`eager` (CPU) lane of lattice_rans: the encoder.
 
-The accelerated path of this package is decode-only; this lane produces the containers it decodes. It restates the
+CPU tensors are encoded here (tensors on an MI355X by the `hip` lane, with this module's orchestration). It restates the
 reference's CPU encoder (entropack/schemes/lattice_rans/eager.py:91-341 and rans.py:12-95,133-258) so that the same
 input and config give the same container, bit for bit: row RMS normalisation, a bisection of the lattice scale
 against an analytic size model on a seeded row subsample, nearest-E8 quantisation, least-squares refit of the row
@@ -116,6 +116,29 @@ def quantize(x: np.ndarray, rms: np.ndarray, scale: float, rows_selected: np.nda
     return Quantized(coset, fields)
 
 
+class HostQuantizer:
+    """The float32 matrix and its row RMS on the CPU; quantises and refits through libentropack_host.so.
+
+    The scale search below talks to this interface only (`rows`, `cols`, `all_zero`, `quantize`, `refit`), which the
+    device lane implements with its own kernels.
+    """
+
+    def __init__(self, x_t: torch.Tensor, rms_t: torch.Tensor):
+        self.x_t, self.rms_t = x_t, rms_t
+        self.rows, self.cols = x_t.shape
+        self._x = x_t.numpy()
+        self._rms = np.ascontiguousarray(rms_t.squeeze(1).numpy())
+
+    def all_zero(self) -> bool:
+        return float(self.x_t.abs().amax()) == 0.0
+
+    def quantize(self, scale: float, rows_selected: np.ndarray | None = None) -> Quantized:
+        return quantize(self._x, self._rms, scale, rows_selected)
+
+    def refit(self, q: Quantized, scale: float) -> torch.Tensor:
+        return refit_row_scales(self.x_t, self.rms_t, q, scale)
+
+
 # ---- frequency tables and the size model -------------------------------------------------------------------------
 
 def normalize_counts(counts: np.ndarray, table_size: int) -> np.ndarray:
@@ -179,19 +202,20 @@ def modelled_bytes(histograms, sizes, rows: int, prob_bits: int, tile_elements: 
     return coded + overflow_bits / 8 + rows * 4 + MODEL_LAYOUT_BYTES + MODEL_STREAM_META_BYTES + MODEL_SLACK_BYTES
 
 
-def _model_of(q: Quantized, rows: int, prob_bits: int, tile_elements: int) -> float:
+def _model_of(q, rows: int, prob_bits: int, tile_elements: int) -> float:
     stats = q.stats()
     return modelled_bytes(q.histograms(stats), [int(n) for n in stats[:, 0]], rows, prob_bits, tile_elements)
 
 
-def _largest_alphabet(q: Quantized) -> int:
+def _largest_alphabet(q) -> int:
     stats = q.stats()
     spans = np.where(stats[:, 0] > 0, stats[:, 2] - stats[:, 1] + 1, 0)
     return int(spans.max())
 
 
-def bisect_scale(x, rms, rows, cols, target_bpp, prob_bits, tile_elements, iterations, max_vectors) -> float:
+def bisect_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, max_vectors) -> float:
     """Geometric bisection of the lattice scale on [0.001, 8] against the size model, on a seeded row subsample."""
+    rows, cols = quantizer.rows, quantizer.cols
     per_row = cols // LATTICE_DIM
     sample_rows = max(1, min(rows, max_vectors // per_row))
     picked = None
@@ -202,7 +226,7 @@ def bisect_scale(x, rms, rows, cols, target_bpp, prob_bits, tile_elements, itera
     low, high = 0.001, 8.0
     for _ in range(iterations):
         middle = math.sqrt(low * high)
-        size = _model_of(quantize(x, rms, middle, picked), sample_rows, prob_bits, tile_elements)
+        size = _model_of(quantizer.quantize(middle, picked), sample_rows, prob_bits, tile_elements)
         if 8 * size / elements > target_bpp:
             low = middle
         else:
@@ -219,23 +243,20 @@ def refit_row_scales(x_t: torch.Tensor, rms_t: torch.Tensor, q: Quantized, scale
     return torch.where(denominator > 0, (numerator / denominator).clamp_min(MIN_RMS), scale * rms_t.squeeze(1))
 
 
-def resolve_scale(x_t, rms_t, target_bpp, prob_bits, tile_elements, iterations, max_vectors):
+def resolve_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, max_vectors):
     """Scale search plus the alphabet guard: grow an automatic prob_bits (to 15 at most) while an alphabet overflows
     the table, after that coarsen the scale by the overflow. Returns (quantised vectors, row scales, prob_bits)."""
-    rows, cols = x_t.shape
-    x = x_t.numpy()
-    rms = np.ascontiguousarray(rms_t.squeeze(1).numpy())
     prob_bits, automatic = resolve_prob_bits(prob_bits, target_bpp)
-    if float(x_t.abs().amax()) == 0.0:
-        q = quantize(x, rms, 1.0)
-        return q, refit_row_scales(x_t, rms_t, q, 1.0), prob_bits
+    if quantizer.all_zero():
+        q = quantizer.quantize(1.0)
+        return q, quantizer.refit(q, 1.0), prob_bits
     clamped = False
     while True:
         table_size = 1 << prob_bits
-        scale = bisect_scale(x, rms, rows, cols, target_bpp, prob_bits, tile_elements, iterations, max_vectors)
+        scale = bisect_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, max_vectors)
         grow = False
         while True:
-            q = quantize(x, rms, scale)
+            q = quantizer.quantize(scale)
             widest = _largest_alphabet(q)
             if widest <= table_size:
                 break
@@ -250,16 +271,15 @@ def resolve_scale(x_t, rms_t, target_bpp, prob_bits, tile_elements, iterations, 
         if clamped:
             log.debug("lattice_rans coarsened the lattice scale to %.6g so a coordinate alphabet of %d fits the "
                       "%d-entry rANS table; actual_bpp for this tensor will fall below target_bpp", scale, widest, table_size)
-        return q, refit_row_scales(x_t, rms_t, q, scale), prob_bits
+        return q, quantizer.refit(q, scale), prob_bits
 
 
 # ---- stream encode ---------------------------------------------------------------------------------------------
 
-def encode_streams(q: Quantized, prob_bits: int, tile_elements: int):
-    """Frequency tables + tiled rANS encode. Returns payload, states, offsets, stream_meta, freq_tables (numpy)."""
+def stream_tables(stats: np.ndarray, histograms, prob_bits: int):
+    """stream_meta and the normalised frequencies / cumulative frequencies of all streams, concatenated in stream order
+    (int64 numpy arrays; entropack/schemes/lattice_rans/cuda.py:481-517 is the reference's form of this step)."""
     table_size = 1 << prob_bits
-    stats = q.stats()
-    histograms = q.histograms(stats)
     meta = np.zeros((NUM_STREAMS, META_WIDTH), dtype=np.int64)
     freq_parts, cdf_parts = [], []
     cursor = 0
@@ -276,6 +296,13 @@ def encode_streams(q: Quantized, prob_bits: int, tile_elements: int):
             cursor += hist.size
     freq_all = np.concatenate(freq_parts) if freq_parts else np.zeros(0, dtype=np.int64)
     cdf_all = np.concatenate(cdf_parts) if cdf_parts else np.zeros(0, dtype=np.int64)
+    return meta, freq_all, cdf_all
+
+
+def encode_streams(q: Quantized, prob_bits: int, tile_elements: int):
+    """Frequency tables + tiled rANS encode. Returns payload, states, offsets, stream_meta, freq_tables (numpy)."""
+    stats = q.stats()
+    meta, freq_all, cdf_all = stream_tables(stats, q.histograms(stats), prob_bits)
 
     tile_vectors = vector_tile_elements(tile_elements)
     tiles = max(1, (q.vectors + tile_vectors - 1) // tile_vectors)
@@ -307,22 +334,32 @@ def _as_torch(array: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
     return torch.from_numpy(np.ascontiguousarray(array).view(signed)).view(dtype)
 
 
-def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0, row_rdo_candidates=5,
-           scale_search_iterations=12, scale_search_max_vectors=262144) -> LatticeBuffers:
+def check_encode_request(weight, row_rdo_iterations) -> None:
     if int(row_rdo_iterations) > 0:
         raise NotImplementedError("per-row rate-distortion refinement is not part of this build; use row_rdo_iterations=0")
     if weight.shape[1] % LATTICE_DIM:
         raise ValueError(
             f"lattice_rans quantizes whole E8 vectors, so the column count must be a multiple of {LATTICE_DIM}; got cols={weight.shape[1]}")
-    device = weight.device
-    x_t = weight.detach().to("cpu").float().contiguous()
-    rows, cols = x_t.shape
+
+
+def row_rms(x_t: torch.Tensor, source_dtype) -> torch.Tensor:
+    """float32 [rows, 1]: root mean square of every row, at least MIN_RMS (torch's reductions on the tensor's device)."""
     rms_t = x_t.square().mean(dim=1, keepdim=True).sqrt().clamp_min(MIN_RMS)
     if not bool(torch.isfinite(rms_t).all()):
         raise ValueError(
-            f"lattice_rans normalizes rows in fp32, and the row RMS of this {weight.dtype} tensor overflowed; rescale the source")
+            f"lattice_rans normalizes rows in fp32, and the row RMS of this {source_dtype} tensor overflowed; rescale the source")
+    return rms_t
+
+
+def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0, row_rdo_candidates=5,
+           scale_search_iterations=12, scale_search_max_vectors=262144) -> LatticeBuffers:
+    check_encode_request(weight, row_rdo_iterations)
+    device = weight.device
+    x_t = weight.detach().to("cpu").float().contiguous()
+    rows, cols = x_t.shape
+    rms_t = row_rms(x_t, weight.dtype)
     q, scales, prob_bits = resolve_scale(
-        x_t, rms_t, float(target_bpp), None if prob_bits in (None, 0) else int(prob_bits), int(tile_elements),
+        HostQuantizer(x_t, rms_t), float(target_bpp), None if prob_bits in (None, 0) else int(prob_bits), int(tile_elements),
         int(scale_search_iterations), int(scale_search_max_vectors))
     payload, states, offsets, meta, freq_tables = encode_streams(q, prob_bits, int(tile_elements))
     return LatticeBuffers(

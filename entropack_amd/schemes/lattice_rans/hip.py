@@ -1,4 +1,4 @@
-"""`hip` lane of lattice_rans: decode on an MI355X through the C ABI of libentropack_hip.so.
+"""`hip` lane of lattice_rans: decode (and encode, hip_encode.py) on an MI355X through the C ABI of libentropack_hip.so.
 
 Module-level `decode(buffers, *, shape, dtype, threads_per_block, l2_prefetch)` is the lane contract of the
 reference's CUDA lane (entropack/schemes/lattice_rans/cuda.py:781-805): all buffers on the device, result
@@ -348,9 +348,7 @@ def check_errors(buffers: LatticeBuffers) -> None:
 
 
 def encode(**kwargs):
-    """Encoding is CPU work in this package; the scheme routes it to the eager lane."""
-    from . import eager
-    weight = kwargs.pop("weight")
-    device = weight.device
-    packed = eager.encode(weight=weight.cpu(), **kwargs)
-    return LatticeBuffers._make(value.to(device) for value in packed)
+    """Lane contract of the reference's CUDA lane (entropack/schemes/lattice_rans/cuda.py:561-597): the weight is on the
+    device and so are the buffers returned. The kernels and their orchestration live in hip_encode.py."""
+    from . import hip_encode
+    return hip_encode.encode(**kwargs)

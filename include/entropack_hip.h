@@ -264,6 +264,62 @@ int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev,
 int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
                                     const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* stream);
 
+/* Encoder (the step before the path) -------------------------------------------------------------------------- *
+ *
+ * The device form of the lattice_rans encoder, one entry point per kernel of the reference's CUDA lane. All pointers are
+ * device pointers; nothing is allocated, nothing synchronises, every launch goes to `stream`. From the same inputs
+ * the integer outputs (coset bits, fields, summary, bins, states, offsets, payload) are bit-identical to the CPU
+ * encoder's (entropack/schemes/lattice_rans/eager.py:18-58, rans.py:133-186), as the reference states of its own
+ * kernels (lattice_rans.cu:3-18); the refitted row scales are float32 sums added in a fixed order of this library's own.
+ * A coset bit is 0 (point of D8) or 1 (point of D8 + 1/2); the fields of a vector are z0..z6 and m, where the point is
+ * (z0..z6, 2 m + parity(z0 + .. + z6)) + coset / 2. Stream 0 carries the coset bits, stream 1 + 2 f + c field f of the
+ * vectors of coset c. */
+
+#define EP_HIP_ENCODE_SUMMARY_WORDS 33
+
+/* Quantises `rows` rows of x[.][cols] (float32, 16-byte aligned, cols a multiple of 8): row i of the output is row
+ * row_index_dev[i] of x (row i when row_index_dev is NULL); y = (x / rms[row]) / scale, nearest E8 point, the first of
+ * equally near ones in the order D8, D8 + 1/2. coset_dev: int8[rows * cols / 8]; fields_dev: int32[rows * cols / 8][8]
+ * (16-byte aligned). summary_dev: int64[EP_HIP_ENCODE_SUMMARY_WORDS], set by the call: [2 k], [2 k + 1] = least and
+ * greatest value of field stream k = 2 f + c (INT64_MAX, INT64_MIN for a stream without symbols), [32] = number of
+ * vectors of coset 1. Replaces the quantise launch and the min/max pass of the reference's CUDA lane
+ * (entropack/schemes/lattice_rans/cuda.py:115-139, lattice_rans.cu:224,334). */
+int ep_hip_encode_quantize(const float* x_dev, const float* rms_dev, int64_t cols, float scale, const int64_t* row_index_dev,
+                           int64_t rows, int8_t* coset_dev, int32_t* fields_dev, int64_t* summary_dev, void* stream);
+
+/* Counts the symbols of all 17 streams into bins_dev (uint64[total_bins], cleared by the call): a symbol of value z of
+ * stream s is counted in bin bin_rel_dev[s] + z, i.e. bin_rel_dev[s] = first bin of the stream - its least value
+ * (int32[17]). Values whose bin falls outside [0, total_bins) are not counted. Replaces cuda.py:181-221
+ * (e8_histogram_kernel, lattice_rans.cu:376). */
+int ep_hip_encode_histogram(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const int32_t* bin_rel_dev,
+                            int32_t total_bins, uint64_t* bins_dev, void* stream);
+
+/* Least-squares row scales against the chosen points: scales_dev[r] = max(sum(x p) / sum(p p), 1e-12) in float32, or
+ * scale * rms[r] for a row whose points are all zero. Replaces cuda.py:142-158 (the refit kernels, lattice_rans.cu:313). */
+int ep_hip_encode_row_scales(const float* x_dev, const float* rms_dev, int64_t cols, float scale, int64_t rows,
+                             const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, void* stream);
+
+/* Tiled 32-way interleaved rANS encode of `vectors` vectors in tiles of `tile_vectors` (>= 32). entries_dev:
+ * uint32[total_entries], frequency | cumulative frequency << 16 of every table position; table_rel_dev: int32[17], first
+ * position of stream s - its least value. states_dev: uint32[tiles][32]; tile_words_dev: uint32[tiles], the number of
+ * payload words of each tile, which the tile leaves at scratch_dev[tile * tile_vectors * 9 ..) (uint16[tiles *
+ * tile_vectors * 9]). *error_dev (int32, cleared by the caller) becomes 1 when a symbol lies outside the tables or has
+ * frequency 0; the outputs are then not a valid container. Replaces cuda.py:520-541 (e8_rans_encode_vector_kernel,
+ * lattice_rans.cu:400). */
+int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const uint32_t* entries_dev,
+                       const int32_t* table_rel_dev, int32_t total_entries, int prob_bits, int tile_vectors, uint32_t* states_dev,
+                       uint32_t* tile_words_dev, uint16_t* scratch_dev, int32_t* error_dev, void* stream);
+
+/* offsets_dev[0] = 0, offsets_dev[t + 1] = tile_words_dev[0] + .. + tile_words_dev[t] modulo 2^32 (uint32[tiles + 1]);
+ * *total_words_dev (uint64, 8-byte aligned) = the sum itself, which the caller compares with 2^32 and sizes the payload
+ * by. Replaces the cumulative sum of cuda.py:542-551. */
+int ep_hip_encode_offsets(const uint32_t* tile_words_dev, int64_t tiles, uint32_t* offsets_dev, uint64_t* total_words_dev, void* stream);
+
+/* payload_dev[offsets_dev[t] ..) = the words of tile t from the scratch of ep_hip_encode_rans. Replaces cuda.py:552-557
+ * (e8_compact_kernel, lattice_rans.cu:467). */
+int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int tile_vectors,
+                         uint16_t* payload_dev, void* stream);
+
 /* Measurement aid --------------------------------------------------------------------------------------------- */
 
 /* Writes `vectors` 16-byte vectors to `out_dev` (16-byte aligned) in the order and shape a bf16 lattice decode of tiles
