@@ -1,6 +1,6 @@
 """Headline benchmark: lossy (lattice_rans) decode throughput on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|store_pattern|encode]
 
 One "step" = one decode of the whole container (entropy decode + E8 reconstruction + BF16 store) from buffers
 already resident in HBM. Prints ONE JSON line. `value` = algorithmic bytes (container bytes read + dense bytes
@@ -716,6 +716,142 @@ def store_pattern_workload(args, ep):
     return 0
 
 
+def encode_workload(args, ep):
+    """The step before the path: `compress` of the target weight (8192 x 28672 bf16, 4.0 bpp) on the device
+    (`hip_encode.encode`, kernels `ep_hip_encode_*`), whole call with its host synchronisations, then kernel by kernel
+    between events with the clocks settled. Parity: the first 1024 rows encoded by both lanes from the CPU lane's row
+    RMS give byte-identical buffers (scales to 1e-5); the full container decodes without an error flag to the rate and
+    error the CPU lane's container of the sample has. CPU baseline: this package's CPU encoder (bit-identical to the
+    reference's eager lane on the golden containers) on 2048 rows, scaled by rows."""
+    from entropack_amd.backends import hip as hip_backend
+    from entropack_amd.schemes.lattice_rans import eager, hip_encode
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    from entropack_amd.schemes.lattice_rans.format import LatticeBuffers, recommended_tile_elements, vector_tile_elements
+    rows, cols, sigma, seed, bpp, outliers = WORKLOADS["target"]
+    weight = make_weight(rows, cols, sigma, seed, outliers)
+    tile_elements = recommended_tile_elements(bpp)
+    options = dict(target_bpp=bpp, prob_bits=None, tile_elements=tile_elements)
+    on_gpu = weight.cuda()
+    hip_encode.encode(weight=on_gpu[:256], **options)                      # loads the library, warms the allocator
+    torch.cuda.synchronize()
+    walls = []
+    for _ in range(3):
+        start = time.perf_counter()
+        buffers = hip_encode.encode(weight=on_gpu, **options)
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - start)
+    wall = sorted(walls)[1]
+
+    # the full container: decodes cleanly, at the rate asked for
+    config = ep.EntroPackLossyConfig(target_bpp=bpp, execution_backend="hip")
+    restored = hip_lane.decode(buffers, shape=(rows, cols), dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    hip_lane.check_errors(buffers)
+    stored = sum(t.numel() * t.element_size() for t in buffers)
+    actual_bpp = 8.0 * stored / (rows * cols)
+    error = float((restored.float() - on_gpu.float()).norm() / on_gpu.float().norm())
+    del restored
+
+    # parity and CPU baseline on a sample of rows
+    sample_rows, cpu_rows = 1024, 2048
+    sample = weight[:sample_rows].float().contiguous()
+    rms = eager.row_rms(sample, weight.dtype)
+    start = time.perf_counter()
+    cpu_container = eager.encode(weight=weight[:cpu_rows], **options)
+    cpu_seconds = time.perf_counter() - start
+    cpu_sample = eager.encode(weight=sample, **options)
+    gpu_sample = hip_encode.encode_normalised(sample.cuda(), rms.cuda(), **options)
+    identical = all(torch.equal(a.cpu(), b) for key, a, b in zip(LatticeBuffers._fields, gpu_sample, cpu_sample) if key != "scales")
+    scales_close = bool(torch.allclose(gpu_sample.scales.cpu(), cpu_sample.scales, rtol=1e-5, atol=0.0))
+    cpu_dense = ep.decompress(ep.compress(weight[:cpu_rows], ep.EntroPackLossyConfig(target_bpp=bpp, execution_backend="eager")).to("cuda"), config)
+    cpu_error = float((cpu_dense.float() - on_gpu[:cpu_rows].float()).norm() / on_gpu[:cpu_rows].float().norm())
+    cpu_bpp = 8.0 * sum(t.numel() * t.element_size() for t in cpu_container) / (cpu_rows * cols)
+    parity = identical and scales_close and abs(actual_bpp - cpu_bpp) <= 0.01 * cpu_bpp and abs(error - cpu_error) <= 0.01 * cpu_error
+
+    # kernel by kernel
+    library, stream = hip_backend.library(), torch.cuda.current_stream().cuda_stream
+    x = on_gpu.float().contiguous()
+    quantizer = hip_encode.DeviceQuantizer(x, hip_encode.row_rms(x, weight.dtype))
+    scale = eager.bisect_scale(quantizer, bpp, 11, tile_elements, 12, 262144)
+    q = quantizer.quantize(scale)
+    stats = q.stats()
+    meta, freq_all, cdf_all = eager.stream_tables(stats, q.histograms(stats), 11)
+    vectors, tile_vectors = q.vectors, vector_tile_elements(tile_elements)
+    tiles = (vectors + tile_vectors - 1) // tile_vectors
+
+    def timed(fn, count=20):
+        settle(fn, 0.1)
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record()
+        for _ in range(count):
+            fn()
+        last.record()
+        torch.cuda.synchronize()
+        return first.elapsed_time(last) / count * 1e3
+
+    def check(status):
+        if status:
+            raise hip_backend.HipError("ep_hip_encode", status, "")
+
+    summary = torch.empty(33, dtype=torch.int64, device="cuda")
+    alphabets = np.where(stats[:, 0] > 0, stats[:, 2] - stats[:, 1] + 1, 0)
+    starts = np.concatenate([[0], np.cumsum(alphabets)]).astype(np.int64)
+    bin_rel = torch.from_numpy((starts[:17] - stats[:, 1]).astype(np.int32)).cuda()
+    bins = torch.empty(int(starts[-1]), dtype=torch.int64, device="cuda")
+    scales = torch.empty(rows, dtype=torch.float32, device="cuda")
+    entries = hip_encode.table_entries(freq_all, cdf_all).cuda()
+    table_rel = torch.from_numpy((meta[:, 2] - meta[:, 1]).astype(np.int32)).cuda()
+    states = torch.empty((tiles, 32), dtype=torch.int32, device="cuda")
+    tile_words = torch.empty(tiles, dtype=torch.int32, device="cuda")
+    scratch = torch.empty(tiles * tile_vectors * 9, dtype=torch.int16, device="cuda")
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    offsets = torch.empty(tiles + 1, dtype=torch.int32, device="cuda")
+    total = torch.empty(1, dtype=torch.int64, device="cuda")
+    kernels = {}
+    kernels["quantize"] = (timed(lambda: check(library.ep_hip_encode_quantize(
+        x.data_ptr(), quantizer.rms.data_ptr(), cols, scale, 0, rows, q.coset.data_ptr(), q.fields.data_ptr(), summary.data_ptr(), stream))),
+        4 * rows * cols + 33 * vectors)
+    kernels["histogram"] = (timed(lambda: check(library.ep_hip_encode_histogram(
+        q.coset.data_ptr(), q.fields.data_ptr(), vectors, bin_rel.data_ptr(), bins.numel(), bins.data_ptr(), stream))), 33 * vectors)
+    kernels["row_scales"] = (timed(lambda: check(library.ep_hip_encode_row_scales(
+        x.data_ptr(), quantizer.rms.data_ptr(), cols, scale, rows, q.coset.data_ptr(), q.fields.data_ptr(), scales.data_ptr(), stream))),
+        4 * rows * cols + 33 * vectors)
+    kernels["rans"] = (timed(lambda: check(library.ep_hip_encode_rans(
+        q.coset.data_ptr(), q.fields.data_ptr(), vectors, entries.data_ptr(), table_rel.data_ptr(), entries.numel(), 11, tile_vectors,
+        states.data_ptr(), tile_words.data_ptr(), scratch.data_ptr(), flag.data_ptr(), stream))), None)
+    check(library.ep_hip_encode_offsets(tile_words.data_ptr(), tiles, offsets.data_ptr(), total.data_ptr(), stream))
+    words = int(total.item())
+    kernels["rans"] = (kernels["rans"][0], 33 * vectors + 2 * words + 132 * tiles)
+    payload = torch.empty(words, dtype=torch.int16, device="cuda")
+    kernels["offsets"] = (timed(lambda: check(library.ep_hip_encode_offsets(
+        tile_words.data_ptr(), tiles, offsets.data_ptr(), total.data_ptr(), stream))), 8 * tiles)
+    kernels["gather"] = (timed(lambda: check(library.ep_hip_encode_gather(
+        scratch.data_ptr(), offsets.data_ptr(), tiles, tile_vectors, payload.data_ptr(), stream))), 4 * words)
+    assert int(flag.item()) == 0
+    by_kernel = {name: {"us": round(us, 1), "algorithmic_bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)} for name, (us, nbytes) in kernels.items()}
+    dominant = max(kernels, key=lambda name: kernels[name][0])
+    us, nbytes = kernels[dominant]
+    weights = rows * cols
+    result = {
+        "metric": "lattice_rans encode, weights per second (whole compress call on the device)", "value": round(weights / wall / 1e9, 3),
+        "unit": "Gweights/s", "n_gpus": 1, "steps": 3, "warmup": 1, "ms_per_step": round(wall * 1e3, 2), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32/f64 quantise, u32 rANS", "data": "synthetic",
+        "config": {"workload": f"compress {rows}x{cols} bf16 N(0,{sigma}) seed {seed} @ {bpp} bpp on the device (12 search iterations on a "
+                               "row subsample, full quantise, histograms, refit, rANS encode, gather)",
+                   "actual_bpp": round(actual_bpp, 4), "relative_error": round(error, 5), "lattice_scale": round(scale, 6), "kernels_sum_ms": round(sum(v[0] for v in kernels.values()) / 1e3, 3),
+                   "by_kernel": by_kernel, "sample_identical_to_cpu_lane": identical, "sample_scales_within_1e-5": scales_close,
+                   "cpu_lane_on_sample": {"rows": cpu_rows, "actual_bpp": round(cpu_bpp, 4), "relative_error": round(cpu_error, 5)}},
+        "parity": parity,
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(nbytes / us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 5), "traffic": None},
+        "cpu_baseline": {"value": round(cpu_rows * cols / cpu_seconds / 1e9, 4), "unit": "Gweights/s", "cores": eager._threads(), "kind": "port",
+                         "sample": f"first {cpu_rows} of {rows} rows through this package's CPU encoder (bit-identical to the reference's eager "
+                                   f"lane on its golden containers), {cpu_seconds:.2f} s"},
+    }
+    print(json.dumps(result))
+    return 0 if parity else 1
+
+
 def copy_probe(args, device):
     """One plain device copy of `--copy-probe-mib` MiB: the calibration of the FETCH_SIZE / WRITE_SIZE counters."""
     if args.copy_probe_mib:
@@ -839,7 +975,7 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "store_pattern"])
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "store_pattern", "encode"])
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
@@ -865,6 +1001,8 @@ def main():
         return gemm_workload(args, ep)
     if args.workload == "store_pattern":
         return store_pattern_workload(args, ep)
+    if args.workload == "encode":
+        return encode_workload(args, ep)
     rows, cols, sigma, seed, bpp, outliers = WORKLOADS[args.workload]
     started = time.perf_counter()
     weight = make_weight(rows, cols, sigma, seed, outliers)

@@ -81,9 +81,13 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
 #pragma unroll
   for (int k = 0; k < kFieldStreams; ++k) { lo[k] = INT_MAX; hi[k] = INT_MIN; }
   unsigned ones = 0;
+  // (picked, v) = (at / vectors_per_row, at % vectors_per_row), carried along instead of divided out for every vector
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t at = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; at < vectors; at += stride) {
-    const int64_t picked = at / vectors_per_row, v = at - picked * vectors_per_row;
+  const int64_t stride_rows = stride / vectors_per_row, stride_rest = stride - stride_rows * vectors_per_row;
+  const int64_t start = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  int64_t picked = start / vectors_per_row, v = start - picked * vectors_per_row;
+  for (int64_t at = start; at < vectors; at += stride, picked += stride_rows, v += stride_rest) {
+    if (v >= vectors_per_row) { v -= vectors_per_row; ++picked; }
     const int64_t row = row_index != nullptr ? row_index[picked] : picked;
     const f32x4* source = reinterpret_cast<const f32x4*>(x + row * cols + v * 8);
     const f32x4 first = source[0], second = source[1];
@@ -218,11 +222,13 @@ __global__ __launch_bounds__(256) void row_scales_kernel(const float* __restrict
 
 // One tile per 32-lane half of a wavefront, lane l carrying state l. A group of 32 vectors is one vector per lane; its
 // symbols go in last to first (field 7 ... field 0, then the coset bit), and the words the lanes push out in one step
-// are appended in lane order, as the sequential encoder appends them. entries[i] = freq | cdf << 16 of table position
-// i; table_rel[s] = first position of stream s - least value of stream s. A symbol outside the tables, or one of
-// frequency 0, raises *error and is coded with frequency 1 so that the launch still ends.
+// are appended in lane order, as the sequential encoder appends them. entries[i] = {freq | cdf << 16, min(floor(2^32 /
+// freq), 2^32 - 1)} of table position i; table_rel[s] = first position of stream s - least value of stream s. The
+// quotient state / freq is the high half of state * floor(2^32 / freq), which is the quotient or one less (the product
+// falls short of 2^32 state / freq by less than state <= 2^32), put right by one comparison of the remainder. A symbol
+// outside the tables, or one of frequency 0, raises *error and is coded with frequency 1 so that the launch still ends.
 __global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restrict__ coset, const int32_t* __restrict__ fields, int64_t vectors,
-                                                          int tile_vectors, int64_t tiles, const uint32_t* __restrict__ entries,
+                                                          int tile_vectors, int64_t tiles, const uint2* __restrict__ entries,
                                                           const int32_t* __restrict__ table_rel, int total_entries, int prob_bits,
                                                           uint32_t* __restrict__ states, uint32_t* __restrict__ tile_words,
                                                           uint16_t* __restrict__ scratch, int* __restrict__ error) {
@@ -253,14 +259,14 @@ __global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restri
     for (int step = 0; step < 9; ++step) {
       const int f = 7 - step;
       const int position = step < 8 ? rel[1 + 2 * f + c] + z[f] : rel[0] + c;
-      uint32_t entry = 1u;
+      uint2 entry = make_uint2(1u, 0xFFFFFFFFu);
       if (valid) {
         if (static_cast<unsigned>(position) < static_cast<unsigned>(total_entries)) entry = entries[position];
         else bad = true;
       }
-      uint32_t freq = entry & 0xFFFFu;
-      const uint32_t cdf = entry >> 16;
-      if (freq == 0) { bad = true; freq = 1; }
+      uint32_t freq = entry.x & 0xFFFFu;
+      const uint32_t cdf = entry.x >> 16;
+      if (freq == 0) { bad = true; freq = 1; entry.y = 0xFFFFFFFFu; }
       const bool push = valid && state >= (freq << renorm_shift);
       const uint32_t pushing = static_cast<uint32_t>(__ballot(push) >> (32 * half));
       if (push) {
@@ -269,8 +275,10 @@ __global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restri
       }
       cursor += __popc(pushing);
       if (valid) {
-        const uint32_t quotient = state / freq;
-        state = (quotient << prob_bits) + (state - quotient * freq) + cdf;
+        uint32_t quotient = __umulhi(state, entry.y);
+        uint32_t rest = state - quotient * freq;
+        if (rest >= freq) { rest -= freq; ++quotient; }
+        state = (quotient << prob_bits) + rest + cdf;
       }
     }
   }
@@ -380,19 +388,19 @@ extern "C" int ep_hip_encode_row_scales(const float* x_dev, const float* rms_dev
   return EP_HIP_OK;
 }
 
-extern "C" int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const uint32_t* entries_dev,
+extern "C" int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const uint64_t* entries_dev,
                                   const int32_t* table_rel_dev, int32_t total_entries, int prob_bits, int tile_vectors,
                                   uint32_t* states_dev, uint32_t* tile_words_dev, uint16_t* scratch_dev, int32_t* error_dev, void* stream) {
   if (coset_dev == nullptr || fields_dev == nullptr || entries_dev == nullptr || table_rel_dev == nullptr || states_dev == nullptr ||
       tile_words_dev == nullptr || scratch_dev == nullptr || error_dev == nullptr)
     return EP_HIP_EINVAL;
   if (vectors <= 0 || total_entries <= 0 || prob_bits < 1 || prob_bits > 15 || tile_vectors < ep::kStatesPerTile) return EP_HIP_EINVAL;
-  if (reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0) return EP_HIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(entries_dev) % 8 != 0) return EP_HIP_EINVAL;
   const int64_t tiles = (vectors + tile_vectors - 1) / tile_vectors;
   const int64_t blocks = (tiles + 7) / 8;                 // 4 wavefronts of two tiles each
   if (blocks > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
   hipLaunchKernelGGL(ep::rans_encode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), coset_dev,
-                     fields_dev, vectors, tile_vectors, tiles, entries_dev, table_rel_dev, total_entries, prob_bits, states_dev, tile_words_dev,
+                     fields_dev, vectors, tile_vectors, tiles, reinterpret_cast<const uint2*>(entries_dev), table_rel_dev, total_entries, prob_bits, states_dev, tile_words_dev,
                      scratch_dev, error_dev);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;

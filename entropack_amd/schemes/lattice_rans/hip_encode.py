@@ -112,6 +112,15 @@ class DeviceQuantizer:
         return scales
 
 
+def table_entries(freq_all: np.ndarray, cdf_all: np.ndarray) -> torch.Tensor:
+    """int64 per table position: frequency | cumulative frequency << 16 in the low half, the reciprocal the kernel divides
+    with, min(floor(2^32 / frequency), 2^32 - 1), in the high half."""
+    freq = freq_all.astype(np.uint64)
+    reciprocal = np.minimum((np.uint64(1) << np.uint64(32)) // np.maximum(freq, np.uint64(1)), np.uint64(0xFFFFFFFF))
+    packed = freq | (cdf_all.astype(np.uint64) << np.uint64(16)) | (reciprocal << np.uint64(32))
+    return torch.from_numpy(packed.view(np.int64))
+
+
 def encode_streams(q: DeviceQuantized, prob_bits: int, tile_elements: int):
     """Frequency tables (host, from the device histograms) and the tiled rANS encode (device). Returns payload
     uint16[words], states uint32[tiles, 32], offsets uint32[tiles + 1] on the device, and stream_meta / freq_tables as
@@ -120,7 +129,7 @@ def encode_streams(q: DeviceQuantized, prob_bits: int, tile_elements: int):
     lib = _hip.library()
     stats = q.stats()
     meta, freq_all, cdf_all = eager.stream_tables(stats, q.histograms(stats), prob_bits)
-    entries = torch.from_numpy((freq_all | (cdf_all << 16)).astype(np.uint32).view(np.int32)).to(device)
+    entries = table_entries(freq_all, cdf_all).to(device)
     relative = torch.from_numpy((meta[:, META_FREQ_OFFSET] - meta[:, META_SYM_MIN]).astype(np.int32)).to(device)
 
     tile_vectors = vector_tile_elements(tile_elements)

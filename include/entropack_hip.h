@@ -300,13 +300,14 @@ int ep_hip_encode_row_scales(const float* x_dev, const float* rms_dev, int64_t c
                              const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, void* stream);
 
 /* Tiled 32-way interleaved rANS encode of `vectors` vectors in tiles of `tile_vectors` (>= 32). entries_dev:
- * uint32[total_entries], frequency | cumulative frequency << 16 of every table position; table_rel_dev: int32[17], first
- * position of stream s - its least value. states_dev: uint32[tiles][32]; tile_words_dev: uint32[tiles], the number of
+ * uint64[total_entries], for every table position frequency | cumulative frequency << 16 in the low half and
+ * min(floor(2^32 / frequency), 2^32 - 1) in the high half; table_rel_dev: int32[17], first position of stream s - its
+ * least value. states_dev: uint32[tiles][32]; tile_words_dev: uint32[tiles], the number of
  * payload words of each tile, which the tile leaves at scratch_dev[tile * tile_vectors * 9 ..) (uint16[tiles *
  * tile_vectors * 9]). *error_dev (int32, cleared by the caller) becomes 1 when a symbol lies outside the tables or has
  * frequency 0; the outputs are then not a valid container. Replaces cuda.py:520-541 (e8_rans_encode_vector_kernel,
  * lattice_rans.cu:400). */
-int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const uint32_t* entries_dev,
+int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64_t vectors, const uint64_t* entries_dev,
                        const int32_t* table_rel_dev, int32_t total_entries, int prob_bits, int tile_vectors, uint32_t* states_dev,
                        uint32_t* tile_words_dev, uint16_t* scratch_dev, int32_t* error_dev, void* stream);
 

@@ -1,0 +1,63 @@
+"""Host-side logic of the device encoder (no GPU): the stream statistics read from the quantise kernel's summary, the
+table entries with their reciprocals, and the quantizer interface the scale search drives."""
+import numpy as np
+import pytest
+import torch
+
+from entropack_amd.schemes.lattice_rans import eager, hip_encode
+
+INT64_MAX, INT64_MIN = np.iinfo(np.int64).max, np.iinfo(np.int64).min
+
+
+def summary_of(q: eager.Quantized) -> np.ndarray:
+    """What ep_hip_encode_quantize leaves for these vectors, computed from the CPU encoder's own statistics."""
+    stats = q.stats()
+    out = np.empty(hip_encode.SUMMARY_WORDS, dtype=np.int64)
+    for k in range(16):
+        n, lo, hi = stats[1 + k]
+        out[2 * k], out[2 * k + 1] = (lo, hi) if n else (INT64_MAX, INT64_MIN)
+    out[32] = int(q.coset.sum())
+    return out
+
+
+@pytest.mark.parametrize("scale", [0.2, 3.0])
+def test_stats_from_the_kernel_summary_are_the_cpu_encoders(scale):
+    x = torch.randn(16, 64, generator=torch.Generator().manual_seed(1))
+    host = eager.HostQuantizer(x, eager.row_rms(x, x.dtype))
+    q = host.quantize(scale)
+    device_form = hip_encode.DeviceQuantized(torch.from_numpy(q.coset), torch.from_numpy(q.fields), summary_of(q))
+    assert np.array_equal(device_form.stats(), q.stats())
+
+
+def test_stats_of_one_coset_only():
+    zeros = eager.HostQuantizer(torch.zeros(2, 16), torch.ones(2, 1)).quantize(1.0)
+    stats = hip_encode.DeviceQuantized(torch.from_numpy(zeros.coset), torch.from_numpy(zeros.fields), summary_of(zeros)).stats()
+    assert np.array_equal(stats, zeros.stats()) and stats[0].tolist() == [4, 0, 0]
+    halves = eager.HostQuantizer(torch.full((2, 16), 0.5), torch.ones(2, 1)).quantize(1.0)
+    stats = hip_encode.DeviceQuantized(torch.from_numpy(halves.coset), torch.from_numpy(halves.fields), summary_of(halves)).stats()
+    assert np.array_equal(stats, halves.stats()) and stats[0].tolist() == [4, 0, 1] and int(stats[1, 0]) == 0
+
+
+def test_table_entries_divide_exactly():
+    """state / freq from the packed reciprocal, as the kernel forms it: the high half of the product, put right once."""
+    freq = np.array([1, 2, 3, 5, 7, 100, 1023, 2047, 2048, 32767, 32768], dtype=np.int64)
+    cdf = np.arange(freq.size, dtype=np.int64) * 3
+    packed = hip_encode.table_entries(freq, cdf).numpy().view(np.uint64)
+    assert np.array_equal(packed & np.uint64(0xFFFF), freq.astype(np.uint64))
+    assert np.array_equal((packed >> np.uint64(16)) & np.uint64(0xFFFF), cdf.astype(np.uint64))
+    reciprocal = packed >> np.uint64(32)
+    rng = np.random.default_rng(0)
+    states = np.concatenate([rng.integers(1, 1 << 31, 20000), [1, 2, (1 << 31) - 1, 1 << 15, (1 << 16) - 1]]).astype(np.uint64)
+    for f, r in zip(freq.astype(np.uint64), reciprocal):
+        quotient = (states * r) >> np.uint64(32)
+        rest = states - quotient * f
+        assert np.all(rest < 2 * f)
+        quotient = np.where(rest >= f, quotient + np.uint64(1), quotient)
+        assert np.array_equal(quotient, states // f)
+
+
+def test_device_quantizer_refuses_host_tensors():
+    with pytest.raises(ValueError, match="on the GPU"):
+        hip_encode.DeviceQuantizer(torch.zeros(2, 8), torch.ones(2, 1))
+    with pytest.raises(ValueError, match="on the GPU"):
+        hip_encode.encode(weight=torch.zeros(2, 8), target_bpp=4.0, prob_bits=None, tile_elements=16384)
