@@ -30,7 +30,9 @@ from ..schemes import EntroPackLossyConfig, RawConfig
 from . import convrot
 
 QUANT_STATE_LEAF = "entropack_quant_state"      # state_dict key suffix of a compressed weight (the reference's, linear.py:190-230)
-ENCODE_BACKEND = "eager"
+#: Lane that compresses a weight: the device lane for a weight that is on the GPU (the reference's layers use their
+#: device lane for both directions, linear.py:15,59-68), the CPU lane for a weight on the CPU.
+ENCODE_BACKEND_BY_DEVICE = {"cuda": "hip", "cpu": "eager"}
 DECODE_BACKEND = "hip"
 FORWARD_MODES = ("decode_then_gemm", "fused")
 _F32_EPS = torch.finfo(torch.float32).eps
@@ -80,9 +82,8 @@ class CompressedLinear(torch.nn.Linear):
             return self.weight.scheme.make_config({"execution_backend": backend})
         return default_config(self.container_dtype, execution_backend=backend)
 
-    @property
-    def _encode_config(self):
-        return self._config_on(ENCODE_BACKEND)
+    def _encode_config_for(self, tensor: torch.Tensor):
+        return self._config_on(ENCODE_BACKEND_BY_DEVICE.get(tensor.device.type, "eager"))
 
     @property
     def _decode_config(self):
@@ -122,7 +123,7 @@ class CompressedLinear(torch.nn.Linear):
             raise ValueError(f"weight has shape {tuple(shape)}, but the layer expects {wanted}")
 
     def _compress_tensor(self, tensor: torch.Tensor) -> CompressedTensor:
-        packed = compress(tensor.to(self.container_dtype), self._encode_config)
+        packed = compress(tensor.to(self.container_dtype), self._encode_config_for(tensor))
         if packed.compress_method == "raw" and "reason" in packed.header:
             raise RuntimeError(
                 f"{packed.header['requested']} cannot store a {tuple(tensor.shape)} {self.container_dtype} weight for "

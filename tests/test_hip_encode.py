@@ -208,3 +208,23 @@ def test_hip_lane_takes_a_cpu_tensor_to_the_device_and_back():
     with pytest.raises(NotImplementedError):
         hip_encode.encode(weight=torch.zeros(4, 16, device="cuda"), target_bpp=4.0, prob_bits=None, tile_elements=16384,
                           row_rdo_iterations=2)
+
+
+def test_layers_compress_device_weights_on_the_device(monkeypatch):
+    """`CompressedLinear.from_linear` of a layer on the GPU never visits the CPU lane, and its forward is the dense
+    product with the weight the container decodes to."""
+    def refuse(**kwargs):
+        raise AssertionError("the CPU lane was asked to encode a device tensor")
+    monkeypatch.setattr(eager, "encode", refuse)
+    torch.manual_seed(5)
+    dense = torch.nn.Linear(512, 256, dtype=torch.bfloat16, device="cuda")
+    layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0))
+    assert layer.weight.buffers["payload"].device.type == "cuda"
+    x = torch.randn(32, 512, dtype=torch.bfloat16, device="cuda")
+    restored = ep.decompress(layer.weight, ep.EntroPackLossyConfig(execution_backend="hip"))
+    assert torch.equal(layer(x), torch.nn.functional.linear(x, restored, dense.bias))
+    original = dense.weight.detach().float()
+    relative = float((restored.float() - original).norm() / original.norm())
+    assert relative < 0.1
+    codes_layer = ep.CompressedINT8Linear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0))
+    assert codes_layer.weight.buffers["payload"].device.type == "cuda"
