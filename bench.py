@@ -826,7 +826,7 @@ def encode_workload(args, ep):
     kernels["offsets"] = (timed(lambda: check(library.ep_hip_encode_offsets(
         tile_words.data_ptr(), tiles, offsets.data_ptr(), total.data_ptr(), stream))), 8 * tiles)
     kernels["gather"] = (timed(lambda: check(library.ep_hip_encode_gather(
-        scratch.data_ptr(), offsets.data_ptr(), tiles, tile_vectors, payload.data_ptr(), stream))), 4 * words)
+        scratch.data_ptr(), offsets.data_ptr(), tiles, tile_vectors * 9, payload.data_ptr(), stream))), 4 * words)
     assert int(flag.item()) == 0
     by_kernel = {name: {"us": round(us, 1), "algorithmic_bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)} for name, (us, nbytes) in kernels.items()}
     dominant = max(kernels, key=lambda name: kernels[name][0])

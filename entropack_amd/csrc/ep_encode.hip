@@ -1,4 +1,4 @@
-// The lattice_rans encoder on the device: nearest-E8 quantisation, stream statistics, row-scale refit and the tiled
+// The encoders on the device. First the lattice_rans encoder: nearest-E8 quantisation, stream statistics, row-scale refit and the tiled
 // 32-way interleaved rANS encode. Every kernel produces, from the same inputs, exactly what the CPU encoder
 // (csrc/host_codec.c) produces: the float work is single IEEE operations in the same order (this file is compiled
 // without contraction), the rest is integer work. The one exception is the row-scale refit, whose float32 row sums are
@@ -9,6 +9,10 @@
 // e8_compact_kernel :467, launched from cuda.py:115-221 and :520-558. The algorithms followed are the eager lane's
 // (eager.py:18-58, rans.py:133-186), with which the reference states its kernels agree bit for bit
 // (lattice_rans.cu:3-18).
+//
+// Then the lossless tile_ans encoder (byte histogram, one rANS or raw stream per byte lane and tile), all integer work
+// and bit-identical to hc_tile_ans_encode; counterparts tile_ans.cu:27 (histogram), :67 (encode), :157 (compact),
+// launched from entropack/schemes/tile_ans/cuda.py:31-119. Both encoders share the cumulative sum and the gather.
 #include <hip/hip_runtime.h>
 #include <limits.h>
 
@@ -313,15 +317,103 @@ __global__ __launch_bounds__(1024) void offsets_kernel(const uint32_t* __restric
   if (t == 1023) *total = sums[1023];
 }
 
-// payload[offsets[t] ..) = the words tile t left at the start of its part of the scratch.
+// payload[offsets[t] ..) = the words stream t left at the start of its `stride` words of the scratch.
 __global__ __launch_bounds__(256) void gather_kernel(const uint16_t* __restrict__ scratch, const uint32_t* __restrict__ offsets, int64_t tiles,
-                                                     int tile_vectors, uint16_t* __restrict__ payload) {
-  const int64_t stride = static_cast<int64_t>(tile_vectors) * 9;
+                                                     int64_t stride, uint16_t* __restrict__ payload) {
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     const uint32_t from = offsets[tile], words = offsets[tile + 1] - from;
     const uint16_t* source = scratch + tile * stride;
     for (uint32_t i = threadIdx.x; i < words && i < stride; i += blockDim.x) payload[static_cast<uint64_t>(from) + i] = source[i];
   }
+}
+
+// ---- tile_ans ----------------------------------------------------------------------------------------------------------
+
+// counts[b][s] = number of elements whose byte b is s. Every thread takes 16 consecutive bytes at a time (the tensor's
+// storage is 16-byte aligned and its byte count a multiple of the element size, so a byte's lane is its index modulo
+// num_lanes); LDS bins, flushed with 64-bit atomics.
+__global__ __launch_bounds__(256) void byte_histogram_kernel(const uint8_t* __restrict__ bytes, int64_t total_bytes, int num_lanes,
+                                                             unsigned long long* __restrict__ counts) {
+  __shared__ unsigned bins[8 * 256];
+  for (int b = threadIdx.x; b < num_lanes * 256; b += blockDim.x) bins[b] = 0;
+  __syncthreads();
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * 16;
+  const int lane_mask = num_lanes - 1;                   // 1, 2, 4 or 8 byte lanes
+  for (int64_t at = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 16; at < total_bytes; at += stride) {
+    if (at + 16 <= total_bytes) {
+      const uint4 chunk = *reinterpret_cast<const uint4*>(bytes + at);
+      const uint32_t words[4] = {chunk.x, chunk.y, chunk.z, chunk.w};
+#pragma unroll
+      for (int j = 0; j < 16; ++j) atomicAdd(&bins[(j & lane_mask) * 256 + ((words[j >> 2] >> (8 * (j & 3))) & 0xFFu)], 1u);
+    } else {
+      for (int64_t i = at; i < total_bytes; ++i) atomicAdd(&bins[(static_cast<int>(i) & lane_mask) * 256 + bytes[i]], 1u);
+    }
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < num_lanes * 256; b += blockDim.x)
+    if (bins[b] != 0) atomicAdd(&counts[b], static_cast<unsigned long long>(bins[b]));
+}
+
+// One stream (byte lane b, tile t; stream index b * tiles + t) per 32-lane half. A raw lane stores its bytes two per
+// word, the even element in the low byte. A coded lane runs 32 interleaved states over its symbols in order, lane l
+// taking symbols l, l + 32, ...; the words a group of 32 symbols pushes out are appended in lane order. entries[b][s] =
+// {freq | cdf << 16, min(floor(2^32 / freq), 2^32 - 1)}. states: [coded lanes before b * tiles + t][32]. A symbol of
+// frequency 0 raises *error and is coded with frequency 1.
+__global__ __launch_bounds__(256) void tile_ans_encode_kernel(const uint8_t* __restrict__ bytes, int64_t num_elements, int num_lanes,
+                                                              int64_t tile_elements, int64_t tiles, int prob_bits, unsigned raw_mask,
+                                                              const uint2* __restrict__ entries, uint32_t* __restrict__ states,
+                                                              uint32_t* __restrict__ stream_words, uint16_t* __restrict__ scratch,
+                                                              int64_t scratch_stride, int* __restrict__ error) {
+  const int lane = threadIdx.x & 63, half = lane >> 5, l = lane & 31;
+  const int64_t stream = (static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2 + half;
+  if (stream >= tiles * num_lanes) return;
+  const int byte_lane = static_cast<int>(stream / tiles);
+  const int64_t tile = stream - byte_lane * tiles;
+  const int64_t begin = tile * tile_elements;
+  const int64_t end = begin + tile_elements < num_elements ? begin + tile_elements : num_elements;
+  uint16_t* out = scratch + stream * scratch_stride;
+  const uint8_t* column = bytes + byte_lane;
+  if ((raw_mask >> byte_lane) & 1u) {
+    const int64_t words = (end - begin + 1) / 2;
+    for (int64_t w = l; w < words; w += 32) {
+      const int64_t e = begin + 2 * w;
+      uint32_t word = column[e * num_lanes];
+      if (e + 1 < end) word |= static_cast<uint32_t>(column[(e + 1) * num_lanes]) << 8;
+      out[w] = static_cast<uint16_t>(word);
+    }
+    if (l == 0) stream_words[stream] = static_cast<uint32_t>(words);
+    return;
+  }
+  const uint2* table = entries + byte_lane * 256;
+  const uint32_t below = (1u << l) - 1u;
+  const int renorm_shift = 31 - prob_bits;
+  uint32_t state = kStateMin, cursor = 0;
+  bool bad = false;
+  for (int64_t base = begin; base < end; base += kStatesPerTile) {
+    const bool valid = base + l < end;
+    uint2 entry = make_uint2(1u, 0xFFFFFFFFu);
+    if (valid) entry = table[column[(base + l) * num_lanes]];
+    uint32_t freq = entry.x & 0xFFFFu;
+    const uint32_t cdf = entry.x >> 16;
+    if (freq == 0) { bad = true; freq = 1; entry.y = 0xFFFFFFFFu; }
+    const bool push = valid && state >= (freq << renorm_shift);
+    const uint32_t pushing = static_cast<uint32_t>(__ballot(push) >> (32 * half));
+    if (push) {
+      out[cursor + __popc(pushing & below)] = static_cast<uint16_t>(state & 0xFFFFu);
+      state >>= 16;
+    }
+    cursor += __popc(pushing);
+    if (valid) {
+      uint32_t quotient = __umulhi(state, entry.y);
+      uint32_t rest = state - quotient * freq;
+      if (rest >= freq) { rest -= freq; ++quotient; }
+      state = (quotient << prob_bits) + rest + cdf;
+    }
+  }
+  const int coded_before = __popc(~raw_mask & ((1u << byte_lane) - 1u));
+  states[(coded_before * tiles + tile) * kStatesPerTile + l] = state;
+  if (l == 0) stream_words[stream] = cursor;
+  if (bad) *error = 1;
 }
 
 static int grid_for(int64_t items, int per_block, int* blocks) {
@@ -416,15 +508,54 @@ extern "C" int ep_hip_encode_offsets(const uint32_t* tile_words_dev, int64_t til
   return EP_HIP_OK;
 }
 
-extern "C" int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int tile_vectors,
+extern "C" int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int64_t stride_words,
                                     uint16_t* payload_dev, void* stream) {
-  if (scratch_dev == nullptr || offsets_dev == nullptr || payload_dev == nullptr || tiles <= 0 || tile_vectors < ep::kStatesPerTile)
-    return EP_HIP_EINVAL;
+  if (scratch_dev == nullptr || offsets_dev == nullptr || payload_dev == nullptr || tiles <= 0 || stride_words <= 0) return EP_HIP_EINVAL;
   int blocks = 0;
   const int status = ep::grid_for(tiles, 1, &blocks);
   if (status != EP_HIP_OK) return status;
   hipLaunchKernelGGL(ep::gather_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), scratch_dev, offsets_dev, tiles,
-                     tile_vectors, payload_dev);
+                     stride_words, payload_dev);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_tile_ans_histogram(const uint8_t* bytes_dev, int64_t num_elements, int num_lanes, uint64_t* counts_dev, void* stream) {
+  if (bytes_dev == nullptr || counts_dev == nullptr || num_elements <= 0) return EP_HIP_EINVAL;
+  if (num_lanes != 1 && num_lanes != 2 && num_lanes != 4 && num_lanes != 8) return EP_HIP_EUNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(bytes_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(counts_dev) % 8 != 0) return EP_HIP_EINVAL;
+  const int64_t total_bytes = num_elements * num_lanes;
+  int blocks = 0;
+  const int status = ep::grid_for(total_bytes, 256 * 16 * 8, &blocks);
+  if (status != EP_HIP_OK) return status;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(ep::zero_words_kernel, dim3(num_lanes), dim3(256), 0, s, reinterpret_cast<unsigned long long*>(counts_dev),
+                     static_cast<int64_t>(num_lanes) * 256);
+  hipLaunchKernelGGL(ep::byte_histogram_kernel, dim3(blocks), dim3(256), 0, s, bytes_dev, total_bytes, num_lanes,
+                     reinterpret_cast<unsigned long long*>(counts_dev));
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+extern "C" int ep_hip_tile_ans_encode(const uint8_t* bytes_dev, int64_t num_elements, int num_lanes, int64_t tile_elements, int prob_bits,
+                                      const uint64_t* entries_dev, const uint8_t* lane_raw_host, uint32_t* states_dev,
+                                      uint32_t* stream_words_dev, uint16_t* scratch_dev, int64_t scratch_stride_words, int32_t* error_dev,
+                                      void* stream) {
+  if (bytes_dev == nullptr || entries_dev == nullptr || lane_raw_host == nullptr || stream_words_dev == nullptr || scratch_dev == nullptr ||
+      error_dev == nullptr)
+    return EP_HIP_EINVAL;
+  if (num_elements <= 0 || tile_elements <= 0 || prob_bits < 1 || prob_bits > 15 || scratch_stride_words < tile_elements) return EP_HIP_EINVAL;
+  if (num_lanes != 1 && num_lanes != 2 && num_lanes != 4 && num_lanes != 8) return EP_HIP_EUNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(entries_dev) % 8 != 0) return EP_HIP_EINVAL;
+  unsigned raw_mask = 0;
+  for (int b = 0; b < num_lanes; ++b) raw_mask |= (lane_raw_host[b] != 0 ? 1u : 0u) << b;
+  if (raw_mask != (1u << num_lanes) - 1u && states_dev == nullptr) return EP_HIP_EINVAL;
+  const int64_t tiles = (num_elements + tile_elements - 1) / tile_elements;
+  const int64_t blocks = (tiles * num_lanes + 7) / 8;
+  if (blocks > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
+  hipLaunchKernelGGL(ep::tile_ans_encode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), bytes_dev,
+                     num_elements, num_lanes, tile_elements, tiles, prob_bits, raw_mask, reinterpret_cast<const uint2*>(entries_dev), states_dev,
+                     stream_words_dev, scratch_dev, scratch_stride_words, error_dev);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }

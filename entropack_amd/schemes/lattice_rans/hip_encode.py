@@ -153,7 +153,7 @@ def encode_streams(q: DeviceQuantized, prob_bits: int, tile_elements: int):
     payload = torch.empty(words, dtype=torch.int16, device=device)
     if words:
         _hip.check("ep_hip_encode_gather", lib.ep_hip_encode_gather(
-            scratch.data_ptr(), offsets.data_ptr(), tiles, tile_vectors, payload.data_ptr(), _stream(device)))
+            scratch.data_ptr(), offsets.data_ptr(), tiles, tile_vectors * SYMBOLS_PER_VECTOR, payload.data_ptr(), _stream(device)))
     return payload.view(torch.uint16), states.view(torch.uint32), offsets.view(torch.uint32), meta, freq_all.astype(np.uint16)
 
 

@@ -2,7 +2,7 @@
 
 Public behaviour of the reference scheme (entropack/schemes/tile_ans/__init__.py:8-52): any tensor of a supported
 dtype, flattened; `tile_elements = 0` means 4096, or 8192 above 32 MiB of storage; buffers come back on the device the
-input was on. Lanes here: `hip` decodes on an MI355X, `eager` encodes on the CPU.
+input was on. Lanes here: `hip` decodes and encodes on an MI355X, `eager` encodes on the CPU.
 """
 import torch
 

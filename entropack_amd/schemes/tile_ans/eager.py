@@ -1,4 +1,5 @@
-"""CPU encoder of `tile_ans` (the `eager` lane). There is no CPU decoder in this package.
+"""CPU encoder of `tile_ans` (the `eager` lane; tensors on an MI355X are encoded there by the `hip` lane with this
+module's decisions). There is no CPU decoder in this package.
 
 Bit-identical to the reference's encoder (entropack/schemes/tile_ans/eager.py:17-228): same frequency normalisation
 (largest-remainder with the same tie order), same lane-mode and probability-precision choice, same stream layout.
@@ -134,6 +135,21 @@ def select_coding_options(counts_by_lane, raw_lane_threshold: float, tile_elemen
     return bits, freq, cdfs, tables, modes
 
 
+def coding_plan(counts: np.ndarray, probability_bits: int, raw_lane_threshold: float, tile_elements: int):
+    """(probability_bits, frequencies, cdfs, decode tables, lane modes) from the byte histograms int64[lanes, 256]: the
+    whole of the encoder's decisions; what remains is the coding of the streams (both lanes of this package share it)."""
+    if probability_bits == AUTO_PROB_BITS:
+        return select_coding_options(counts, raw_lane_threshold, tile_elements)
+    freq = np.stack([normalize_counts(c, 1 << probability_bits) for c in counts])
+    cdfs, tables = tables_from_frequencies(freq, probability_bits)
+    return probability_bits, freq, cdfs, tables, lane_modes_from_counts(counts, raw_lane_threshold, tile_elements)
+
+
+def as_unsigned_tensor(array: np.ndarray, kind) -> torch.Tensor:
+    """A numpy unsigned array as the torch tensor of the same unsigned dtype (through the signed view `kind`)."""
+    return torch.from_numpy(array.view(kind)).view({np.int16: torch.uint16, np.int32: torch.uint32}[kind])
+
+
 def encode(*, weight: torch.Tensor, tile_elements: int, probability_bits: int, raw_lane_threshold: float, **_ignored) -> TileBuffers:
     if weight.numel() == 0:
         raise ValueError("tile_ans does not support empty tensors")
@@ -143,12 +159,7 @@ def encode(*, weight: torch.Tensor, tile_elements: int, probability_bits: int, r
     raw = np.ascontiguousarray(contiguous.reshape(-1).view(torch.uint8).numpy())
     by_lane = raw.reshape(num_elements, num_lanes)
     counts = np.stack([np.bincount(by_lane[:, lane], minlength=256) for lane in range(num_lanes)])
-    if probability_bits == AUTO_PROB_BITS:
-        probability_bits, freq, cdfs, tables, modes = select_coding_options(counts, raw_lane_threshold, tile_elements)
-    else:
-        freq = np.stack([normalize_counts(c, 1 << probability_bits) for c in counts])
-        cdfs, tables = tables_from_frequencies(freq, probability_bits)
-        modes = lane_modes_from_counts(counts, raw_lane_threshold, tile_elements)
+    probability_bits, freq, cdfs, tables, modes = coding_plan(counts, probability_bits, raw_lane_threshold, tile_elements)
 
     tiles = num_tiles(num_elements, tile_elements)
     coded = int((modes == LANE_ANS).sum())
@@ -171,7 +182,7 @@ def encode(*, weight: torch.Tensor, tile_elements: int, probability_bits: int, r
         payload = np.ctypeslib.as_array(ctypes.cast(words, ctypes.POINTER(ctypes.c_uint16)), shape=(max(total, 1),))[:total].copy()
     finally:
         lib.hc_free(words)
-    as_torch = lambda array, kind: torch.from_numpy(array.view(kind)).view({np.int16: torch.uint16, np.int32: torch.uint32}[kind])
+    as_torch = as_unsigned_tensor
     return TileBuffers(
         payload=as_torch(payload, np.int16), offsets=as_torch(offsets, np.int32), states=as_torch(states, np.int32),
         decode_tables=as_torch(tables, np.int32), lane_modes=torch.from_numpy(np.ascontiguousarray(modes, dtype=np.uint8)),

@@ -316,10 +316,30 @@ int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64
  * by. Replaces the cumulative sum of cuda.py:542-551. */
 int ep_hip_encode_offsets(const uint32_t* tile_words_dev, int64_t tiles, uint32_t* offsets_dev, uint64_t* total_words_dev, void* stream);
 
-/* payload_dev[offsets_dev[t] ..) = the words of tile t from the scratch of ep_hip_encode_rans. Replaces cuda.py:552-557
- * (e8_compact_kernel, lattice_rans.cu:467). */
-int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int tile_vectors,
+/* payload_dev[offsets_dev[t] ..) = the words stream t left at scratch_dev[t * stride_words ..): stride_words =
+ * tile_vectors * 9 after ep_hip_encode_rans, the scratch stride after ep_hip_tile_ans_encode. Replaces cuda.py:552-557
+ * (e8_compact_kernel, lattice_rans.cu:467) and tile_ans/cuda.py:110-115 (tile_ans_compact_kernel, tile_ans.cu:157). */
+int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int64_t stride_words,
                          uint16_t* payload_dev, void* stream);
+
+/* The lossless tile_ans encoder. An element is num_lanes (1, 2, 4 or 8) bytes; byte b of elements [t * tile_elements, ..)
+ * is stream b * tiles + t. All integer work: the streams are bit-identical to the CPU encoder's
+ * (entropack/schemes/tile_ans/eager.py:145-228).
+ *
+ * ep_hip_tile_ans_histogram: counts_dev[b][s] (uint64[num_lanes][256], cleared by the call) = number of elements whose
+ * byte b is s; bytes_dev 16-byte aligned. Replaces tile_ans/cuda.py:31-47 (tile_ans_histogram_kernel, tile_ans.cu:27).
+ *
+ * ep_hip_tile_ans_encode: entries_dev uint64[num_lanes][256] = frequency | cumulative frequency << 16 in the low half,
+ * min(floor(2^32 / frequency), 2^32 - 1) in the high half (anything for symbols that do not occur); lane_raw_host
+ * (host memory, num_lanes bytes): non-zero = the lane is stored raw, two bytes per word. states_dev: uint32[coded lanes *
+ * tiles][32], coded lanes in lane order (may be NULL when every lane is raw); stream_words_dev: uint32[num_lanes * tiles];
+ * stream s leaves its words at scratch_dev[s * scratch_stride_words ..), scratch_stride_words >= tile_elements.
+ * *error_dev (cleared by the caller) becomes 1 when a coded symbol has frequency 0. Follow with ep_hip_encode_offsets and
+ * ep_hip_encode_gather. Replaces tile_ans/cuda.py:84-100 (tile_ans_encode_kernel, tile_ans.cu:67). */
+int ep_hip_tile_ans_histogram(const uint8_t* bytes_dev, int64_t num_elements, int num_lanes, uint64_t* counts_dev, void* stream);
+int ep_hip_tile_ans_encode(const uint8_t* bytes_dev, int64_t num_elements, int num_lanes, int64_t tile_elements, int prob_bits,
+                           const uint64_t* entries_dev, const uint8_t* lane_raw_host, uint32_t* states_dev, uint32_t* stream_words_dev,
+                           uint16_t* scratch_dev, int64_t scratch_stride_words, int32_t* error_dev, void* stream);
 
 /* Measurement aid --------------------------------------------------------------------------------------------- */
 
