@@ -1,6 +1,6 @@
 """Headline benchmark: lossy (lattice_rans) decode throughput on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|store_pattern|encode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|store_pattern|encode|tile_ans_encode]
 
 One "step" = one decode of the whole container (entropy decode + E8 reconstruction + BF16 store) from buffers
 already resident in HBM. Prints ONE JSON line. `value` = algorithmic bytes (container bytes read + dense bytes
@@ -852,6 +852,100 @@ def encode_workload(args, ep):
     return 0 if parity else 1
 
 
+def lossless_encode_workload(args, ep):
+    """`compress` of the 8192 x 28672 bf16 weight with the lossless tile_ans scheme on the device (default options: 8192
+    elements per tile, automatic precision; low byte raw, high byte coded): whole call, then kernel by kernel between
+    events. Parity: the first 2048 rows give the CPU lane's container byte for byte, and the full container decodes to
+    the input. CPU baseline: this package's CPU encoder on those rows (byte-identical to the reference's on its golden
+    containers), scaled by rows."""
+    from entropack_amd.backends import hip as hip_backend
+    from entropack_amd.schemes.lattice_rans.hip_encode import table_entries
+    from entropack_amd.schemes.tile_ans import eager as tile_eager
+    from entropack_amd.schemes.tile_ans.format import TileBuffers, num_tiles
+    rows, cols, sigma, seed = 8192, 28672, 0.015, 4
+    weight = make_weight(rows, cols, sigma, seed, False)
+    on_gpu = weight.cuda()
+    config = ep.TileANSConfig(execution_backend="hip")
+    ep.compress(on_gpu[:64], config)
+    torch.cuda.synchronize()
+    walls = []
+    for _ in range(3):
+        start = time.perf_counter()
+        container = ep.compress(on_gpu, config)
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - start)
+    wall = sorted(walls)[1]
+    lossless = bool(torch.equal(ep.decompress(container, ep.TileANSConfig()).view(torch.int16), on_gpu.view(torch.int16)))
+    stored = sum(t.numel() * t.element_size() for t in container.buffers.values())
+
+    cpu_rows = 2048
+    start = time.perf_counter()
+    on_cpu = ep.compress(weight[:cpu_rows], ep.TileANSConfig(execution_backend="eager"))
+    cpu_seconds = time.perf_counter() - start
+    sample = ep.compress(on_gpu[:cpu_rows], config)
+    identical = all(torch.equal(sample.buffers[key].cpu(), on_cpu.buffers[key]) for key in TileBuffers._fields)
+
+    library, stream = hip_backend.library(), torch.cuda.current_stream().cuda_stream
+    tile_elements, prob_bits, num_lanes, num_elements = (int(v) for v in container.buffers["layout"].tolist())
+    counts_device = torch.empty((num_lanes, 256), dtype=torch.int64, device="cuda")
+
+    def check(status):
+        if status:
+            raise hip_backend.HipError("ep_hip_tile_ans", status, "")
+
+    def timed(fn, count=20):
+        settle(fn, 0.1)
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record()
+        for _ in range(count):
+            fn()
+        last.record()
+        torch.cuda.synchronize()
+        return first.elapsed_time(last) / count * 1e3
+
+    nbytes = num_elements * num_lanes
+    kernels = {"histogram": (timed(lambda: check(library.ep_hip_tile_ans_histogram(on_gpu.data_ptr(), num_elements, num_lanes, counts_device.data_ptr(), stream))), nbytes)}
+    _, freq, cdfs, _, modes = tile_eager.coding_plan(counts_device.cpu().numpy(), prob_bits, 7.9, tile_elements)
+    tiles = num_tiles(num_elements, tile_elements)
+    streams, coded = tiles * num_lanes, int((modes == 0).sum())
+    entries = table_entries(freq.astype(np.int64).reshape(-1), cdfs.astype(np.int64).reshape(-1)).cuda()
+    raw_flags = np.ascontiguousarray(modes != 0, dtype=np.uint8)
+    states = torch.empty((tiles * coded, 32), dtype=torch.int32, device="cuda")
+    stream_words = torch.empty(streams, dtype=torch.int32, device="cuda")
+    scratch = torch.empty(streams * tile_elements, dtype=torch.int16, device="cuda")
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    offsets = torch.empty(streams + 1, dtype=torch.int32, device="cuda")
+    total = torch.empty(1, dtype=torch.int64, device="cuda")
+    words = container.buffers["payload"].numel()
+    payload = torch.empty(words, dtype=torch.int16, device="cuda")
+    kernels["encode"] = (timed(lambda: check(library.ep_hip_tile_ans_encode(
+        on_gpu.data_ptr(), num_elements, num_lanes, tile_elements, prob_bits, entries.data_ptr(), raw_flags.ctypes.data, states.data_ptr(),
+        stream_words.data_ptr(), scratch.data_ptr(), tile_elements, flag.data_ptr(), stream))), nbytes + 2 * words + 128 * tiles * coded)
+    kernels["offsets"] = (timed(lambda: check(library.ep_hip_encode_offsets(stream_words.data_ptr(), streams, offsets.data_ptr(), total.data_ptr(), stream))), 8 * streams)
+    kernels["gather"] = (timed(lambda: check(library.ep_hip_encode_gather(scratch.data_ptr(), offsets.data_ptr(), streams, tile_elements, payload.data_ptr(), stream))), 4 * words)
+    assert int(flag.item()) == 0 and int(total.item()) == words
+    by_kernel = {name: {"us": round(us, 1), "algorithmic_bytes": b, "GBps": round(b / us / 1e3, 1)} for name, (us, b) in kernels.items()}
+    dominant = max(kernels, key=lambda name: kernels[name][0])
+    us, b = kernels[dominant]
+    parity = lossless and identical
+    result = {
+        "metric": "tile_ans encode, input GB/s (whole compress call on the device)", "value": round(nbytes / wall / 1e9, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": 3, "warmup": 1, "ms_per_step": round(wall * 1e3, 2), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8 symbols, u32 rANS", "data": "synthetic",
+        "config": {"workload": f"lossless compress {rows}x{cols} bf16 N(0,{sigma}) seed {seed} on the device, default options "
+                               f"(tile_elements {tile_elements}, probability_bits {prob_bits}, lane modes {modes.tolist()})",
+                   "stored_over_input": round(stored / nbytes, 4), "kernels_sum_ms": round(sum(v[0] for v in kernels.values()) / 1e3, 3),
+                   "by_kernel": by_kernel, "sample_identical_to_cpu_lane": identical, "lossless": lossless},
+        "parity": parity,
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(b / us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 5), "traffic": None},
+        "cpu_baseline": {"value": round(cpu_rows * cols * 2 / cpu_seconds / 1e9, 4), "unit": "GB/s", "cores": tile_eager._threads(), "kind": "port",
+                         "sample": f"first {cpu_rows} of {rows} rows through this package's CPU encoder, {cpu_seconds:.2f} s"},
+    }
+    print(json.dumps(result))
+    return 0 if parity else 1
+
+
 def copy_probe(args, device):
     """One plain device copy of `--copy-probe-mib` MiB: the calibration of the FETCH_SIZE / WRITE_SIZE counters."""
     if args.copy_probe_mib:
@@ -975,7 +1069,7 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "store_pattern", "encode"])
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "store_pattern", "encode", "tile_ans_encode"])
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
@@ -1003,6 +1097,8 @@ def main():
         return store_pattern_workload(args, ep)
     if args.workload == "encode":
         return encode_workload(args, ep)
+    if args.workload == "tile_ans_encode":
+        return lossless_encode_workload(args, ep)
     rows, cols, sigma, seed, bpp, outliers = WORKLOADS[args.workload]
     started = time.perf_counter()
     weight = make_weight(rows, cols, sigma, seed, outliers)

@@ -321,9 +321,19 @@ __global__ __launch_bounds__(1024) void offsets_kernel(const uint32_t* __restric
 __global__ __launch_bounds__(256) void gather_kernel(const uint16_t* __restrict__ scratch, const uint32_t* __restrict__ offsets, int64_t tiles,
                                                      int64_t stride, uint16_t* __restrict__ payload) {
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const uint32_t from = offsets[tile], words = offsets[tile + 1] - from;
+    const uint32_t from = offsets[tile];
+    uint32_t words = offsets[tile + 1] - from;
+    if (words > stride) words = static_cast<uint32_t>(stride);
     const uint16_t* source = scratch + tile * stride;
-    for (uint32_t i = threadIdx.x; i < words && i < stride; i += blockDim.x) payload[static_cast<uint64_t>(from) + i] = source[i];
+    uint16_t* to = payload + from;
+    // one word to reach a 4-byte boundary of the destination, then two words per thread and store, then the last one
+    const uint32_t head = (from & 1u) < words ? (from & 1u) : words;
+    if (head != 0 && threadIdx.x == 0) to[0] = source[0];
+    const uint32_t pairs = (words - head) / 2;
+    uint32_t* to_pairs = reinterpret_cast<uint32_t*>(to + head);
+    for (uint32_t i = threadIdx.x; i < pairs; i += blockDim.x)
+      to_pairs[i] = static_cast<uint32_t>(source[head + 2 * i]) | static_cast<uint32_t>(source[head + 2 * i + 1]) << 16;
+    if (head + 2 * pairs < words && threadIdx.x == 0) to[words - 1] = source[words - 1];
   }
 }
 
@@ -331,12 +341,17 @@ __global__ __launch_bounds__(256) void gather_kernel(const uint16_t* __restrict_
 
 // counts[b][s] = number of elements whose byte b is s. Every thread takes 16 consecutive bytes at a time (the tensor's
 // storage is 16-byte aligned and its byte count a multiple of the element size, so a byte's lane is its index modulo
-// num_lanes); LDS bins, flushed with 64-bit atomics.
+// num_lanes). The bins are in LDS, in 2048 / (256 num_lanes) copies taken by the low bits of the thread index and one
+// word apart in their bank alignment: the bytes of a weight tensor crowd into a few values, and lanes of a wavefront
+// that add to one address (or to different addresses of one bank) take turns. Flushed with 64-bit atomics.
+constexpr int kByteBins = 2048;
 __global__ __launch_bounds__(256) void byte_histogram_kernel(const uint8_t* __restrict__ bytes, int64_t total_bytes, int num_lanes,
                                                              unsigned long long* __restrict__ counts) {
-  __shared__ unsigned bins[8 * 256];
-  for (int b = threadIdx.x; b < num_lanes * 256; b += blockDim.x) bins[b] = 0;
+  __shared__ unsigned bins[kByteBins + 8];
+  for (int b = threadIdx.x; b < kByteBins + 8; b += blockDim.x) bins[b] = 0;
   __syncthreads();
+  const int per_copy = num_lanes * 256, copies = kByteBins / per_copy;
+  unsigned* mine = bins + (threadIdx.x & (copies - 1)) * (per_copy + 1);
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * 16;
   const int lane_mask = num_lanes - 1;                   // 1, 2, 4 or 8 byte lanes
   for (int64_t at = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 16; at < total_bytes; at += stride) {
@@ -344,14 +359,17 @@ __global__ __launch_bounds__(256) void byte_histogram_kernel(const uint8_t* __re
       const uint4 chunk = *reinterpret_cast<const uint4*>(bytes + at);
       const uint32_t words[4] = {chunk.x, chunk.y, chunk.z, chunk.w};
 #pragma unroll
-      for (int j = 0; j < 16; ++j) atomicAdd(&bins[(j & lane_mask) * 256 + ((words[j >> 2] >> (8 * (j & 3))) & 0xFFu)], 1u);
+      for (int j = 0; j < 16; ++j) atomicAdd(&mine[(j & lane_mask) * 256 + ((words[j >> 2] >> (8 * (j & 3))) & 0xFFu)], 1u);
     } else {
-      for (int64_t i = at; i < total_bytes; ++i) atomicAdd(&bins[(static_cast<int>(i) & lane_mask) * 256 + bytes[i]], 1u);
+      for (int64_t i = at; i < total_bytes; ++i) atomicAdd(&mine[(static_cast<int>(i) & lane_mask) * 256 + bytes[i]], 1u);
     }
   }
   __syncthreads();
-  for (int b = threadIdx.x; b < num_lanes * 256; b += blockDim.x)
-    if (bins[b] != 0) atomicAdd(&counts[b], static_cast<unsigned long long>(bins[b]));
+  for (int b = threadIdx.x; b < per_copy; b += blockDim.x) {
+    unsigned sum = 0;
+    for (int c = 0; c < copies; ++c) sum += bins[c * (per_copy + 1) + b];
+    if (sum != 0) atomicAdd(&counts[b], static_cast<unsigned long long>(sum));
+  }
 }
 
 // One stream (byte lane b, tile t; stream index b * tiles + t) per 32-lane half. A raw lane stores its bytes two per
@@ -375,11 +393,18 @@ __global__ __launch_bounds__(256) void tile_ans_encode_kernel(const uint8_t* __r
   const uint8_t* column = bytes + byte_lane;
   if ((raw_mask >> byte_lane) & 1u) {
     const int64_t words = (end - begin + 1) / 2;
-    for (int64_t w = l; w < words; w += 32) {
-      const int64_t e = begin + 2 * w;
-      uint32_t word = column[e * num_lanes];
-      if (e + 1 < end) word |= static_cast<uint32_t>(column[(e + 1) * num_lanes]) << 8;
-      out[w] = static_cast<uint16_t>(word);
+    constexpr int kWordsAhead = 8;                         // 16 byte loads in flight per lane, then 8 stores
+    for (int64_t first = l; first < words; first += 32 * kWordsAhead) {
+      uint32_t low[kWordsAhead], high[kWordsAhead];
+#pragma unroll
+      for (int u = 0; u < kWordsAhead; ++u) {
+        const int64_t e = begin + 2 * (first + 32 * u);
+        low[u] = e < end ? column[e * num_lanes] : 0u;
+        high[u] = e + 1 < end ? column[(e + 1) * num_lanes] : 0u;
+      }
+#pragma unroll
+      for (int u = 0; u < kWordsAhead; ++u)
+        if (first + 32 * u < words) out[first + 32 * u] = static_cast<uint16_t>(low[u] | high[u] << 8);
     }
     if (l == 0) stream_words[stream] = static_cast<uint32_t>(words);
     return;
@@ -389,25 +414,41 @@ __global__ __launch_bounds__(256) void tile_ans_encode_kernel(const uint8_t* __r
   const int renorm_shift = 31 - prob_bits;
   uint32_t state = kStateMin, cursor = 0;
   bool bad = false;
-  for (int64_t base = begin; base < end; base += kStatesPerTile) {
-    const bool valid = base + l < end;
-    uint2 entry = make_uint2(1u, 0xFFFFFFFFu);
-    if (valid) entry = table[column[(base + l) * num_lanes]];
-    uint32_t freq = entry.x & 0xFFFFu;
-    const uint32_t cdf = entry.x >> 16;
-    if (freq == 0) { bad = true; freq = 1; entry.y = 0xFFFFFFFFu; }
-    const bool push = valid && state >= (freq << renorm_shift);
-    const uint32_t pushing = static_cast<uint32_t>(__ballot(push) >> (32 * half));
-    if (push) {
-      out[cursor + __popc(pushing & below)] = static_cast<uint16_t>(state & 0xFFFFu);
-      state >>= 16;
+  // The symbols and table entries of kAhead groups are fetched before the first of them is coded: neither depends on
+  // the state, and a step that waited for its own two loads would last as long as two trips to memory.
+  constexpr int kAhead = 8;
+  for (int64_t base = begin; base < end; base += kAhead * kStatesPerTile) {
+    uint32_t symbol[kAhead];
+    uint2 entry[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int64_t at = base + u * kStatesPerTile + l;
+      symbol[u] = at < end ? column[at * num_lanes] : 0u;
     }
-    cursor += __popc(pushing);
-    if (valid) {
-      uint32_t quotient = __umulhi(state, entry.y);
-      uint32_t rest = state - quotient * freq;
-      if (rest >= freq) { rest -= freq; ++quotient; }
-      state = (quotient << prob_bits) + rest + cdf;
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) entry[u] = table[symbol[u]];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int64_t group = base + u * kStatesPerTile;
+      if (group >= end) break;
+      const bool valid = group + l < end;
+      uint32_t freq = entry[u].x & 0xFFFFu;
+      const uint32_t cdf = entry[u].x >> 16;
+      uint32_t reciprocal = entry[u].y;
+      if (freq == 0) { bad = bad || valid; freq = 1; reciprocal = 0xFFFFFFFFu; }
+      const bool push = valid && state >= (freq << renorm_shift);
+      const uint32_t pushing = static_cast<uint32_t>(__ballot(push) >> (32 * half));
+      if (push) {
+        out[cursor + __popc(pushing & below)] = static_cast<uint16_t>(state & 0xFFFFu);
+        state >>= 16;
+      }
+      cursor += __popc(pushing);
+      if (valid) {
+        uint32_t quotient = __umulhi(state, reciprocal);
+        uint32_t rest = state - quotient * freq;
+        if (rest >= freq) { rest -= freq; ++quotient; }
+        state = (quotient << prob_bits) + rest + cdf;
+      }
     }
   }
   const int coded_before = __popc(~raw_mask & ((1u << byte_lane) - 1u));
