@@ -814,7 +814,7 @@ def encode_workload(args, ep):
     kernels["histogram"] = (timed(lambda: check(library.ep_hip_encode_histogram(
         q.coset.data_ptr(), q.fields.data_ptr(), vectors, bin_rel.data_ptr(), bins.numel(), bins.data_ptr(), stream))), 33 * vectors)
     kernels["row_scales"] = (timed(lambda: check(library.ep_hip_encode_row_scales(
-        x.data_ptr(), quantizer.rms.data_ptr(), cols, scale, rows, q.coset.data_ptr(), q.fields.data_ptr(), scales.data_ptr(), stream))),
+        x.data_ptr(), quantizer.rms.data_ptr(), cols, scale, rows, q.coset.data_ptr(), q.fields.data_ptr(), scales.data_ptr(), 0, stream))),
         4 * rows * cols + 33 * vectors)
     kernels["rans"] = (timed(lambda: check(library.ep_hip_encode_rans(
         q.coset.data_ptr(), q.fields.data_ptr(), vectors, entries.data_ptr(), table_rel.data_ptr(), entries.numel(), 11, tile_vectors,

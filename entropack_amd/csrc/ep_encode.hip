@@ -183,14 +183,16 @@ __global__ void zero_words_kernel(unsigned long long* __restrict__ words, int64_
 }
 
 // Least-squares scale of a row against the lattice points chosen for it: sum(x p) / sum(p p) in float32, at least
-// 1e-12; scale * rms[row] for a row of zeros. One block per row; every thread adds its vectors (t, t + 256, ...) in
-// order, coordinate 0 to 7, and the 256 partial sums are added pairwise (t with t + 128, then + 64, ...).
+// 1e-12; scale * rms[row] for a row of zeros. row_sse (optional) = the squared error that scale leaves,
+// max(sum(x x) - sum(x p)^2 / sum(p p), 0), or sum(x x) for a row of zeros. One block per row; every thread adds its
+// vectors (t, t + 256, ...) in order, coordinate 0 to 7, and the 256 partial sums are added pairwise (t with t + 128,
+// then + 64, ...).
 __global__ __launch_bounds__(256) void row_scales_kernel(const float* __restrict__ x, const float* __restrict__ rms, int64_t cols, float scale,
                                                          const int8_t* __restrict__ coset, const int32_t* __restrict__ fields,
-                                                         float* __restrict__ scales) {
-  __shared__ float numerators[256], denominators[256];
+                                                         float* __restrict__ scales, float* __restrict__ row_sse) {
+  __shared__ float numerators[256], denominators[256], energies[256];
   const int64_t row = blockIdx.x, vectors_per_row = cols / 8;
-  float numerator = 0.0f, denominator = 0.0f;
+  float numerator = 0.0f, denominator = 0.0f, energy = 0.0f;
   for (int64_t v = threadIdx.x; v < vectors_per_row; v += 256) {
     const int64_t at = row * vectors_per_row + v;
     const f32x4* source = reinterpret_cast<const f32x4*>(x + row * cols + v * 8);
@@ -206,21 +208,28 @@ __global__ __launch_bounds__(256) void row_scales_kernel(const float* __restrict
       const float level = static_cast<float>(j < 7 ? z[j] : 2 * z[7] + parity) + half;
       numerator += raw[j] * level;
       denominator += level * level;
+      energy += raw[j] * raw[j];
     }
   }
   numerators[threadIdx.x] = numerator;
   denominators[threadIdx.x] = denominator;
+  energies[threadIdx.x] = energy;
   __syncthreads();
   for (int width = 128; width > 0; width >>= 1) {
     if (threadIdx.x < width) {
       numerators[threadIdx.x] += numerators[threadIdx.x + width];
       denominators[threadIdx.x] += denominators[threadIdx.x + width];
+      energies[threadIdx.x] += energies[threadIdx.x + width];
     }
     __syncthreads();
   }
   if (threadIdx.x == 0) {
     const float fitted = numerators[0] / denominators[0];
     scales[row] = denominators[0] > 0.0f ? (fitted > 1.0e-12f ? fitted : 1.0e-12f) : scale * rms[row];
+    if (row_sse != nullptr) {
+      const float left = energies[0] - numerators[0] * numerators[0] / denominators[0];
+      row_sse[row] = denominators[0] > 0.0f ? (left > 0.0f ? left : 0.0f) : energies[0];
+    }
   }
 }
 
@@ -510,13 +519,14 @@ extern "C" int ep_hip_encode_histogram(const int8_t* coset_dev, const int32_t* f
 }
 
 extern "C" int ep_hip_encode_row_scales(const float* x_dev, const float* rms_dev, int64_t cols, float scale, int64_t rows,
-                                        const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, void* stream) {
+                                        const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, float* row_sse_dev,
+                                        void* stream) {
   if (x_dev == nullptr || rms_dev == nullptr || coset_dev == nullptr || fields_dev == nullptr || scales_dev == nullptr) return EP_HIP_EINVAL;
   if (rows <= 0 || cols <= 0 || cols % 8 != 0) return EP_HIP_EINVAL;
   if (rows > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(fields_dev) % 16 != 0) return EP_HIP_EINVAL;
   hipLaunchKernelGGL(ep::row_scales_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream), x_dev, rms_dev,
-                     cols, scale, coset_dev, fields_dev, scales_dev);
+                     cols, scale, coset_dev, fields_dev, scales_dev, row_sse_dev);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }

@@ -7,7 +7,7 @@ against an analytic size model on a seeded row subsample, nearest-E8 quantisatio
 scales, Hamilton-normalised frequency tables and the tiled 32-way interleaved rANS encode. The per-vector and
 per-symbol loops run in libentropack_host.so (csrc/host_codec.c).
 
-Not restated: the optional per-row rate-distortion pass (`row_rdo_iterations > 0` raises).
+The optional per-row rate-distortion pass (`row_rdo_iterations > 0`) is rdo.py.
 
 `decode` is deliberately absent: containers are decoded by the `hip` lane. Asking this lane to decode raises.
 """
@@ -103,6 +103,10 @@ class Quantized:
         host_library().hc_levels(_address(self.coset), _address(self.fields), self.vectors, _address(out), _threads())
         return torch.from_numpy(out)
 
+    def planes(self):
+        """(coset int8 [V], fields int32 [V, 8]) as torch tensors over the same memory."""
+        return torch.from_numpy(self.coset), torch.from_numpy(self.fields)
+
 
 def quantize(x: np.ndarray, rms: np.ndarray, scale: float, rows_selected: np.ndarray | None = None) -> Quantized:
     rows, cols = x.shape
@@ -136,7 +140,15 @@ class HostQuantizer:
         return quantize(self._x, self._rms, scale, rows_selected)
 
     def refit(self, q: Quantized, scale: float) -> torch.Tensor:
+        return refit_row_scales(self.x_t, self.rms_t, q, scale)[0]
+
+    def refit_with_error(self, q: Quantized, scale: float):
+        """(row scales, squared error of every row at its fitted scale)."""
         return refit_row_scales(self.x_t, self.rms_t, q, scale)
+
+    def assemble(self, coset: torch.Tensor, fields: torch.Tensor) -> Quantized:
+        """Quantised vectors from integer tensors [V] and [V, 8] (rows picked from several quantisations)."""
+        return Quantized(np.ascontiguousarray(coset.numpy().astype(np.int8)), np.ascontiguousarray(fields.numpy().astype(np.int32)))
 
 
 # ---- frequency tables and the size model -------------------------------------------------------------------------
@@ -234,18 +246,25 @@ def bisect_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, ma
     return math.sqrt(low * high)
 
 
-def refit_row_scales(x_t: torch.Tensor, rms_t: torch.Tensor, q: Quantized, scale: float) -> torch.Tensor:
-    """Least-squares scale of each row against the points chosen for it (float32 row sums, as torch computes them)."""
+def refit_row_scales(x_t: torch.Tensor, rms_t: torch.Tensor, q: Quantized, scale: float):
+    """Least-squares scale of each row against the points chosen for it, and the squared error that scale leaves
+    (float32 row sums, as torch computes them; the reference's eager.py:209-225)."""
     rows, cols = x_t.shape
     levels = q.levels().reshape(rows, cols)
     numerator = (x_t * levels).sum(1)
     denominator = levels.square().sum(1)
-    return torch.where(denominator > 0, (numerator / denominator).clamp_min(MIN_RMS), scale * rms_t.squeeze(1))
+    scales = torch.where(denominator > 0, (numerator / denominator).clamp_min(MIN_RMS), scale * rms_t.squeeze(1))
+    energy = x_t.square().sum(1)
+    row_sse = torch.where(denominator > 0, (energy - numerator * numerator / denominator).clamp_min(0.0), energy)
+    return scales, row_sse
 
 
-def resolve_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, max_vectors):
+def resolve_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, max_vectors, rdo_iterations=0, rdo_candidates=5):
     """Scale search plus the alphabet guard: grow an automatic prob_bits (to 15 at most) while an alphabet overflows
-    the table, after that coarsen the scale by the overflow. Returns (quantised vectors, row scales, prob_bits)."""
+    the table, after that coarsen the scale by the overflow. With `rdo_iterations` > 0 the rows are then refined one by
+    one (rdo.py), which can widen an alphabet again, so the guard looks at what that pass returns. Returns (quantised
+    vectors, row scales, prob_bits)."""
+    from . import rdo
     prob_bits, automatic = resolve_prob_bits(prob_bits, target_bpp)
     if quantizer.all_zero():
         q = quantizer.quantize(1.0)
@@ -258,6 +277,14 @@ def resolve_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, m
         while True:
             q = quantizer.quantize(scale)
             widest = _largest_alphabet(q)
+            scales = None
+            if widest <= table_size and rdo_iterations > 0:
+                baseline = rdo.RowCandidate(q, *quantizer.refit_with_error(q, scale))
+                rows = quantizer.rows
+                q, scales = rdo.refine_rows(
+                    quantizer, baseline, scale, rdo_iterations, rdo_candidates,
+                    lambda stats, histograms: modelled_bytes(histograms, [int(n) for n in stats[:, 0]], rows, prob_bits, tile_elements))
+                widest = _largest_alphabet(q)
             if widest <= table_size:
                 break
             if automatic and prob_bits < 15:
@@ -271,7 +298,7 @@ def resolve_scale(quantizer, target_bpp, prob_bits, tile_elements, iterations, m
         if clamped:
             log.debug("lattice_rans coarsened the lattice scale to %.6g so a coordinate alphabet of %d fits the "
                       "%d-entry rANS table; actual_bpp for this tensor will fall below target_bpp", scale, widest, table_size)
-        return q, quantizer.refit(q, scale), prob_bits
+        return q, (quantizer.refit(q, scale) if scales is None else scales), prob_bits
 
 
 # ---- stream encode ---------------------------------------------------------------------------------------------
@@ -335,8 +362,6 @@ def _as_torch(array: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
 
 
 def check_encode_request(weight, row_rdo_iterations) -> None:
-    if int(row_rdo_iterations) > 0:
-        raise NotImplementedError("per-row rate-distortion refinement is not part of this build; use row_rdo_iterations=0")
     if weight.shape[1] % LATTICE_DIM:
         raise ValueError(
             f"lattice_rans quantizes whole E8 vectors, so the column count must be a multiple of {LATTICE_DIM}; got cols={weight.shape[1]}")
@@ -360,7 +385,7 @@ def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0
     rms_t = row_rms(x_t, weight.dtype)
     q, scales, prob_bits = resolve_scale(
         HostQuantizer(x_t, rms_t), float(target_bpp), None if prob_bits in (None, 0) else int(prob_bits), int(tile_elements),
-        int(scale_search_iterations), int(scale_search_max_vectors))
+        int(scale_search_iterations), int(scale_search_max_vectors), int(row_rdo_iterations), int(row_rdo_candidates))
     payload, states, offsets, meta, freq_tables = encode_streams(q, prob_bits, int(tile_elements))
     return LatticeBuffers(
         payload=_as_torch(payload, torch.uint16).to(device), offsets=_as_torch(offsets, torch.uint32).to(device),

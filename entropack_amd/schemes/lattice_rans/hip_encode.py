@@ -67,6 +67,10 @@ class DeviceQuantized:
             raise RuntimeError("lattice_rans device histogram lost symbols: the stream minima do not cover the fields")
         return [counts[starts[s]:starts[s + 1]] for s in range(NUM_STREAMS)]
 
+    def planes(self):
+        """(coset int8 [V], fields int32 [V, 8]) on the device."""
+        return self.coset, self.fields
+
 
 class DeviceQuantizer:
     """`eager.HostQuantizer`'s interface over a float32 matrix and its row RMS on the device."""
@@ -103,13 +107,44 @@ class DeviceQuantizer:
             coset.data_ptr(), fields.data_ptr(), summary.data_ptr(), _stream(device)))
         return DeviceQuantized(coset, fields, summary.cpu().numpy())
 
-    def refit(self, q: DeviceQuantized, scale: float) -> torch.Tensor:
+    def _refit(self, q: DeviceQuantized, scale: float, with_error: bool):
         device = self.x.device
         scales = torch.empty(self.rows, dtype=torch.float32, device=device)
+        row_sse = torch.empty(self.rows, dtype=torch.float32, device=device) if with_error else None
         _hip.check("ep_hip_encode_row_scales", _hip.library().ep_hip_encode_row_scales(
             self.x.data_ptr(), self.rms.data_ptr(), self.cols, float(scale), self.rows, q.coset.data_ptr(), q.fields.data_ptr(),
-            scales.data_ptr(), _stream(device)))
-        return scales
+            scales.data_ptr(), row_sse.data_ptr() if with_error else 0, _stream(device)))
+        return scales, row_sse
+
+    def refit(self, q: DeviceQuantized, scale: float) -> torch.Tensor:
+        return self._refit(q, scale, False)[0]
+
+    def refit_with_error(self, q: DeviceQuantized, scale: float):
+        """(row scales, squared error of every row at its fitted scale), float32 on the device."""
+        return self._refit(q, scale, True)
+
+    def assemble(self, coset: torch.Tensor, fields: torch.Tensor) -> DeviceQuantized:
+        return quantized_from_planes(coset, fields)
+
+
+def quantized_from_planes(coset: torch.Tensor, fields: torch.Tensor) -> DeviceQuantized:
+    """Quantised vectors from integer tensors [V] and [V, 8] (rows picked from several quantisations); the summary the
+    quantise kernel would have left is taken with torch reductions on the tensors' device."""
+    coset = coset.to(torch.int8).contiguous()
+    fields = fields.to(torch.int32).contiguous()
+    summary = np.empty(SUMMARY_WORDS, dtype=np.int64)
+    halves = coset.bool()
+    for bit, mask in ((0, ~halves), (1, halves)):
+        chosen = fields[mask]
+        if chosen.shape[0]:
+            low, high = chosen.amin(0).cpu().numpy(), chosen.amax(0).cpu().numpy()
+        else:
+            low = np.full(NUM_FIELDS, np.iinfo(np.int64).max, dtype=np.int64)
+            high = np.full(NUM_FIELDS, np.iinfo(np.int64).min, dtype=np.int64)
+        for field in range(NUM_FIELDS):
+            summary[2 * (2 * field + bit)], summary[2 * (2 * field + bit) + 1] = int(low[field]), int(high[field])
+    summary[2 * (NUM_STREAMS - 1)] = int(halves.sum())
+    return DeviceQuantized(coset, fields, summary)
 
 
 def table_entries(freq_all: np.ndarray, cdf_all: np.ndarray) -> torch.Tensor:
@@ -158,14 +193,14 @@ def encode_streams(q: DeviceQuantized, prob_bits: int, tile_elements: int):
 
 
 def encode_normalised(x: torch.Tensor, rms: torch.Tensor, *, target_bpp, prob_bits, tile_elements, scale_search_iterations=12,
-                      scale_search_max_vectors=262144) -> LatticeBuffers:
+                      scale_search_max_vectors=262144, row_rdo_iterations=0, row_rdo_candidates=5) -> LatticeBuffers:
     """The container of the float32 device matrix `x` whose rows are normalised by `rms` (float32 [rows, 1], on the device).
     With the CPU lane's row RMS this is the CPU lane's container except for the order of the refit's float32 sums."""
     device = x.device
     cols = x.shape[1]
     q, scales, prob_bits = eager.resolve_scale(
         DeviceQuantizer(x, rms), float(target_bpp), None if prob_bits in (None, 0) else int(prob_bits), int(tile_elements),
-        int(scale_search_iterations), int(scale_search_max_vectors))
+        int(scale_search_iterations), int(scale_search_max_vectors), int(row_rdo_iterations), int(row_rdo_candidates))
     payload, states, offsets, meta, freq_tables = encode_streams(q, prob_bits, int(tile_elements))
     return LatticeBuffers(
         payload=payload, offsets=offsets, states=states, stream_meta=torch.from_numpy(meta.astype(np.int32)).to(device),
@@ -191,4 +226,5 @@ def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0
         raise ValueError("the hip lane encodes tensors that are on the GPU; use execution_backend='eager' for CPU tensors")
     x = weight.detach().float().contiguous()
     return encode_normalised(x, row_rms(x, weight.dtype), target_bpp=target_bpp, prob_bits=prob_bits, tile_elements=tile_elements,
-                             scale_search_iterations=scale_search_iterations, scale_search_max_vectors=scale_search_max_vectors)
+                             scale_search_iterations=scale_search_iterations, scale_search_max_vectors=scale_search_max_vectors,
+                             row_rdo_iterations=row_rdo_iterations, row_rdo_candidates=row_rdo_candidates)

@@ -295,9 +295,12 @@ int ep_hip_encode_histogram(const int8_t* coset_dev, const int32_t* fields_dev, 
                             int32_t total_bins, uint64_t* bins_dev, void* stream);
 
 /* Least-squares row scales against the chosen points: scales_dev[r] = max(sum(x p) / sum(p p), 1e-12) in float32, or
- * scale * rms[r] for a row whose points are all zero. Replaces cuda.py:142-158 (the refit kernels, lattice_rans.cu:313). */
+ * scale * rms[r] for a row whose points are all zero; row_sse_dev (may be NULL) receives the squared error of every row
+ * at that scale, max(sum(x x) - sum(x p)^2 / sum(p p), 0), or sum(x x) for such a row. Replaces cuda.py:142-158 (the
+ * refit kernels, lattice_rans.cu:313). */
 int ep_hip_encode_row_scales(const float* x_dev, const float* rms_dev, int64_t cols, float scale, int64_t rows,
-                             const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, void* stream);
+                             const int8_t* coset_dev, const int32_t* fields_dev, float* scales_dev, float* row_sse_dev,
+                             void* stream);
 
 /* Tiled 32-way interleaved rANS encode of `vectors` vectors in tiles of `tile_vectors` (>= 32). entries_dev:
  * uint64[total_entries], for every table position frequency | cumulative frequency << 16 in the low half and

@@ -49,7 +49,7 @@ class Golden:
     def config_kwargs(self):
         out = {}
         for key, value in self.options.items():
-            out[key] = int(value) if key in ("tile_elements", "prob_bits") else value
+            out[key] = int(value) if key in ("tile_elements", "prob_bits", "row_rdo_iterations", "row_rdo_candidates") else value
         return out
 
 

@@ -11,7 +11,7 @@ fixture records, for one small tensor:
   * the symbol planes its entropy decoder returns (coset + 8 shifted fields),
   * the dense tensor ``decompress`` returns (raw bits), and ``actual_bpp``.
 
-Usage:  PYTHONDONTWRITEBYTECODE=1 python tests/golden/make_fixtures.py
+Usage:  PYTHONDONTWRITEBYTECODE=1 python tests/golden/make_fixtures.py [NAME_PREFIX]
 """
 import os
 import sys
@@ -65,6 +65,11 @@ def cases():
     yield "f16_48x128_5p0", gauss(17, 48, 128, 0.5, torch.float16), dict(target_bpp=5.0)
     yield "f32_40x72_6p0_pb13", gauss(18, 40, 72, 1.5, torch.float32), dict(target_bpp=6.0, prob_bits=13)
     yield "pb9_64x128_bf16_1p5", gauss(19, 64, 128, 0.02), dict(target_bpp=1.5, prob_bits=9)
+    # the optional per-row rate-distortion pass (row_rdo_iterations > 0)
+    yield "rdo2_96x256_bf16_3p0", gauss(30, 96, 256, 0.02), dict(target_bpp=3.0, row_rdo_iterations=2)
+    yield "rdo1_k3_64x512_bf16_4p0", outliers(31, 64, 512, 0.02, 0.002, 12.0), dict(target_bpp=4.0, row_rdo_iterations=1, row_rdo_candidates=3)
+    yield "rdo3_k7_40x72_f32_5p0", gauss(32, 40, 72, 1.5, torch.float32), dict(target_bpp=5.0, row_rdo_iterations=3, row_rdo_candidates=7)
+    yield "rdo2_rows_differ_128x128_bf16_2p5", (gauss(33, 128, 128, 0.02).float() * torch.logspace(-1, 1, 128).unsqueeze(1)).to(torch.bfloat16), dict(target_bpp=2.5, row_rdo_iterations=2)
 
 
 def main() -> None:
@@ -75,8 +80,13 @@ def main() -> None:
     from entropack.schemes.lattice_rans import rans as ref_rans
     from entropack.schemes.lattice_rans.format import LatticeBuffers, decode_geometry, vector_tile_elements
 
+    only = sys.argv[1] if len(sys.argv) > 1 else None        # a name prefix: write those fixtures only, keep the others
     names = []
     for name, weight, options in cases():
+        if only is not None and not name.startswith(only):
+            if os.path.exists(os.path.join(OUT_DIR, name + ".npz")):
+                names.append(name)
+            continue
         config = ep.EntroPackLossyConfig(execution_backend="eager", **options)
         compressed = ep.compress(weight, config)
         assert compressed.compress_method == "lattice_rans", compressed.header

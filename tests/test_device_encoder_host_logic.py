@@ -38,6 +38,17 @@ def test_stats_of_one_coset_only():
     assert np.array_equal(stats, halves.stats()) and stats[0].tolist() == [4, 0, 1] and int(stats[1, 0]) == 0
 
 
+def test_quantised_vectors_put_together_from_planes_carry_the_right_summary():
+    x = torch.randn(24, 64, generator=torch.Generator().manual_seed(2))
+    q = eager.HostQuantizer(x, eager.row_rms(x, x.dtype)).quantize(0.4)
+    coset, fields = q.planes()
+    rebuilt = hip_encode.quantized_from_planes(coset.to(torch.int32), fields.clone())
+    assert np.array_equal(rebuilt.stats(), q.stats())
+    assert rebuilt.coset.dtype == torch.int8 and rebuilt.fields.dtype == torch.int32
+    zeros = hip_encode.quantized_from_planes(torch.zeros(4, dtype=torch.int32), torch.zeros((4, 8), dtype=torch.int32))
+    assert zeros.stats()[0].tolist() == [4, 0, 0] and int(zeros.stats()[2, 0]) == 0
+
+
 def test_table_entries_divide_exactly():
     """state / freq from the packed reciprocal, as the kernel forms it: the high half of the product, put right once."""
     freq = np.array([1, 2, 3, 5, 7, 100, 1023, 2047, 2048, 32767, 32768], dtype=np.int64)

@@ -65,5 +65,25 @@ def test_encoder_rejects_what_the_reference_rejects():
     assert raw.compress_method == "raw" and raw.header["requested"] == "lattice_rans"
     with pytest.raises(TypeError):
         ep.compress(raw, ep.EntroPackLossyConfig())
-    with pytest.warns(ep.CompressionFallbackWarning):
-        ep.compress(torch.randn(8, 16), ep.EntroPackLossyConfig(execution_backend="eager", row_rdo_iterations=1))
+
+
+def test_row_refinement_lowers_the_error_at_the_same_size():
+    """What the per-row pass is for: against the plain encode of the same weight at the same target, rows whose energy
+    differs take different scales, the container does not grow and the squared error falls. (That the choice of every
+    row is the reference's is what the `rdo*` fixtures check, byte for byte.)"""
+    from entropack_amd.schemes.lattice_rans import rdo
+    assert rdo.scale_ratios(1) == (1.0,)
+    ladder = rdo.scale_ratios(5)
+    assert len(ladder) == 5 and 1.0 in ladder and list(ladder) == sorted(ladder) and 0.70 < ladder[0] and ladder[-1] < 1.45
+    assert set(rdo.scale_ratios(3)) <= set(ladder)
+    golden = Golden("rdo2_rows_differ_128x128_bf16_2p5")
+    weight = _weight(golden)
+    plain = eager.encode(weight=weight, target_bpp=2.5, prob_bits=None, tile_elements=16384)
+    refined = eager.encode(weight=weight, target_bpp=2.5, prob_bits=None, tile_elements=16384, row_rdo_iterations=2)
+    assert not np.array_equal(refined.payload.view(torch.int16).numpy(), plain.payload.view(torch.int16).numpy())
+    assert refined.payload.numel() <= plain.payload.numel() + 8
+    restored = torch.from_numpy(golden.restored_bits.copy()).view(torch.bfloat16).float()
+    quantizer = eager.HostQuantizer(weight.float().contiguous(), eager.row_rms(weight.float(), weight.dtype))
+    q, scales, _ = eager.resolve_scale(quantizer, 2.5, None, 16384, 12, 262144)
+    plain_dense = (q.levels().reshape(128, 128) * scales.unsqueeze(1)).to(torch.bfloat16).float()
+    assert float((restored - weight.float()).square().sum()) < float((plain_dense - weight.float()).square().sum())

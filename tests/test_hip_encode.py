@@ -11,6 +11,7 @@ import torch
 
 import entropack_amd as ep
 from entropack_amd.schemes.lattice_rans import eager, hip_encode
+from entropack_amd.schemes.lattice_rans import hip as hip_lane
 from entropack_amd.schemes.lattice_rans.format import LatticeBuffers, validate_packed
 from oracle import c_oracle
 
@@ -205,9 +206,42 @@ def test_hip_lane_takes_a_cpu_tensor_to_the_device_and_back():
         hip_encode.encode(weight=weight.float(), target_bpp=4.0, prob_bits=None, tile_elements=16384)
     with pytest.raises(ValueError, match="multiple of 8"):
         hip_encode.encode(weight=torch.zeros(4, 12, device="cuda"), target_bpp=4.0, prob_bits=None, tile_elements=16384)
-    with pytest.raises(NotImplementedError):
-        hip_encode.encode(weight=torch.zeros(4, 16, device="cuda"), target_bpp=4.0, prob_bits=None, tile_elements=16384,
-                          row_rdo_iterations=2)
+
+
+def test_row_refinement_on_the_device():
+    """`row_rdo_iterations` on the device lane: the same pass over the device's kernels. Its float32 row sums (prices,
+    squared errors) are added in another order than the CPU lane's, so a row on the fence may choose differently: the
+    container is valid, decodes as the oracle decodes it, and has the CPU lane's rate and error to 1 %; and it beats
+    the plain encode's error at no more bytes, which is what the pass is for."""
+    weight = (matrix(33, 128, 256) * torch.logspace(-1, 1, 128).unsqueeze(1)).to(torch.bfloat16)
+    options = dict(target_bpp=3.0, prob_bits=None, tile_elements=16384)
+    x = weight.float().contiguous()
+    rms = eager.row_rms(x, weight.dtype)
+    host, device = both_quantizers(x, rms)
+    q_host, q_device = host.quantize(0.3), device.quantize(0.3)
+    scales_host, sse_host = host.refit_with_error(q_host, 0.3)
+    scales_device, sse_device = device.refit_with_error(q_device, 0.3)
+    assert torch.allclose(scales_device.cpu(), scales_host, rtol=1e-5, atol=0.0)
+    assert torch.allclose(sse_device.cpu(), sse_host, rtol=1e-3, atol=0.0)        # a difference of two nearly equal sums
+
+    def error_of(buffers):
+        dense = hip_lane.decode(buffers, shape=(128, 256), dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        hip_lane.check_errors(buffers)
+        expect = c_oracle.decode(host_arrays(buffers), (128, 256), "bfloat16", threads=4)
+        assert np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), expect)
+        return float((dense.float().cpu() - x).square().sum())
+
+    def size_of(buffers):
+        return sum(t.numel() * t.element_size() for t in buffers)
+
+    plain = hip_encode.encode_normalised(x.cuda(), rms.cuda(), **options)
+    refined = hip_encode.encode_normalised(x.cuda(), rms.cuda(), row_rdo_iterations=2, **options)
+    on_cpu = LatticeBuffers(*(t.cuda() for t in eager.encode(weight=weight, row_rdo_iterations=2, **options)))
+    validate_packed(dict(zip(LatticeBuffers._fields, refined)), (128, 256), torch.bfloat16)
+    assert error_of(refined) < error_of(plain) and size_of(refined) <= size_of(plain) + 16
+    assert abs(size_of(refined) - size_of(on_cpu)) <= 0.01 * size_of(on_cpu)
+    assert abs(error_of(refined) - error_of(on_cpu)) <= 0.01 * error_of(on_cpu)
 
 
 def test_layers_compress_device_weights_on_the_device(monkeypatch):

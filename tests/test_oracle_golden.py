@@ -152,4 +152,4 @@ def test_truncated_and_unread_payloads_raise():
 
 
 def test_golden_set_is_complete():
-    assert len(golden_names()) == 13
+    assert len(golden_names()) == 17
