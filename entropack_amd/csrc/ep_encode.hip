@@ -240,17 +240,28 @@ __global__ __launch_bounds__(256) void row_scales_kernel(const float* __restrict
 // quotient state / freq is the high half of state * floor(2^32 / freq), which is the quotient or one less (the product
 // falls short of 2^32 state / freq by less than state <= 2^32), put right by one comparison of the remainder. A symbol
 // outside the tables, or one of frequency 0, raises *error and is coded with frequency 1 so that the launch still ends.
+// STAGED: the block first copies the table entries into LDS (total_entries * 8 bytes of dynamic LDS) and the nine
+// lookups of a vector go there; all nine are made before the first symbol is coded, since none depends on the state.
+template <bool STAGED>
 __global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restrict__ coset, const int32_t* __restrict__ fields, int64_t vectors,
                                                           int tile_vectors, int64_t tiles, const uint2* __restrict__ entries,
                                                           const int32_t* __restrict__ table_rel, int total_entries, int prob_bits,
                                                           uint32_t* __restrict__ states, uint32_t* __restrict__ tile_words,
                                                           uint16_t* __restrict__ scratch, int* __restrict__ error) {
+  extern __shared__ uint2 staged_entries[];
   __shared__ int rel[kStreams];
   if (threadIdx.x < kStreams) rel[threadIdx.x] = table_rel[threadIdx.x];
+  if (STAGED)
+    for (int i = threadIdx.x; i < total_entries; i += blockDim.x) staged_entries[i] = entries[i];
   __syncthreads();
+  const uint2* table = STAGED ? staged_entries : entries;
   const int lane = threadIdx.x & 63, half = lane >> 5, l = lane & 31;
   const int64_t tile = (static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2 + half;
   if (tile >= tiles) return;
+  int rel_even[kFields], rel_odd[kFields];               // first table position - least value, of the field's two streams
+#pragma unroll
+  for (int f = 0; f < kFields; ++f) { rel_even[f] = rel[1 + 2 * f]; rel_odd[f] = rel[2 + 2 * f]; }
+  const int rel_coset = rel[0];
   const int64_t begin = tile * tile_vectors;
   const int64_t end = begin + tile_vectors < vectors ? begin + tile_vectors : vectors;
   uint16_t* out = scratch + tile * (static_cast<int64_t>(tile_vectors) * 9);
@@ -268,18 +279,21 @@ __global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restri
       const i32x4v a = from[0], b = from[1];
       z[0] = a.x; z[1] = a.y; z[2] = a.z; z[3] = a.w; z[4] = b.x; z[5] = b.y; z[6] = b.z; z[7] = b.w;
     }
+    uint2 looked_up[9];
 #pragma unroll
     for (int step = 0; step < 9; ++step) {
       const int f = 7 - step;
-      const int position = step < 8 ? rel[1 + 2 * f + c] + z[f] : rel[0] + c;
-      uint2 entry = make_uint2(1u, 0xFFFFFFFFu);
-      if (valid) {
-        if (static_cast<unsigned>(position) < static_cast<unsigned>(total_entries)) entry = entries[position];
-        else bad = true;
-      }
+      const int position = step < 8 ? (c ? rel_odd[f] : rel_even[f]) + z[f] : rel_coset + c;
+      const bool inside = static_cast<unsigned>(position) < static_cast<unsigned>(total_entries);
+      bad = bad || (valid && !inside);
+      looked_up[step] = table[inside ? position : 0];
+    }
+#pragma unroll
+    for (int step = 0; step < 9; ++step) {
+      uint2 entry = looked_up[step];
       uint32_t freq = entry.x & 0xFFFFu;
       const uint32_t cdf = entry.x >> 16;
-      if (freq == 0) { bad = true; freq = 1; entry.y = 0xFFFFFFFFu; }
+      if (freq == 0) { bad = bad || valid; freq = 1; entry.y = 0xFFFFFFFFu; }
       const bool push = valid && state >= (freq << renorm_shift);
       const uint32_t pushing = static_cast<uint32_t>(__ballot(push) >> (32 * half));
       if (push) {
@@ -585,9 +599,16 @@ extern "C" int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields
   const int64_t tiles = (vectors + tile_vectors - 1) / tile_vectors;
   const int64_t blocks = (tiles + 7) / 8;                 // 4 wavefronts of two tiles each
   if (blocks > 0x7FFFFFFF) return EP_HIP_EUNSUPPORTED;
-  hipLaunchKernelGGL(ep::rans_encode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), coset_dev,
-                     fields_dev, vectors, tile_vectors, tiles, reinterpret_cast<const uint2*>(entries_dev), table_rel_dev, total_entries, prob_bits, states_dev, tile_words_dev,
-                     scratch_dev, error_dev);
+  constexpr int kMostStagedEntries = 6144;                // 48 KiB of LDS
+  if (total_entries <= kMostStagedEntries)
+    hipLaunchKernelGGL(ep::rans_encode_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(256), static_cast<size_t>(total_entries) * 8,
+                       static_cast<hipStream_t>(stream), coset_dev, fields_dev, vectors, tile_vectors, tiles,
+                       reinterpret_cast<const uint2*>(entries_dev), table_rel_dev, total_entries, prob_bits, states_dev, tile_words_dev,
+                       scratch_dev, error_dev);
+  else
+    hipLaunchKernelGGL(ep::rans_encode_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       coset_dev, fields_dev, vectors, tile_vectors, tiles, reinterpret_cast<const uint2*>(entries_dev), table_rel_dev,
+                       total_entries, prob_bits, states_dev, tile_words_dev, scratch_dev, error_dev);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }
