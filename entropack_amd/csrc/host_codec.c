@@ -135,6 +135,76 @@ void hc_stream_counts(const int8_t* coset, const int32_t* fields, int64_t vector
   }
 }
 
+/* Largest-remainder (Hamilton) allocation of table_size slots over the symbols of a histogram, every present symbol
+ * getting at least one (entropack/schemes/lattice_rans/rans.py:12-71 of the reference): ideal = count * (table_size /
+ * total) in float64, floor, at least 1 where the count is not 0; a shortfall goes one slot at a time to the present
+ * symbols in order of descending residual ideal - freq, a surplus comes one slot at a time from the symbols still above
+ * 1 in order of ascending residual; equal residuals go by symbol, and a pass over the order repeats until the gap is
+ * closed. Returns 0, -1 for an empty histogram, -2 when a surplus cannot be taken back, -3 out of memory. */
+typedef struct {
+  double key;
+  int64_t symbol;
+} ranked_symbol;
+
+static int by_key_then_symbol(const void* a, const void* b) {
+  const ranked_symbol* x = (const ranked_symbol*)a;
+  const ranked_symbol* y = (const ranked_symbol*)b;
+  if (x->key < y->key) return -1;
+  if (x->key > y->key) return 1;
+  return (x->symbol > y->symbol) - (x->symbol < y->symbol);
+}
+
+int hc_normalize_counts(const int64_t* counts, int64_t n, int64_t table_size, uint16_t* freq_out) {
+  int64_t total = 0;
+  for (int64_t i = 0; i < n; ++i) total += counts[i];
+  if (n <= 0 || total == 0) return -1;
+  int64_t* freq = (int64_t*)malloc((size_t)n * sizeof(int64_t));
+  double* residual = (double*)malloc((size_t)n * sizeof(double));
+  ranked_symbol* order = (ranked_symbol*)malloc((size_t)n * sizeof(ranked_symbol));
+  if (!freq || !residual || !order) { free(freq); free(residual); free(order); return -3; }
+  const double scale = (double)table_size / (double)total;
+  int64_t given = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const double ideal = (double)counts[i] * scale;
+    freq[i] = (int64_t)floor(ideal);
+    if (counts[i] != 0 && freq[i] < 1) freq[i] = 1;
+    residual[i] = ideal - (double)freq[i];
+    given += freq[i];
+  }
+  int64_t gap = table_size - given;
+  int status = 0;
+  if (gap > 0) {
+    int64_t present = 0;
+    for (int64_t i = 0; i < n; ++i)
+      if (counts[i] != 0) { order[present].key = -residual[i]; order[present].symbol = i; ++present; }
+    qsort(order, (size_t)present, sizeof(ranked_symbol), by_key_then_symbol);
+    while (gap > 0) {
+      const int64_t take = gap < present ? gap : present;
+      for (int64_t k = 0; k < take; ++k) freq[order[k].symbol] += 1;
+      gap -= take;
+    }
+  } else if (gap < 0) {
+    int64_t pool = 0;
+    for (int64_t i = 0; i < n; ++i)
+      if (counts[i] != 0 && freq[i] > 1) { order[pool].key = residual[i]; order[pool].symbol = i; ++pool; }
+    if (pool == 0) status = -2;
+    else qsort(order, (size_t)pool, sizeof(ranked_symbol), by_key_then_symbol);
+    while (status == 0 && gap < 0) {
+      int64_t taken = 0;
+      for (int64_t k = 0; k < pool && taken < -gap; ++k)
+        if (freq[order[k].symbol] > 1) { freq[order[k].symbol] -= 1; ++taken; }
+      if (taken == 0) status = -2;
+      gap += taken;
+    }
+  }
+  if (status == 0)
+    for (int64_t i = 0; i < n; ++i) freq_out[i] = (uint16_t)freq[i];
+  free(freq);
+  free(residual);
+  free(order);
+  return status;
+}
+
 typedef struct {
   uint16_t* words;
   size_t size, capacity;

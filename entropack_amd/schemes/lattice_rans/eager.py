@@ -51,6 +51,8 @@ def host_library() -> ctypes.CDLL:
         lib.hc_stream_stats.restype = None
         lib.hc_stream_counts.argtypes = [p, p, i64, p, p, p]
         lib.hc_stream_counts.restype = None
+        lib.hc_normalize_counts.argtypes = [p, i64, i64, p]
+        lib.hc_normalize_counts.restype = i32
         lib.hc_rans_encode.argtypes = [p, p, i64, p, p, p, p, i32, i32, p, p, ctypes.POINTER(ctypes.c_void_p), i32]
         lib.hc_rans_encode.restype = i32
         lib.hc_tile_ans_encode.argtypes = [p, i64, i32, i64, i32, p, p, p, p, p, ctypes.POINTER(ctypes.c_void_p), i32]
@@ -157,40 +159,23 @@ def normalize_counts(counts: np.ndarray, table_size: int) -> np.ndarray:
     """Largest-remainder (Hamilton) allocation of `table_size` slots, every present symbol getting at least one.
 
     A surplus is handed out by descending residual, a deficit taken back by ascending residual from symbols still
-    above 1; ties go to the smaller symbol (stable sorts), and a symbol can be visited again in a later pass.
+    above 1; ties go to the smaller symbol, and a symbol can be visited again in a later pass. The arithmetic is
+    hc_normalize_counts of libentropack_host.so (float64 shares, as the reference's numpy code computes them).
     """
-    counts = np.asarray(counts, dtype=np.int64)
+    counts = np.ascontiguousarray(counts, dtype=np.int64)
     if counts.size == 0 or int(counts.sum()) == 0:
         raise ValueError("cannot build an rANS table from an empty symbol stream")
     if counts.size > table_size:
         raise ValueError(
             f"E8 coordinate alphabet {counts.size} exceeds rANS table_size {table_size}; "
             "raise prob_bits or coarsen the lattice scale")
-    seen = np.flatnonzero(counts)
-    ideal = counts.astype(np.float64) * (table_size / int(counts.sum()))
-    freq = np.floor(ideal).astype(np.int64)
-    freq[seen] = np.maximum(freq[seen], 1)
-    gap = table_size - int(freq.sum())
-    if gap > 0:
-        order = seen[np.argsort(-(ideal - freq)[seen], kind="stable")]
-        while gap > 0:
-            chosen = order[:gap]
-            freq[chosen] += 1
-            gap -= chosen.size
-    elif gap < 0:
-        rest = ideal - freq
-        pool = seen[freq[seen] > 1]
-        if pool.size == 0:
-            raise ValueError("unable to normalize rANS frequencies")
-        order = pool[np.argsort(rest[pool], kind="stable")]
-        while gap < 0:
-            alive = order[freq[order] > 1]
-            if alive.size == 0:
-                raise ValueError("unable to normalize rANS frequencies")
-            chosen = alive[:-gap]
-            freq[chosen] -= 1
-            gap += chosen.size
-    return freq.astype(np.uint16)
+    freq = np.empty(counts.size, dtype=np.uint16)
+    status = host_library().hc_normalize_counts(_address(counts), counts.size, table_size, _address(freq))
+    if status == -3:
+        raise MemoryError("frequency normalisation ran out of memory")
+    if status != 0:
+        raise ValueError("unable to normalize rANS frequencies")
+    return freq
 
 
 def modelled_bytes(histograms, sizes, rows: int, prob_bits: int, tile_elements: int) -> float:

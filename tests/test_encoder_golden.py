@@ -38,6 +38,78 @@ def test_config_1_rate_and_error_window():
     assert 0.11 < rel < 0.14
 
 
+def hamilton_in_numpy(counts: np.ndarray, table_size: int) -> np.ndarray:
+    """The allocation written out with numpy, step for step as the reference's rans.py:12-71 computes it (float64
+    shares, floor, at least one slot per present symbol, stable sorts of the residuals, repeated passes): what the C
+    routine behind `eager.normalize_counts` has to reproduce for every histogram, beyond the golden containers."""
+    counts = np.asarray(counts, dtype=np.int64)
+    seen = np.flatnonzero(counts)
+    ideal = counts.astype(np.float64) * (table_size / int(counts.sum()))
+    freq = np.floor(ideal).astype(np.int64)
+    freq[seen] = np.maximum(freq[seen], 1)
+    gap = table_size - int(freq.sum())
+    if gap > 0:
+        order = seen[np.argsort(-(ideal - freq)[seen], kind="stable")]
+        while gap > 0:
+            chosen = order[:gap]
+            freq[chosen] += 1
+            gap -= chosen.size
+    elif gap < 0:
+        rest = ideal - freq
+        pool = seen[freq[seen] > 1]
+        if pool.size == 0:
+            raise ValueError("unable to normalize rANS frequencies")
+        order = pool[np.argsort(rest[pool], kind="stable")]
+        while gap < 0:
+            alive = order[freq[order] > 1]
+            if alive.size == 0:
+                raise ValueError("unable to normalize rANS frequencies")
+            chosen = alive[:-gap]
+            freq[chosen] -= 1
+            gap += chosen.size
+    return freq.astype(np.uint16)
+
+
+def test_hamilton_normalisation_matches_the_numpy_formulation():
+    rng = np.random.default_rng(7)
+    shortfalls = surpluses = 0
+    for trial in range(3000):
+        size = 1 << int(rng.integers(9, 16))
+        width = int(rng.integers(1, min(size, 700) + 1))
+        kind = trial % 5
+        if kind == 0:
+            counts = rng.integers(0, 50, size=width)
+        elif kind == 1:                                   # a few heavy symbols over a long tail of ones: slots must be taken back
+            counts = np.ones(width, dtype=np.int64)
+            counts[rng.integers(0, width, size=3)] = rng.integers(10 ** 3, 10 ** 7, size=3)
+        elif kind == 2:                                   # many exact ties
+            counts = np.full(width, int(rng.integers(1, 9)), dtype=np.int64)
+            counts[rng.integers(0, width, size=width // 3)] *= 2
+        elif kind == 3:
+            counts = np.floor(rng.exponential(40.0, size=width)).astype(np.int64)
+        else:
+            counts = (rng.integers(0, 2, size=width) * rng.integers(1, 10 ** 9, size=width)).astype(np.int64)
+        if int(counts.sum()) == 0:
+            counts[0] = 1
+        try:
+            want = hamilton_in_numpy(counts, size)
+        except ValueError:
+            with pytest.raises(ValueError):
+                eager.normalize_counts(counts, size)
+            continue
+        floor_sum = int(np.maximum(np.floor(counts * (size / counts.sum())), counts > 0).sum())
+        shortfalls += floor_sum < size
+        surpluses += floor_sum > size
+        got = eager.normalize_counts(counts, size)
+        assert np.array_equal(got, want), (trial, counts.tolist(), size)
+    assert shortfalls > 500 and surpluses > 200           # both directions were exercised, not only the common one
+    assert eager.normalize_counts(np.array([5]), 2048).tolist() == [2048]
+    full = eager.normalize_counts(np.ones(512, dtype=np.int64), 512)
+    assert full.tolist() == [1] * 512
+    with pytest.raises(ValueError):                      # every symbol already at one slot and still too many
+        eager.normalize_counts(np.ones(513, dtype=np.int64), 512)
+
+
 def test_hamilton_normalisation_properties():
     rng = np.random.default_rng(1)
     for size in (512, 2048):
