@@ -314,30 +314,42 @@ __global__ __launch_bounds__(256) void rans_encode_kernel(const int8_t* __restri
   if (bad) *error = 1;
 }
 
-// offsets[0] = 0, offsets[t + 1] = words of tiles 0..t (modulo 2^32; *total holds the full sum). One block.
+// offsets[0] = 0, offsets[t + 1] = words of tiles 0..t (modulo 2^32; *total holds the full sum). One block walks the
+// counts 1024 at a time: every thread holds one count (the next chunk's is already on its way), the wavefronts scan
+// theirs with shuffles, sixteen wavefront totals meet in LDS, and a 64-bit carry runs from chunk to chunk.
 __global__ __launch_bounds__(1024) void offsets_kernel(const uint32_t* __restrict__ tile_words, int64_t tiles, uint32_t* __restrict__ offsets,
                                                        unsigned long long* __restrict__ total) {
-  __shared__ unsigned long long sums[1024];
-  const int t = threadIdx.x;
-  const int64_t share = (tiles + 1023) / 1024;
-  const int64_t first = t * share, last = first + share < tiles ? first + share : tiles;
-  unsigned long long mine = 0;
-  for (int64_t i = first; i < last; ++i) mine += tile_words[i];
-  sums[t] = mine;
-  __syncthreads();
-  for (int distance = 1; distance < 1024; distance <<= 1) {
-    const unsigned long long before = t >= distance ? sums[t - distance] : 0;
+  __shared__ unsigned long long wave_totals[16];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  unsigned long long carry = 0;
+  uint32_t coming = t < tiles ? tile_words[t] : 0u;
+  for (int64_t base = 0; base < tiles; base += 1024) {
+    const uint32_t mine = coming;
+    const int64_t after = base + 1024 + t;
+    coming = after < tiles ? tile_words[after] : 0u;
+    unsigned long long upto = mine;                        // inclusive sum over the lanes of this wavefront up to this one
+#pragma unroll
+    for (int distance = 1; distance < 64; distance <<= 1) {
+      const unsigned long long from_below = __shfl_up(upto, distance);
+      if (lane >= distance) upto += from_below;
+    }
+    if (lane == 63) wave_totals[wave] = upto;
     __syncthreads();
-    sums[t] += before;
+    unsigned long long before = 0, chunk = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const unsigned long long one = wave_totals[w];
+      before += w < wave ? one : 0ull;
+      chunk += one;
+    }
+    if (base + t < tiles) offsets[base + t + 1] = static_cast<uint32_t>(carry + before + upto);
+    carry += chunk;
     __syncthreads();
   }
-  unsigned long long running = sums[t] - mine;
-  if (t == 0) offsets[0] = 0;
-  for (int64_t i = first; i < last; ++i) {
-    running += tile_words[i];
-    offsets[i + 1] = static_cast<uint32_t>(running);
+  if (t == 0) {
+    offsets[0] = 0;
+    *total = carry;
   }
-  if (t == 1023) *total = sums[1023];
 }
 
 // payload[offsets[t] ..) = the words stream t left at the start of its `stride` words of the scratch.
