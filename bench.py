@@ -697,6 +697,7 @@ def store_pattern_workload(args, ep):
     for tile_vectors in (3640, 1820, 1824, 910, 912, 455, 456):
         streamed = pattern(tile_vectors, 0)
         by_tile[f"tile_vectors={tile_vectors}"] = {"streaming_stores_us": streamed, "plain_stores_us": pattern(tile_vectors, 1),
+                                                   "streaming_heads_delayed_us": pattern(tile_vectors, 2),
                                                    "GBps_streaming": round(nbytes / streamed / 1e3, 1)}
     fill = timed(lambda: out.fill_(1.0))
     copy = timed(lambda: other.copy_(out))

@@ -13,7 +13,7 @@ namespace ep {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <int POLICY>     // 0: streaming stores (the decode kernels'), 1: stores through the cache
+template <int POLICY>     // 0: streaming stores (the decode kernels'), 1: stores through the cache, 2: streaming, heads delayed
 __global__ __launch_bounds__(1024) void store_pattern_kernel(uint8_t* __restrict__ out, int64_t vectors, int tile_vectors) {
   const int lane = threadIdx.x & 63, half = lane >> 5, l32 = lane & 31;
   const int64_t wave = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -25,6 +25,18 @@ __global__ __launch_bounds__(1024) void store_pattern_kernel(uint8_t* __restrict
     const int64_t first = tile * tile_vectors;
     const int64_t left = vectors - first;
     const int count = static_cast<int>(left < tile_vectors ? left : tile_vectors);
+    if (POLICY == 2) {
+      // The first `late` lanes of a group hold the vectors in front of the next 64-byte boundary: they wait one turn and go
+      // out with the group below, so that every store instruction covers whole 64-byte lines.
+      const int late = static_cast<int>((4 - (first & 3)) & 3);
+      for (int offset = (count - 1) & ~31; offset >= -32; offset -= 32) {
+        const int vector = l32 < late ? offset + 32 + l32 : offset + l32;
+        if (vector < 0 || vector >= count || (offset < 0 && l32 >= late)) continue;
+        const u32x4 value = {static_cast<uint32_t>(tile), static_cast<uint32_t>(vector & ~31), static_cast<uint32_t>(l32), 0u};
+        __builtin_nontemporal_store(value, reinterpret_cast<u32x4*>(out + 16 * (first + vector)));
+      }
+      continue;
+    }
     for (int offset = (count - 1) & ~31; offset >= 0; offset -= 32) {
       if (offset + l32 >= count) continue;
       const u32x4 value = {static_cast<uint32_t>(tile), static_cast<uint32_t>(offset), static_cast<uint32_t>(l32), 0u};
@@ -44,7 +56,8 @@ extern "C" int ep_hip_probe_store_pattern(void* out_dev, int64_t vectors, int ti
   EP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
   const dim3 grid(static_cast<unsigned>(2 * (cus > 0 ? cus : 256))), block(1024);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (through_cache) hipLaunchKernelGGL(ep::store_pattern_kernel<1>, grid, block, 0, s, static_cast<uint8_t*>(out_dev), vectors, tile_vectors);
+  if (through_cache == 2) hipLaunchKernelGGL(ep::store_pattern_kernel<2>, grid, block, 0, s, static_cast<uint8_t*>(out_dev), vectors, tile_vectors);
+  else if (through_cache) hipLaunchKernelGGL(ep::store_pattern_kernel<1>, grid, block, 0, s, static_cast<uint8_t*>(out_dev), vectors, tile_vectors);
   else hipLaunchKernelGGL(ep::store_pattern_kernel<0>, grid, block, 0, s, static_cast<uint8_t*>(out_dev), vectors, tile_vectors);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;

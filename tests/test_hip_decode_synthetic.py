@@ -227,7 +227,7 @@ def test_store_pattern_probe_writes_every_vector_once(vectors, tile_vectors):
     """The measurement aid of bench.py --workload store_pattern: every vector of the buffer, and nothing beyond it, gets
     the (tile, offset in the tile, lane) that a decode of such tiles would have written it from."""
     library = hip_backend.library()
-    for through_cache in (0, 1):
+    for through_cache in (0, 1, 2):
         out = torch.full((vectors + 8, 4), -1, dtype=torch.int32, device="cuda")
         status = library.ep_hip_probe_store_pattern(out.data_ptr(), vectors, tile_vectors, through_cache, torch.cuda.current_stream().cuda_stream)
         assert status == hip_backend.OK
