@@ -1,5 +1,5 @@
-// The encoders on the device. First the lattice_rans encoder: nearest-E8 quantisation, stream statistics, row-scale refit and the tiled
-// 32-way interleaved rANS encode. Every kernel produces, from the same inputs, exactly what the CPU encoder
+// The encoders on the device. First the lattice_rans encoder: nearest-E8 quantisation, stream statistics, row-scale refit
+// and the tiled 32-way interleaved rANS encode. Every kernel produces, from the same inputs, exactly what the CPU encoder
 // (csrc/host_codec.c) produces: the float work is single IEEE operations in the same order (this file is compiled
 // without contraction), the rest is integer work. The one exception is the row-scale refit, whose float32 row sums are
 // added in this kernel's own fixed order (the CPU lane adds them in torch's).
