@@ -205,6 +205,62 @@ int hc_normalize_counts(const int64_t* counts, int64_t n, int64_t table_size, ui
   return status;
 }
 
+/* The lossless scheme's allocation of table_size slots (entropack/schemes/tile_ans/eager.py:17-60 of the reference):
+ * floor of the exact float64 share, at least 1 for a present symbol; then one slot at a time, a shortfall to the symbol
+ * with the largest remainder (its remainder drops by one when it is served), a surplus from the symbol with the
+ * smallest remainder among those above one slot (its remainder rises by one; at one slot it leaves the pool); the
+ * smallest symbol among equals. Returns 0, -1 for an empty histogram, -2 when a surplus cannot be taken back, -3 out of
+ * memory. */
+int hc_tile_ans_normalize_counts(const int64_t* counts, int64_t n, int64_t table_size, uint16_t* freq_out) {
+  int64_t total = 0;
+  for (int64_t i = 0; i < n; ++i) total += counts[i];
+  if (n <= 0 || total == 0) return -1;
+  int64_t* freq = (int64_t*)malloc((size_t)n * sizeof(int64_t));
+  double* key = (double*)malloc((size_t)n * sizeof(double));
+  if (!freq || !key) { free(freq); free(key); return -3; }
+  const double scale = (double)table_size / (double)total;
+  int64_t given = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const double share = (double)counts[i] * scale;
+    freq[i] = (int64_t)floor(share);
+    if (counts[i] != 0 && freq[i] < 1) freq[i] = 1;
+    key[i] = share - (double)freq[i];           /* the remainder, for now */
+    given += freq[i];
+  }
+  const int64_t gap = table_size - given;
+  int status = 0;
+  if (gap > 0) {
+    for (int64_t i = 0; i < n; ++i) key[i] = counts[i] != 0 ? -key[i] : INFINITY;
+    for (int64_t step = 0; step < gap; ++step) {
+      int64_t best = 0;
+      for (int64_t i = 1; i < n; ++i)
+        if (key[i] < key[best]) best = i;       /* first minimum */
+      freq[best] += 1;
+      key[best] += 1.0;
+    }
+  } else if (gap < 0) {
+    int64_t pool = 0;
+    for (int64_t i = 0; i < n; ++i) {
+      if (counts[i] != 0 && freq[i] > 1) ++pool;
+      else key[i] = INFINITY;
+    }
+    if (pool == 0) status = -2;
+    for (int64_t step = 0; status == 0 && step < -gap; ++step) {
+      int64_t best = 0;
+      for (int64_t i = 1; i < n; ++i)
+        if (key[i] < key[best]) best = i;
+      if (isinf(key[best])) { status = -2; break; }
+      freq[best] -= 1;
+      key[best] = freq[best] > 1 ? key[best] + 1.0 : INFINITY;
+    }
+  }
+  if (status == 0)
+    for (int64_t i = 0; i < n; ++i) freq_out[i] = (uint16_t)freq[i];
+  free(freq);
+  free(key);
+  return status;
+}
+
 typedef struct {
   uint16_t* words;
   size_t size, capacity;

@@ -53,6 +53,8 @@ def host_library() -> ctypes.CDLL:
         lib.hc_stream_counts.restype = None
         lib.hc_normalize_counts.argtypes = [p, i64, i64, p]
         lib.hc_normalize_counts.restype = i32
+        lib.hc_tile_ans_normalize_counts.argtypes = [p, i64, i64, p]
+        lib.hc_tile_ans_normalize_counts.restype = i32
         lib.hc_rans_encode.argtypes = [p, p, i64, p, p, p, p, i32, i32, p, p, ctypes.POINTER(ctypes.c_void_p), i32]
         lib.hc_rans_encode.restype = i32
         lib.hc_tile_ans_encode.argtypes = [p, i64, i32, i64, i32, p, p, p, p, p, ctypes.POINTER(ctypes.c_void_p), i32]

@@ -25,37 +25,19 @@ def normalize_counts(counts: np.ndarray, table_size: int) -> np.ndarray:
 
     Floor of the exact share, then the deficit goes one unit at a time to the symbol with the largest remainder (a
     symbol's remainder drops by one when it is served; ties go to the smaller symbol); a surplus is taken one unit at
-    a time from the symbol with the smallest remainder among those above 1 (its remainder rises by one).
+    a time from the symbol with the smallest remainder among those above 1 (its remainder rises by one). The loop is
+    hc_tile_ans_normalize_counts of libentropack_host.so.
     """
-    counts = np.asarray(counts, dtype=np.int64)
-    present = np.flatnonzero(counts)
-    if present.size == 0:
+    counts = np.ascontiguousarray(counts, dtype=np.int64)
+    freq = np.empty(counts.size, dtype=np.uint16)
+    status = host_library().hc_tile_ans_normalize_counts(counts.ctypes.data, counts.size, table_size, freq.ctypes.data)
+    if status == -1:
         raise ValueError("cannot build an rANS codebook from empty input")
-    share = counts.astype(np.float64) * (table_size / int(counts.sum()))
-    freq = np.floor(share).astype(np.int64)
-    freq[present] = np.maximum(freq[present], 1)
-    gap = table_size - int(freq.sum())
-    remainder = share - freq
-    if gap > 0:
-        key = np.full(counts.shape, np.inf)
-        key[present] = -remainder[present]
-        for _ in range(gap):
-            symbol = int(np.argmin(key))              # first minimum = smallest symbol among equals
-            freq[symbol] += 1
-            key[symbol] += 1.0
-    elif gap < 0:
-        key = np.full(counts.shape, np.inf)
-        pool = present[freq[present] > 1]
-        if pool.size == 0:
-            raise ValueError("unable to normalize rANS frequencies")
-        key[pool] = remainder[pool]
-        for step in range(-gap):
-            symbol = int(np.argmin(key))
-            if not np.isfinite(key[symbol]):
-                raise ValueError("unable to normalize rANS frequencies")
-            freq[symbol] -= 1
-            key[symbol] = key[symbol] + 1.0 if freq[symbol] > 1 else np.inf
-    return freq.astype(np.uint16)
+    if status == -3:
+        raise MemoryError("frequency normalisation ran out of memory")
+    if status != 0:
+        raise ValueError("unable to normalize rANS frequencies")
+    return freq
 
 
 def tables_from_frequencies(frequencies: np.ndarray, probability_bits: int):

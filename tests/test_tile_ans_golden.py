@@ -179,6 +179,72 @@ def test_normalised_frequencies_keep_every_symbol_and_the_total(seed):
         assert np.all((tables[0] >> 20) == cdfs[0][symbols])
 
 
+def one_slot_at_a_time_in_numpy(counts: np.ndarray, table_size: int) -> np.ndarray:
+    """The allocation written out with numpy, step for step as the reference's tile_ans/eager.py:17-60 computes it: what
+    the C loop behind `tile_eager.normalize_counts` has to reproduce for every histogram, beyond the golden containers."""
+    counts = np.asarray(counts, dtype=np.int64)
+    present = np.flatnonzero(counts)
+    share = counts.astype(np.float64) * (table_size / int(counts.sum()))
+    freq = np.floor(share).astype(np.int64)
+    freq[present] = np.maximum(freq[present], 1)
+    gap = table_size - int(freq.sum())
+    remainder = share - freq
+    if gap > 0:
+        key = np.full(counts.shape, np.inf)
+        key[present] = -remainder[present]
+        for _ in range(gap):
+            symbol = int(np.argmin(key))
+            freq[symbol] += 1
+            key[symbol] += 1.0
+    elif gap < 0:
+        key = np.full(counts.shape, np.inf)
+        pool = present[freq[present] > 1]
+        if pool.size == 0:
+            raise ValueError("unable to normalize rANS frequencies")
+        key[pool] = remainder[pool]
+        for _ in range(-gap):
+            symbol = int(np.argmin(key))
+            if not np.isfinite(key[symbol]):
+                raise ValueError("unable to normalize rANS frequencies")
+            freq[symbol] -= 1
+            key[symbol] = key[symbol] + 1.0 if freq[symbol] > 1 else np.inf
+    return freq.astype(np.uint16)
+
+
+def test_normalised_frequencies_match_the_numpy_formulation():
+    rng = np.random.default_rng(11)
+    shortfalls = surpluses = 0
+    for trial in range(1500):
+        bits = int(rng.choice(tile_format.SUPPORTED_PROB_BITS))
+        counts = np.zeros(256, dtype=np.int64)
+        kind = trial % 4
+        if kind == 0:
+            present = rng.choice(256, size=rng.integers(1, 257), replace=False)
+            counts[present] = rng.integers(1, 10 ** rng.integers(1, 8), size=present.size)
+        elif kind == 1:                                  # a long tail of rare symbols under a few heavy ones: slots come back
+            counts[:] = rng.integers(0, 3, size=256)
+            counts[rng.integers(0, 256, size=4)] = rng.integers(10 ** 5, 10 ** 8, size=4)
+        elif kind == 2:                                  # exact ties
+            counts[rng.choice(256, size=rng.integers(2, 200), replace=False)] = int(rng.integers(1, 50))
+        else:
+            counts[:] = np.floor(rng.exponential(200.0, size=256)).astype(np.int64)
+        if int(counts.sum()) == 0:
+            counts[7] = 3
+        try:
+            want = one_slot_at_a_time_in_numpy(counts, 1 << bits)
+        except ValueError:
+            with pytest.raises(ValueError):
+                tile_eager.normalize_counts(counts, 1 << bits)
+            continue
+        floors = int(np.maximum(np.floor(counts * ((1 << bits) / counts.sum())), counts > 0).sum())
+        shortfalls += floors < (1 << bits)
+        surpluses += floors > (1 << bits)
+        assert np.array_equal(tile_eager.normalize_counts(counts, 1 << bits), want), (trial, bits, counts.tolist())
+    assert shortfalls > 300 and surpluses > 100
+    with pytest.raises(ValueError, match="empty"):
+        tile_eager.normalize_counts(np.zeros(256, dtype=np.int64), 512)
+
+
 def test_config_validation_and_defaults():
     from entropack_amd.schemes.config import validate_config
     validate_config(ep.TileANSConfig())
