@@ -348,7 +348,7 @@ def _as_torch(array: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
     return torch.from_numpy(np.ascontiguousarray(array).view(signed)).view(dtype)
 
 
-def check_encode_request(weight, row_rdo_iterations) -> None:
+def check_encode_request(weight) -> None:
     if weight.shape[1] % LATTICE_DIM:
         raise ValueError(
             f"lattice_rans quantizes whole E8 vectors, so the column count must be a multiple of {LATTICE_DIM}; got cols={weight.shape[1]}")
@@ -365,7 +365,7 @@ def row_rms(x_t: torch.Tensor, source_dtype) -> torch.Tensor:
 
 def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0, row_rdo_candidates=5,
            scale_search_iterations=12, scale_search_max_vectors=262144) -> LatticeBuffers:
-    check_encode_request(weight, row_rdo_iterations)
+    check_encode_request(weight)
     device = weight.device
     x_t = weight.detach().to("cpu").float().contiguous()
     rows, cols = x_t.shape

@@ -221,7 +221,7 @@ def row_rms(x: torch.Tensor, source_dtype) -> torch.Tensor:
 
 def encode(*, weight, target_bpp, prob_bits, tile_elements, row_rdo_iterations=0, row_rdo_candidates=5,
            scale_search_iterations=12, scale_search_max_vectors=262144) -> LatticeBuffers:
-    eager.check_encode_request(weight, row_rdo_iterations)
+    eager.check_encode_request(weight)
     if weight.device.type != "cuda":
         raise ValueError("the hip lane encodes tensors that are on the GPU; use execution_backend='eager' for CPU tensors")
     x = weight.detach().float().contiguous()
