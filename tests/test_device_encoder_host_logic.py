@@ -1,5 +1,7 @@
 """Host-side logic of the device encoder (no GPU): the stream statistics read from the quantise kernel's summary, the
 table entries with their reciprocals, and the quantizer interface the scale search drives."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -72,3 +74,32 @@ def test_device_quantizer_refuses_host_tensors():
         hip_encode.DeviceQuantizer(torch.zeros(2, 8), torch.ones(2, 1))
     with pytest.raises(ValueError, match="on the GPU"):
         hip_encode.encode(weight=torch.zeros(2, 8), target_bpp=4.0, prob_bits=None, tile_elements=16384)
+
+
+def test_entry_points_refuse_bad_arguments_before_touching_a_device():
+    """Argument checks come first in every encoder entry point, so they can be exercised without a GPU: null pointers,
+    column counts that are no whole vectors, a scale that is not positive, misaligned buffers, tiles below 32 vectors,
+    element sizes the lossless coder does not take."""
+    from entropack_amd.backends import hip
+    lib = hip.library()
+    a = 1 << 20                                            # any 16-byte aligned non-null value: never dereferenced
+    assert lib.ep_hip_encode_quantize(None, a, 64, 1.0, None, 4, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_quantize(a, a, 60, 1.0, None, 4, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_quantize(a, a, 64, 0.0, None, 4, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_quantize(a + 4, a, 64, 1.0, None, 4, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_histogram(a, a, 0, a, 8, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_histogram(a, a + 8, 16, a, 8, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_row_scales(a, a, 64, 1.0, 0, a, a, a, None, None) == hip.EINVAL
+    assert lib.ep_hip_encode_row_scales(a, a, 63, 1.0, 4, a, a, a, None, None) == hip.EINVAL
+    assert lib.ep_hip_encode_rans(a, a, 64, a, a, 10, 11, 31, a, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_rans(a, a, 64, a, a, 10, 16, 32, a, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_rans(a, a, 64, a + 4, a, 10, 11, 32, a, a, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_offsets(a, 0, a, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_offsets(a, 4, a, a + 4, None) == hip.EINVAL
+    assert lib.ep_hip_encode_gather(a, a, 4, 0, a, None) == hip.EINVAL
+    assert lib.ep_hip_tile_ans_histogram(a, 16, 3, a, None) == hip.EUNSUPPORTED
+    assert lib.ep_hip_tile_ans_histogram(a + 1, 16, 2, a, None) == hip.EINVAL
+    raw = (ctypes.c_uint8 * 2)(1, 0)
+    assert lib.ep_hip_tile_ans_encode(a, 16, 2, 8, 10, a, raw, None, a, a, 8, a, None) == hip.EINVAL       # a coded lane needs states
+    assert lib.ep_hip_tile_ans_encode(a, 16, 2, 8, 10, a, raw, a, a, a, 4, a, None) == hip.EINVAL          # stride below the tile
+    assert lib.ep_hip_tile_ans_encode(a, 16, 5, 8, 10, a, raw, a, a, a, 8, a, None) == hip.EUNSUPPORTED
