@@ -133,9 +133,12 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
   }
   if (ones != 0) atomicAdd(&ones_shared, ones);
   __syncthreads();
+  // Most blocks have nothing to add to what others already recorded: a look at the current value (it only ever moves
+  // one way, so a stale look costs an atomic that changes nothing) spares the device thousands of atomics on 32 words.
   if (threadIdx.x < kFieldStreams && lo_shared[threadIdx.x] != INT_MAX) {
-    atomicMin(&summary[2 * threadIdx.x], static_cast<long long>(lo_shared[threadIdx.x]));
-    atomicMax(&summary[2 * threadIdx.x + 1], static_cast<long long>(hi_shared[threadIdx.x]));
+    const volatile long long* seen = summary;
+    if (lo_shared[threadIdx.x] < seen[2 * threadIdx.x]) atomicMin(&summary[2 * threadIdx.x], static_cast<long long>(lo_shared[threadIdx.x]));
+    if (hi_shared[threadIdx.x] > seen[2 * threadIdx.x + 1]) atomicMax(&summary[2 * threadIdx.x + 1], static_cast<long long>(hi_shared[threadIdx.x]));
   }
   if (threadIdx.x == 0 && ones_shared != 0)
     atomicAdd(reinterpret_cast<unsigned long long*>(&summary[kSummaryOnes]), static_cast<unsigned long long>(ones_shared));
