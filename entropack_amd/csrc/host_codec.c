@@ -205,6 +205,16 @@ int hc_normalize_counts(const int64_t* counts, int64_t n, int64_t table_size, ui
   return status;
 }
 
+/* hc_normalize_counts for several histograms laid end to end: histogram s is counts[starts[s] .. starts[s + 1]), its
+ * frequencies go to the same positions of freq_out. Returns 0, or the first histogram's error code. */
+int hc_normalize_streams(const int64_t* counts, const int64_t* starts, int64_t n_streams, int64_t table_size, uint16_t* freq_out) {
+  for (int64_t s = 0; s < n_streams; ++s) {
+    const int status = hc_normalize_counts(counts + starts[s], starts[s + 1] - starts[s], table_size, freq_out + starts[s]);
+    if (status != 0) return status;
+  }
+  return 0;
+}
+
 /* The lossless scheme's allocation of table_size slots (entropack/schemes/tile_ans/eager.py:17-60 of the reference):
  * floor of the exact float64 share, at least 1 for a present symbol; then one slot at a time, a shortfall to the symbol
  * with the largest remainder (its remainder drops by one when it is served), a surplus from the symbol with the

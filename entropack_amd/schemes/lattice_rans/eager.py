@@ -53,6 +53,8 @@ def host_library() -> ctypes.CDLL:
         lib.hc_stream_counts.restype = None
         lib.hc_normalize_counts.argtypes = [p, i64, i64, p]
         lib.hc_normalize_counts.restype = i32
+        lib.hc_normalize_streams.argtypes = [p, p, i64, i64, p]
+        lib.hc_normalize_streams.restype = i32
         lib.hc_tile_ans_normalize_counts.argtypes = [p, i64, i64, p]
         lib.hc_tile_ans_normalize_counts.restype = i32
         lib.hc_rans_encode.argtypes = [p, p, i64, p, p, p, p, i32, i32, p, p, ctypes.POINTER(ctypes.c_void_p), i32]
@@ -181,24 +183,39 @@ def normalize_counts(counts: np.ndarray, table_size: int) -> np.ndarray:
 
 
 def modelled_bytes(histograms, sizes, rows: int, prob_bits: int, tile_elements: int) -> float:
-    """Analytic container size for a set of stream histograms (reference rans.py:224-258 + eager.py:102-107)."""
+    """Analytic container size for a set of stream histograms (reference rans.py:224-258 + eager.py:102-107).
+
+    Per coded stream the reference adds count * (prob_bits - log2(freq)) over the symbols present, in float64 with
+    numpy's sum, and the streams' sums in stream order. The same numbers come out of one normalisation call and one
+    pass of element-wise arithmetic over the histograms laid end to end, with numpy's sum over each stream's slice
+    (element-wise results and a slice's sum do not depend on where in an array the elements lie).
+    """
     table_size = 1 << prob_bits
+    coded = [hist for n, hist in zip(sizes, histograms) if n and hist.size <= table_size]
+    overflow_bits = float(sum(n * prob_bits for n, hist in zip(sizes, histograms) if not (n and hist.size <= table_size)))
     bits = 0.0
     table_bytes = 0
-    overflow_bits = 0.0
-    for n, hist in zip(sizes, histograms):
-        if n and hist.size <= table_size:
-            freq = normalize_counts(hist, table_size)
-            live = hist > 0
-            bits += float(np.sum(hist[live].astype(np.float64) * (prob_bits - np.log2(freq[live].astype(np.float64)))))
-            table_bytes += freq.size * 2
-        else:
-            overflow_bits += n * prob_bits
+    if coded:
+        counts = np.ascontiguousarray(np.concatenate(coded), dtype=np.int64)
+        starts = np.zeros(len(coded) + 1, dtype=np.int64)
+        np.cumsum([hist.size for hist in coded], out=starts[1:])
+        freq = np.empty(counts.size, dtype=np.uint16)
+        status = host_library().hc_normalize_streams(_address(counts), _address(starts), len(coded), table_size, _address(freq))
+        if status == -3:
+            raise MemoryError("frequency normalisation ran out of memory")
+        if status != 0:
+            raise ValueError("unable to normalize rANS frequencies")
+        live = counts > 0
+        terms = counts[live].astype(np.float64) * (prob_bits - np.log2(freq[live].astype(np.float64)))
+        ends = np.concatenate([[0], np.cumsum(live)])[starts]          # where each stream's present symbols begin in `terms`
+        for k in range(len(coded)):
+            bits += float(np.sum(terms[ends[k]:ends[k + 1]]))
+        table_bytes = 2 * counts.size
     tile_vectors = vector_tile_elements(tile_elements)
     tiles = max(1, (sizes[0] + tile_vectors - 1) // tile_vectors)
     payload_words = int(np.ceil(max(0.0, bits - tiles * NUM_STATES * 16) / 16.0))
-    coded = payload_words * 2 + tiles * NUM_STATES * 4 + (tiles + 1) * 4 + table_bytes
-    return coded + overflow_bits / 8 + rows * 4 + MODEL_LAYOUT_BYTES + MODEL_STREAM_META_BYTES + MODEL_SLACK_BYTES
+    coded_bytes = payload_words * 2 + tiles * NUM_STATES * 4 + (tiles + 1) * 4 + table_bytes
+    return coded_bytes + overflow_bits / 8 + rows * 4 + MODEL_LAYOUT_BYTES + MODEL_STREAM_META_BYTES + MODEL_SLACK_BYTES
 
 
 def _model_of(q, rows: int, prob_bits: int, tile_elements: int) -> float:

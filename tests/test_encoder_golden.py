@@ -110,6 +110,46 @@ def test_hamilton_normalisation_matches_the_numpy_formulation():
         eager.normalize_counts(np.ones(513, dtype=np.int64), 512)
 
 
+def size_model_stream_by_stream(histograms, sizes, rows, prob_bits, tile_elements):
+    """The size model with one normalisation, one log2 and one sum per stream, as the reference's rans.py:224-258 and
+    eager.py:102-107 go about it: what `eager.modelled_bytes`, which works on the histograms laid end to end, has to
+    return to the last bit (the scale search compares its result with the target)."""
+    from entropack_amd.schemes.lattice_rans.format import NUM_STATES, vector_tile_elements
+    table_size = 1 << prob_bits
+    bits, table_bytes, overflow_bits = 0.0, 0, 0.0
+    for n, hist in zip(sizes, histograms):
+        if n and hist.size <= table_size:
+            freq = hamilton_in_numpy(hist, table_size)
+            live = hist > 0
+            bits += float(np.sum(hist[live].astype(np.float64) * (prob_bits - np.log2(freq[live].astype(np.float64)))))
+            table_bytes += freq.size * 2
+        else:
+            overflow_bits += n * prob_bits
+    tile_vectors = vector_tile_elements(tile_elements)
+    tiles = max(1, (sizes[0] + tile_vectors - 1) // tile_vectors)
+    payload_words = int(np.ceil(max(0.0, bits - tiles * NUM_STATES * 16) / 16.0))
+    coded = payload_words * 2 + tiles * NUM_STATES * 4 + (tiles + 1) * 4 + table_bytes
+    return (coded + overflow_bits / 8 + rows * 4 + eager.MODEL_LAYOUT_BYTES + eager.MODEL_STREAM_META_BYTES + eager.MODEL_SLACK_BYTES), bits
+
+
+def test_size_model_matches_the_stream_by_stream_formulation():
+    rng = np.random.default_rng(3)
+    for trial in range(400):
+        prob_bits = int(rng.integers(9, 16))
+        histograms, sizes = [], []
+        for stream in range(17):
+            width = int(rng.integers(1, 90)) if rng.random() < 0.9 else int(rng.integers(400, 1200))      # some overflow a 9-bit table
+            if stream and rng.random() < 0.1:
+                histograms.append(np.zeros(0, dtype=np.int64)); sizes.append(0)                           # an empty stream
+                continue
+            hist = np.floor(rng.exponential(10.0 ** rng.uniform(0, 5), size=width)).astype(np.int64)
+            hist[0] = max(hist[0], 1); hist[-1] = max(hist[-1], 1)
+            histograms.append(hist); sizes.append(int(hist.sum()))
+        want, want_bits = size_model_stream_by_stream(histograms, sizes, 64, prob_bits, 16384)
+        assert eager.modelled_bytes(histograms, sizes, 64, prob_bits, 16384) == want, trial
+        assert want_bits > 0.0
+
+
 def test_hamilton_normalisation_properties():
     rng = np.random.default_rng(1)
     for size in (512, 2048):
