@@ -1,6 +1,6 @@
 """Headline benchmark: lossy (lattice_rans) decode throughput on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|store_pattern|encode|tile_ans_encode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|encode|tile_ans_encode]
 
 One "step" = one decode of the whole container (entropy decode + E8 reconstruction + BF16 store) from buffers
 already resident in HBM. Prints ONE JSON line. `value` = algorithmic bytes (container bytes read + dense bytes
@@ -662,61 +662,6 @@ def gemm_workload(args, ep):
     return 0
 
 
-def store_pattern_workload(args, ep):
-    """The output side of the headline decode on its own: the 8192 x 28672 bf16 weight written in the decode kernels' order
-    and shape with nothing decoded (`ep_hip_probe_store_pattern`), for the tile lengths the encoder's defaults give (3640,
-    1820, 910, 455 vectors) and their neighbours that are multiples of four or eight vectors, beside a plain fill and a
-    plain copy of the same tensor. Device times: the launches between one pair of events, after the clocks have settled."""
-    from entropack_amd.backends import hip as hip_backend
-    library = hip_backend.library()
-    rows, cols = WORKLOADS["target"][:2]
-    vectors = rows * cols // 8
-    out = torch.empty(rows * cols, dtype=torch.bfloat16, device="cuda")
-    other = torch.empty_like(out)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def timed(fn, count=100):
-        settle(fn)
-        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        first.record()
-        for _ in range(count):
-            fn()
-        last.record()
-        torch.cuda.synchronize()
-        return round(first.elapsed_time(last) / count * 1e3, 2)
-
-    def pattern(tile_vectors, through_cache):
-        def launch():
-            status = library.ep_hip_probe_store_pattern(out.data_ptr(), vectors, tile_vectors, through_cache, stream)
-            if status:
-                raise hip_backend.HipError(status, "ep_hip_probe_store_pattern")
-        return timed(launch)
-
-    nbytes = 2 * rows * cols
-    by_tile = {}
-    for tile_vectors in (3640, 1820, 1824, 910, 912, 455, 456):
-        streamed = pattern(tile_vectors, 0)
-        by_tile[f"tile_vectors={tile_vectors}"] = {"streaming_stores_us": streamed, "plain_stores_us": pattern(tile_vectors, 1),
-                                                   "streaming_heads_delayed_us": pattern(tile_vectors, 2),
-                                                   "GBps_streaming": round(nbytes / streamed / 1e3, 1)}
-    fill = timed(lambda: out.fill_(1.0))
-    copy = timed(lambda: other.copy_(out))
-    headline = by_tile["tile_vectors=1820"]["streaming_stores_us"]
-    result = {
-        "metric": "GB/s written in the decode kernels' store pattern, 8192x28672 bf16, default tiles", "value": round(nbytes / headline / 1e3, 1),
-        "unit": "GB/s", "n_gpus": 1, "steps": 100, "warmup": 0, "ms_per_step": round(headline / 1e3, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "u32", "data": "synthetic",
-        "config": {"workload": "store pattern of a bf16 lattice decode without the decode: one tile per 32-lane half, top-down, 16 bytes per lane",
-                   "bytes_written": nbytes, "by_tile_length": by_tile,
-                   "plain_fill_us": fill, "plain_fill_GBps": round(nbytes / fill / 1e3, 1),
-                   "plain_copy_us": copy, "plain_copy_GBps_read_plus_write": round(2 * nbytes / copy / 1e3, 1)},
-        "roofline": {"bound": "hbm", "achieved": round(nbytes / headline / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(nbytes / headline / 1e3 / HBM_PEAK_GBPS, 5), "traffic": None},
-    }
-    print(json.dumps(result))
-    return 0
-
-
 def encode_workload(args, ep):
     """The step before the path: `compress` of the target weight (8192 x 28672 bf16, 4.0 bpp) on the device
     (`hip_encode.encode`, kernels `ep_hip_encode_*`), whole call with its host synchronisations, then kernel by kernel
@@ -1070,7 +1015,7 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "store_pattern", "encode", "tile_ans_encode"])
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "encode", "tile_ans_encode"])
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
@@ -1094,8 +1039,6 @@ def main():
         return lossless_workload(args, ep)
     if args.workload == "gemm":
         return gemm_workload(args, ep)
-    if args.workload == "store_pattern":
-        return store_pattern_workload(args, ep)
     if args.workload == "encode":
         return encode_workload(args, ep)
     if args.workload == "tile_ans_encode":

@@ -6,10 +6,11 @@ a 1-D uint8 blob) of the reference layers (entropack/linear/linear.py:18-230, 24
 the change of hardware forces:
 
   * decoding selects the `hip` backend (the reference hard-codes "cuda", linear.py:15,58-68); encoding, which the
-    reference also runs on its CUDA lane, runs on this package's CPU encoder;
+    reference also runs on its CUDA lane, runs on this package's device encoder for a weight that is on the GPU and
+    on its CPU encoder for a weight that is on the host;
   * `forward` has two modes. "decode_then_gemm" materialises the dense weight with the decode kernel and multiplies
     with the library GEMM, exactly the reference's data flow. "fused" picks by the number of activation rows
-    (`linear/fused.py`): for one row (up to four on weights whose decode is chain-bound) the decode kernel multiplies
+    (`linear/fused.py`): for one row (up to four on weights large enough that their decode is bound by throughput) the decode kernel multiplies
     in registers and the dense weight is never written; beyond that the weight is decoded to memory once and
     multiplied by the split-K skinny product (up to 128 rows) or a tiled matrix-core product;
   * the W8A8 layer gates on a gfx950 device instead of a CUDA compute capability (linear.py:324-336) and its int8

@@ -9,6 +9,7 @@ by the data pointers it was built from (cuda.py:697-741); the tables themselves 
 There is no CPU path in this module and no fallback: a missing library or device raises.
 """
 import ctypes
+import weakref
 from dataclasses import dataclass
 
 import numpy as np
@@ -116,7 +117,11 @@ def _checked_geometry(buffers: LatticeBuffers, shape, dtype):
 class _PreparedDecode:
     """Everything one container's decode call needs except the output and the stream, checked once and kept on the
     container's `layout` tensor: the second and later decodes of a container skip the geometry checks, the plan lookup
-    and the conversion of a dozen arguments (which together cost more host time than a small layer's kernel runs)."""
+    and the conversion of a dozen arguments (which together cost more host time than a small layer's kernel runs).
+
+    The object lives on the `layout` tensor, so it refers to the container's tensors weakly: a strong reference would
+    close a cycle (layout -> cache -> prepared call -> layout) and a dropped container would keep its device memory until
+    the cycle collector runs."""
 
     __slots__ = ("tensors", "pointers", "shape", "dtype", "out_dtype", "via_float32", "rows", "cols", "device", "index",
                  "plan", "call", "head", "tail")
@@ -126,7 +131,7 @@ class _PreparedDecode:
         device = buffers.payload.device
         with torch.cuda.device(device):
             plan = _plan_for(buffers, info)
-        self.tensors = tuple(buffers)
+        self.tensors = tuple(weakref.ref(tensor) for tensor in buffers)
         self.pointers = tuple(tensor.data_ptr() for tensor in buffers)
         self.shape, self.dtype, self.out_dtype, self.via_float32 = tuple(shape), dtype, out_dtype, via_float32
         self.rows, self.cols = info["rows"], info["cols"]
@@ -141,7 +146,7 @@ class _PreparedDecode:
     def serves(self, buffers: LatticeBuffers, shape, dtype) -> bool:
         """The same tensor objects at the same addresses, with the plan still theirs."""
         for tensor, held, address in zip(buffers, self.tensors, self.pointers):
-            if tensor is not held or tensor.data_ptr() != address:
+            if held() is not tensor or tensor.data_ptr() != address:
                 return False
         return getattr(buffers.layout, "_lattice_rans_hip_plan", None) is self.plan and self.plan.key[3] == FORCE_TABLE_KIND
 

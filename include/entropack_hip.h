@@ -344,17 +344,6 @@ int ep_hip_tile_ans_encode(const uint8_t* bytes_dev, int64_t num_elements, int n
                            const uint64_t* entries_dev, const uint8_t* lane_raw_host, uint32_t* states_dev, uint32_t* stream_words_dev,
                            uint16_t* scratch_dev, int64_t scratch_stride_words, int32_t* error_dev, void* stream);
 
-/* Measurement aid --------------------------------------------------------------------------------------------- */
-
-/* Writes `vectors` 16-byte vectors to `out_dev` (16-byte aligned) in the order and shape a bf16 lattice decode of tiles
- * of `tile_vectors` vectors writes them (one tile per 32-lane half of a persistent grid, top-down in groups of 32
- * vectors, 16 bytes per lane), with streaming stores like the decode kernels (`through_cache` 0), plain ones (1), or
- * streaming ones whose lanes in front of a group's first 64-byte boundary wait a turn and go out with the group below, so
- * that every store instruction covers whole 64-byte lines (2), and decodes nothing: the time of this launch is what the
- * decode kernels' output side costs on its own.
- * No counterpart in the reference; `bench.py --workload store_pattern` is its caller. */
-int ep_hip_probe_store_pattern(void* out_dev, int64_t vectors, int tile_vectors, int through_cache, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -382,3 +382,38 @@ def test_hip_lane_refuses_tile_sizes_the_c_abi_would_truncate():
     for bad in (2 ** 31, 2 ** 32 + 16384, 2 ** 40):
         with pytest.raises(ValueError, match="tile_elements"):
             lane._check_abi_ranges({"tile_elements": bad})
+
+
+def test_prepared_decode_cache_keeps_no_container_alive(monkeypatch):
+    """The hip lane caches a prepared call on the container's `layout` tensor. The cache must refer to the container's
+    tensors weakly: dropping the container frees its payload by reference count alone, with no cycle-collector pass."""
+    import contextlib
+    import gc
+    import types
+    import weakref
+
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+
+    torch.manual_seed(0)
+    container = ep.compress((torch.randn(32, 64) * 0.02).to(torch.bfloat16), ep.EntroPackLossyConfig(target_bpp=4.0, execution_backend="eager"))
+    buffers = fmt.LatticeBuffers(**{key: container.buffers[key].clone() for key in fmt.LatticeBuffers._fields})
+    info = fmt.decode_geometry(buffers._asdict(), (32, 64))
+    plan = hip_lane.DecodePlan(desc=hip_backend.PlanDesc(), tables=torch.zeros(256, dtype=torch.uint8), error=torch.zeros(1, dtype=torch.int32),
+                               key=(0, 0, None, None))
+    monkeypatch.setattr(hip_lane, "_checked_geometry", lambda *a: (info, torch.bfloat16, False))
+    monkeypatch.setattr(hip_lane, "_plan_for", lambda *a: plan)
+    monkeypatch.setattr(hip_lane._hip, "library", lambda: types.SimpleNamespace(ep_hip_decode_lattice=None))
+    monkeypatch.setattr(torch.cuda, "device", lambda device: contextlib.nullcontext())
+    monkeypatch.setattr(torch.cuda, "current_device", lambda: 0)
+
+    prepared = hip_lane._PreparedDecode(buffers, (32, 64), torch.bfloat16)
+    buffers.layout._lattice_rans_hip_calls = {(torch.bfloat16, (32, 64)): prepared}
+    buffers.layout._lattice_rans_hip_plan = plan
+    assert prepared.serves(buffers, (32, 64), torch.bfloat16)
+    watched = [weakref.ref(tensor) for tensor in buffers]
+    gc.disable()
+    try:
+        del buffers, prepared
+        assert all(ref() is None for ref in watched)
+    finally:
+        gc.enable()

@@ -220,23 +220,3 @@ def test_full_size_target_8192x28672():
         assert hip_lane.launch_table_kind(lattice, shape=(8192, 28672), dtype=torch.bfloat16) == expected
         del first, second, on_gpu, container
         torch.cuda.empty_cache()
-
-
-@pytest.mark.parametrize("vectors, tile_vectors", [(1, 1), (31, 455), (4096, 455), (100_000, 1820), (65_537, 912)])
-def test_store_pattern_probe_writes_every_vector_once(vectors, tile_vectors):
-    """The measurement aid of bench.py --workload store_pattern: every vector of the buffer, and nothing beyond it, gets
-    the (tile, offset in the tile, lane) that a decode of such tiles would have written it from."""
-    library = hip_backend.library()
-    for through_cache in (0, 1, 2):
-        out = torch.full((vectors + 8, 4), -1, dtype=torch.int32, device="cuda")
-        status = library.ep_hip_probe_store_pattern(out.data_ptr(), vectors, tile_vectors, through_cache, torch.cuda.current_stream().cuda_stream)
-        assert status == hip_backend.OK
-        torch.cuda.synchronize()
-        got = out.cpu().numpy()
-        index = np.arange(vectors)
-        within = index % tile_vectors
-        assert np.array_equal(got[:vectors, 0], index // tile_vectors)
-        assert np.array_equal(got[:vectors, 1], within - within % 32)
-        assert np.array_equal(got[:vectors, 2], within % 32)
-        assert np.all(got[:vectors, 3] == 0) and np.all(got[vectors:] == -1)
-    assert library.ep_hip_probe_store_pattern(None, 8, 8, 0, None) == hip_backend.EINVAL
