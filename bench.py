@@ -185,7 +185,10 @@ def linear_section(ep, steps):
     reference = None
     # `fused_own_gemm` = the fused mode made to multiply with this library's tiled kernel instead of the vendor library's
     # (fused.TILED_PRODUCT = "own"); the mode's default is the faster of the two on a freshly decoded weight.
-    variants = (("decode_then_gemm", "decode_then_gemm", "library"), ("fused", "fused", "library"), ("fused_own_gemm", "fused", "own"))
+    # `fused_through_lds` = the one kernel in which the matrix cores multiply decoded tiles taken from LDS (the dense weight is
+    # never written); selected by name only, because it is the slower one.
+    variants = (("decode_then_gemm", "decode_then_gemm", "library"), ("fused", "fused", "library"), ("fused_own_gemm", "fused", "own"),
+                ("fused_through_lds", "fused_through_lds", "library"))
     for name, mode, product in variants:
         layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
         fused_mode.TILED_PRODUCT = product
@@ -224,6 +227,12 @@ def linear_section(ep, steps):
         ms = _median_ms(lambda: layer(x), steps)
         out["smaller_tiles"][f"tile_elements={tile_elements}"] = {
             "stored_bits_per_weight": round(layer.compressed_bits, 3), "decode_ms": round(_median_ms(lambda: layer.dequantize("cuda"), steps), 5),
+            "ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2), "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5),
+            "rel_l2_vs_f32_reference": ((y.double() - own).norm() / own.norm()).item()}
+        layer.forward_mode = "fused_through_lds"
+        y = layer(x)
+        ms = _median_ms(lambda: layer(x), steps)
+        out["smaller_tiles"][f"tile_elements={tile_elements}"]["fused_through_lds"] = {
             "ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 2), "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_BF16_TFLOPS, 5),
             "rel_l2_vs_f32_reference": ((y.double() - own).norm() / own.norm()).item()}
     # The same layer with its weight stored losslessly (tile_ans, the scheme a layer takes when given no config).
@@ -387,7 +396,8 @@ def small_m_section(ep, on_gpu, rows, cols, bpp, steps):
     dense_bytes = rows * cols * 2
     out = {"workload": f"CompressedLinear {rows}x{cols} @ {bpp} bpp, X [M, {cols}] bf16 N(0,1), seed 4"}
     layers = {}
-    for mode in ("decode_then_gemm", "fused"):
+    modes = ("decode_then_gemm", "fused") + (("fused_through_lds",) if bpp <= 7.0 else ())      # prob_bits 12 has no two-level tables
+    for mode in modes:
         layer = ep.CompressedLinear(cols, rows, bias=False, device="cuda", dtype=torch.bfloat16, forward_mode=mode)
         layer.weight = torch.nn.Parameter(on_gpu, requires_grad=False)
         layers[mode] = layer
@@ -402,7 +412,7 @@ def small_m_section(ep, on_gpu, rows, cols, bpp, steps):
             rel = ((y.double() - reference).norm() / reference.norm()).item()
             ms = _median_ms(lambda: layer(x), max(5, steps // 2), warmup=2)
             moved = compressed_bytes + 2 * m * cols + 2 * m * rows
-            if mode == "decode_then_gemm" or m > 4:
+            if mode == "decode_then_gemm" or (mode == "fused" and m > 4):
                 moved += 2 * dense_bytes
             entry[mode] = {"ms": round(ms, 5), "GBps_on_bytes_moved": round(moved / ms / 1e6, 1),
                            "tflops": round(2.0 * m * rows * cols / ms / 1e9, 3), "rel_l2_vs_f64_reference": rel}
@@ -511,7 +521,7 @@ def stack_workload(args, ep):
     return 0 if parity_holds(result) else 1
 
 
-def decode_case(ep, name, steps, warmup, check):
+def decode_case(ep, name, steps, warmup, check, small_m=False):
     """One decode-only configuration (a row of `decode_configs`): encode on the host, decode on the device, time the
     launches with HIP events, compare the result with the C oracle bit for bit."""
     from entropack_amd.schemes.lattice_rans import hip as hip_lane
@@ -539,18 +549,45 @@ def decode_case(ep, name, steps, warmup, check):
     last.record()
     torch.cuda.synchronize()
     avg_ms = first.elapsed_time(last) / steps
+    # The same launches rotating through device copies of the container (see main()).
+    copies = max(2, -(-ROTATING_INPUT_BYTES // max(1, alg_bytes - 2 * rows * cols_padded)))
+    rotating = [lattice] + [LatticeBuffers(**{key: one.buffers[key] for key in LatticeBuffers._fields})
+                            for one in (container.to("cuda") for _ in range(min(copies, 48) - 1))]
+    turn = [0]
+
+    def rotating_step():
+        turn[0] = (turn[0] + 1) % len(rotating)
+        return hip_lane.decode(rotating[turn[0]], shape=(rows, cols), dtype=torch.bfloat16)
+
+    for _ in rotating:
+        rotating_step()
+    settle(rotating_step)
+    torch.cuda.synchronize()
+    first.record()
+    for _ in range(steps):
+        rotating_step()
+    last.record()
+    torch.cuda.synchronize()
+    rotating_ms = first.elapsed_time(last) / steps
+    del rotating
     entry = {
         "workload": f"{rows}x{cols} N(0,{sigma}) seed {seed}{' +0.1% x20 outliers' if outliers else ''} @ {bpp} bpp -> bf16",
         "tiles": int(lattice.states.shape[0]), "prob_bits": int(container.buffers["layout"][1]),
         "table_kind": hip_lane.launch_table_kind(lattice, shape=(rows, cols), dtype=torch.bfloat16),
         "algorithmic_bytes": alg_bytes, "kernel_ms_avg": round(avg_ms, 5), "GBps": round(alg_bytes / avg_ms / 1e6, 1),
         "frac_of_hbm_peak": round(alg_bytes / avg_ms / 1e6 / HBM_PEAK_GBPS, 5), "params_per_s": round(rows * cols / (avg_ms * 1e-3), 1),
+        "kernel_ms_avg_rotating_inputs": round(rotating_ms, 5),
+        "frac_of_hbm_peak_rotating_inputs": round(alg_bytes / rotating_ms / 1e6 / HBM_PEAK_GBPS, 5),
     }
     if check:
         from oracle import c_oracle
         c_oracle.load()
         expect = c_oracle.decode(host_arrays(container.buffers), (rows, cols_padded), "bfloat16", threads=min(16, os.cpu_count() or 1))
         entry["bit_exact_vs_oracle"] = bool(np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), expect[:, :cols]))
+        del expect
+    del dense
+    if small_m:
+        entry["linear_small_m"] = small_m_section(ep, on_gpu, rows, cols, bpp, steps)
     return entry
 
 
@@ -1059,15 +1096,30 @@ def main():
     cols_padded = int(container.buffers["layout"][0])
     alg_bytes = algorithmic_bytes(container.buffers, rows, cols_padded, 2)
 
+    # Every launch of the timed region reads its container from memory, as a model that decodes each layer once per
+    # forward does: the steps rotate through enough device copies of the container that none of them is still in the
+    # card's 256 MB last-level cache when its turn comes again. (One container decoded over and over keeps its compressed
+    # bytes there; that figure is reported beside, as `same_container`.)
+    copies = max(2, -(-ROTATING_INPUT_BYTES // max(1, alg_bytes - 2 * rows * cols_padded)))
+    rotation = [on_gpu] + [container.to(device) for _ in range(copies - 1)]
+    rotating = [LatticeBuffers(**{key: one.buffers[key] for key in LatticeBuffers._fields}) for one in rotation]
+    turn = [0]
+
     def step():
+        turn[0] = (turn[0] + 1) % len(rotating)
+        return hip_lane.decode(rotating[turn[0]], shape=(rows, cols), dtype=torch.bfloat16)
+
+    def same_container_step():
         return hip_lane.decode(lattice, shape=(rows, cols), dtype=torch.bfloat16)
 
     copy_probe(args, device)
 
     # From idle first (the device has done nothing while the host encoded): `warmup` + `steps` launches as they come.
-    dense = step()                                    # builds the plan
+    for _ in rotating:
+        dense = step()                                # builds the plans
     torch.cuda.synchronize()
-    hip_lane.check_errors(lattice)
+    for one in rotating:
+        hip_lane.check_errors(one)
     time.sleep(0.2)
     for _ in range(max(args.warmup, 1)):
         dense = step()
@@ -1083,7 +1135,6 @@ def main():
     for _ in range(max(args.warmup, 1)):
         dense = step()
     torch.cuda.synchronize()
-    hip_lane.check_errors(lattice)
 
     # The timed region: exactly `steps` launches back to back between two synchronisations, with one pair of HIP events
     # on the launch stream around all of them (average launch duration = their distance / steps; events between the
@@ -1107,33 +1158,22 @@ def main():
         end.record()
     torch.cuda.synchronize()
     kernel_ms = sorted(begin.elapsed_time(end) for begin, end in events)
-
-    # The same container over and over keeps its compressed bytes in the card's 256 MB last-level cache between launches,
-    # which a container that is decoded once (a model being loaded) does not have: the same launches again, rotating
-    # through enough device copies of the container that every one comes from memory.
-    copies = max(2, -(-ROTATING_INPUT_BYTES // max(1, alg_bytes - 2 * rows * cols_padded)))
-    rotation = [on_gpu] + [container.to(device) for _ in range(copies - 1)]
-    rotating = [LatticeBuffers(**{key: one.buffers[key] for key in LatticeBuffers._fields}) for one in rotation]
-    turn = [0]
-
-    def rotating_step():
-        turn[0] = (turn[0] + 1) % len(rotating)
-        return hip_lane.decode(rotating[turn[0]], shape=(rows, cols), dtype=torch.bfloat16)
-
-    for _ in rotating:
-        rotating_step()                               # builds the copies' plans
-    settle(rotating_step)
-    torch.cuda.synchronize()
-    first_rotating, last_rotating = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    first_rotating.record()
-    for _ in range(args.steps):
-        rotating_step()
-    last_rotating.record()
-    torch.cuda.synchronize()
-    rotating_ms = first_rotating.elapsed_time(last_rotating) / args.steps
     for one in rotating:
         hip_lane.check_errors(one)
+    dense = same_container_step()                     # the tensor the oracle check below compares
     del rotation, rotating
+
+    # The same launches on one container over and over: its compressed bytes stay in the last-level cache.
+    settle(same_container_step)
+    torch.cuda.synchronize()
+    first_same, last_same = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    first_same.record()
+    for _ in range(args.steps):
+        same_container_step()
+    last_same.record()
+    torch.cuda.synchronize()
+    same_ms = first_same.elapsed_time(last_same) / args.steps
+    hip_lane.check_errors(lattice)
 
     result = {
         "metric": "lossy decode GB/s (+% HBM roofline); CompressedLinear TFLOPS @ M=4096, 4 bpp",
@@ -1158,10 +1198,10 @@ def main():
             "kernel_ms_min": round(kernel_ms[0], 5),
             "kernel_ms_avg_from_idle": round(from_idle_ms, 5),
             "frac_from_idle": round(alg_bytes / (from_idle_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
-            "kernel_ms_avg_rotating_inputs": round(rotating_ms, 5),
-            "frac_rotating_inputs": round(alg_bytes / (rotating_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
-            "inputs": f"kernel_ms_avg: the same container every launch (its compressed bytes stay in the 256 MB last-level cache); "
-                      f"rotating inputs: {copies} device copies of it in turn, so that each launch reads its container from memory",
+            "kernel_ms_avg_same_container": round(same_ms, 5),
+            "frac_same_container": round(alg_bytes / (same_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
+            "inputs": f"timed region: {copies} device copies of the container in turn, so that each launch reads its container "
+                      f"from memory; same_container: one container every launch (its compressed bytes stay in the 256 MB last-level cache)",
             "clocks": f"settled: {SETTLE_SECONDS} s of untimed launches of the same kernel before the warm-up steps; "
                       f"from idle = the first {args.warmup} + {args.steps} launches after 0.2 s without work",
         },
@@ -1190,7 +1230,8 @@ def main():
         torch.cuda.empty_cache()
         configs = {}
         for name in ("c2", "c5a", "c5b"):
-            configs[name] = decode_case(ep, name, max(10, args.steps // 2), args.warmup, not args.no_cpu)
+            configs[name] = decode_case(ep, name, max(10, args.steps // 2), args.warmup, not args.no_cpu,
+                                        small_m=name in ("c5a", "c5b") and not args.no_linear)
             torch.cuda.empty_cache()
         configs["c4"] = stack_case(ep, args.steps, not args.no_cpu)
         result["decode_configs"] = configs

@@ -60,6 +60,15 @@ class DecodeJob(ctypes.Structure):
     ]
 
 
+FUSED_SLOTS = 32                    # EP_HIP_FUSED_SLOTS
+
+
+class FusedBatch(ctypes.Structure):
+    """ep_hip_fused_batch: up to 32 tiles whose chains stay aligned in k (decode-to-GEMM through LDS)."""
+    _fields_ = [("base", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3), ("tile", ctypes.c_int32 * FUSED_SLOTS),
+                ("delta", ctypes.c_int32 * FUSED_SLOTS)]
+
+
 class HipError(RuntimeError):
     """A C-ABI call returned a non-zero status."""
 
@@ -95,6 +104,11 @@ _SIGNATURES = {
     "ep_hip_linear_fused_bf16_static": (ctypes.c_int, [
         ctypes.POINTER(DecodeJob), ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
         ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
+    "ep_hip_fused_plan": (ctypes.c_int, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]),
+    "ep_hip_linear_fused_mfma_bf16": (ctypes.c_int, [
+        ctypes.POINTER(DecodeJob), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
+    "ep_hip_linear_fused_mfma_workspace": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int64]),
     "ep_hip_gemm_bf16": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
         ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),

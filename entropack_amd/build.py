@@ -11,7 +11,7 @@ PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PACKAGE_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PACKAGE_DIR), "include")
 HIP_LIBRARY = os.path.join(PACKAGE_DIR, "libentropack_hip.so")
-HIP_SOURCES = ("ep_plan.hip", "ep_decode.hip", "ep_decode_lds.hip", "ep_decode_rank.hip", "ep_decode_dot.hip", "ep_decode_sym.hip", "ep_tile_ans.hip", "ep_linear.hip", "ep_encode.hip")
+HIP_SOURCES = ("ep_plan.hip", "ep_decode.hip", "ep_decode_lds.hip", "ep_decode_rank.hip", "ep_decode_dot.hip", "ep_decode_sym.hip", "ep_decode_mfma.hip", "ep_tile_ans.hip", "ep_linear.hip", "ep_encode.hip")
 HOST_LIBRARY = os.path.join(PACKAGE_DIR, "libentropack_host.so")
 HOST_SOURCES = ("host_codec.c",)
 HOST_FLAGS = ("-O2", "-std=c11", "-fPIC", "-shared", "-fopenmp", "-ffp-contract=off", "-Wall", "-Wextra")

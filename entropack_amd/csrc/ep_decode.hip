@@ -517,3 +517,33 @@ extern "C" int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, 
   if (status != EP_HIP_OK) return status;
   return linear_fused_bf16(weight, x_dev, m_rows, ldx, bias_dev, y_dev, ldy, out_kind, accumulator, static_cast<hipStream_t>(stream));
 }
+
+extern "C" int ep_hip_linear_fused_mfma_bf16(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
+                                             const void* x_dev, int64_t m_rows, int64_t ldx, const void* bias_dev, void* y_dev,
+                                             int64_t ldy, int out_kind, float* workspace_dev, void* stream) {
+  using namespace ep;
+  if (weight == nullptr || batches_dev == nullptr || x_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
+  if (out_kind < EP_FLOAT_BF16 || out_kind > EP_FLOAT_F32 || m_rows <= 0 || n_batches <= 0 || weight->desc == nullptr) return EP_HIP_EINVAL;
+  const int64_t outer = weight->rows, inner = weight->cols_padded;
+  if (ldx < inner || ldy < outer || reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || ldx % 8 != 0) return EP_HIP_EINVAL;
+  if (m_rows > 0x7FFFFFFF || weight->store_kind != EP_STORE_BF16 || weight->desc->table_kind == EP_TABLE_GLOBAL64) return EP_HIP_EUNSUPPORTED;
+  DecodeArgs args;
+  int pairs = 0;
+  const int status = fill_decode_args(weight->payload_dev, weight->payload_words, weight->offsets_dev, weight->states_dev, weight->scales_dev,
+                                      weight->tables_dev, weight->desc, nullptr, weight->store_kind, weight->rows, weight->cols_padded,
+                                      weight->tile_elements, weight->error_dev, args, pairs);
+  if (status != EP_HIP_OK) return status;
+  // The kernel takes nothing in the batch table on trust (tile indices, shifts and bases are range-checked there), so a
+  // stale table yields an error code or wrong sums, never an access outside the buffers.
+  if (n_batches > args.num_tiles || reinterpret_cast<uintptr_t>(workspace_dev) % 256 != 0) return EP_HIP_EINVAL;
+  args.m_rows = static_cast<int>(m_rows);
+  args.x = static_cast<const uint16_t*>(x_dev);
+  args.ldx = ldx;
+  args.y32 = workspace_dev;
+  return launch_fused_mfma(args, *weight->desc, batches_dev, n_batches, bias_dev, y_dev, ldy, out_kind, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t ep_hip_linear_fused_mfma_workspace(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows) {
+  if (rows <= 0 || cols_padded < 8 || tile_elements <= 0 || m_rows <= 0) return 0;
+  return ep::fused_workspace_bytes(rows, cols_padded, tile_elements, m_rows);
+}

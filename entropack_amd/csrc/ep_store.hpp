@@ -267,5 +267,9 @@ int launch_sym(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, cons
 // the launch is larger than one pass of resident waves (where occupancy, not the length of a step, sets the pace).
 int effective_table_kind(const ep_hip_plan_desc& desc, int kind, int64_t pairs, int cus);
 int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int kind, int num_pairs, hipStream_t stream);
+// Decode-to-GEMM through LDS (ep_decode_mfma.hip): args.x / m_rows / y32 set, one workgroup per batch and block of rows.
+int launch_fused_mfma(DecodeArgs args, const ep_hip_plan_desc& desc, const ep_hip_fused_batch* batches, int n_batches, const void* bias, void* y,
+                      int64_t ldy, int out_kind, hipStream_t stream);
+size_t fused_workspace_bytes(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows);
 
 }  // namespace ep

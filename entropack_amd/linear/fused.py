@@ -1,4 +1,6 @@
-"""`forward_mode="fused"` of the compressed linear layers: what runs for how many activation rows.
+"""`forward_mode="fused"` and `"fused_through_lds"` of the compressed linear layers: what runs for how many activation rows.
+
+"fused":
 
   rows M            weight written to memory?   kernels
   1 (and 2..4 on    no                          the decode kernel multiplies every decoded vector with the activations in
@@ -12,13 +14,24 @@
                                                 (`TILED_PRODUCT = "library"`, the default) or this package's
                                                 (`"own"`, `ep_hip_gemm_bf16`)
 
-Beyond four rows nothing is multiplied inside the decode kernel: a tile is a chain of dependent rANS steps that lasts
-as long whatever is fused behind it, a wave's two tiles hold unrelated (row, k) ranges that form no matrix-core operand,
-and the vector ALU, which the decode saturates, would have to do the multiplying. The default for the tiled product is
-the library because its kernel is the faster one wherever the weight has just been decoded, i.e. is not in any cache:
-3072 x 3072 weight, 256 / 1024 / 4096 rows: 20 / 31 / 63 us against 46 / 46 / 67 us for this package's kernel, which
-keeps less than one K step of loads in flight (with both operands cache-resident the two are within 5 % of each
-other at 4096 rows). The reference has one path for every M: decode, then `F.linear` (entropack/linear/linear.py:163-165).
+"fused_through_lds": any M, weight never written. One kernel (`ep_hip_linear_fused_mfma_bf16`) in which every workgroup
+decodes 32 tiles whose chains stay aligned in k, passes each group of decoded vectors through an LDS ring and multiplies
+them on the matrix cores (`v_mfma_f32_32x32x16_bf16`) with activations it streams from memory; containers it cannot take
+(no two-level tables: prob_bits 12 and up, alphabets beyond a byte; rows of an odd number of vectors) fall through to
+"fused". It is correct to the same tolerance and slower than "fused" everywhere it was measured (MI355X, kernel times):
+3072 x 3072 @ 4 bpp, M = 16 / 256 / 4096: 129 / 184 / 447 us (+ 11-53 us for its two small helper kernels) against 90 /
+92 / 130 us for decode + product. The reasons are the format's, not the kernel's: a tile yields 32 vectors per chain of
+nine dependent steps whatever is fused behind it, so a workgroup's operand is 32 weight rows wide per 256 k and every
+activation byte it loads meets only 32 weight rows (a tiled GEMM reuses it 192-256 times: 2.4 GB of activation traffic
+from L2 at M = 4096 where the GEMM needs 0.7 GB); gathering 32 aligned tiles on one compute unit puts four chains on every
+SIMD, which lengthens each chain step from 138 to 219 ns; and for M > 256 the same tiles are decoded once per block of
+256 activation rows. It stays in the package as the built and measured form of the idea, selected only by name.
+
+The default for the tiled product is the library because its kernel is the faster one wherever the weight has just been
+decoded, i.e. is not in any cache: 3072 x 3072 weight, 256 / 1024 / 4096 rows: 20 / 31 / 63 us against 46 / 46 / 67 us for
+this package's kernel, which keeps less than one K step of loads in flight (with both operands cache-resident the two
+are within 5 % of each other at 4096 rows). The reference has one path for every M: decode, then `F.linear`
+(entropack/linear/linear.py:163-165).
 
 The forward is differentiable with respect to the activations (like the reference's `F.linear` on a constant weight):
 under autograd the kernels run inside a `torch.autograd.Function` whose backward multiplies the output gradient with
@@ -41,6 +54,8 @@ def _forward_kernels(layer, x: torch.Tensor) -> torch.Tensor:
     if container.compress_method == "lattice_rans" and container.encoded_dtype == torch.bfloat16:
         on_device = container.to(device=x.device)
         buffers = packed_buffers(on_device.buffers, LatticeBuffers)
+        if layer.forward_mode == "fused_through_lds" and hip_lane.mfma_linear_usable(buffers, tuple(container.shape), x):
+            return hip_lane.linear_mfma(buffers, shape=tuple(container.shape), x=x, bias=layer._bias_on(x.device))
         if hip_lane.fused_linear_pays(buffers, tuple(container.shape), x):
             return hip_lane.linear_rows(buffers, shape=tuple(container.shape), x=x, bias=layer._bias_on(x.device))
     weight = layer._decoded_for(x)

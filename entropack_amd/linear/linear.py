@@ -12,7 +12,10 @@ the change of hardware forces:
     with the library GEMM, exactly the reference's data flow. "fused" picks by the number of activation rows
     (`linear/fused.py`): for one row (up to four on weights large enough that their decode is bound by throughput) the decode kernel multiplies
     in registers and the dense weight is never written; beyond that the weight is decoded to memory once and
-    multiplied by the split-K skinny product (up to 128 rows) or a tiled matrix-core product;
+    multiplied by the split-K skinny product (up to 128 rows) or a tiled matrix-core product. "fused_through_lds" is the
+    one kernel for any number of rows in which the matrix cores multiply decoded tiles taken from LDS (the weight is
+    never written either); it is slower than "fused" on every shape measured and exists as the measured answer to
+    "why not fuse decode and GEMM" (`linear/fused.py`);
   * the W8A8 layer gates on a gfx950 device instead of a CUDA compute capability (linear.py:324-336) and its int8
     GEMM + row quantiser are HIP kernels with the semantics of the reference's Triton kernels
     (entropack/linear/quant_kernels.py:15-79).
@@ -35,7 +38,7 @@ QUANT_STATE_LEAF = "entropack_quant_state"      # state_dict key suffix of a com
 #: device lane for both directions, linear.py:15,59-68), the CPU lane for a weight on the CPU.
 ENCODE_BACKEND_BY_DEVICE = {"cuda": "hip", "cpu": "eager"}
 DECODE_BACKEND = "hip"
-FORWARD_MODES = ("decode_then_gemm", "fused")
+FORWARD_MODES = ("decode_then_gemm", "fused", "fused_through_lds")
 _F32_EPS = torch.finfo(torch.float32).eps
 
 
@@ -47,7 +50,7 @@ class CompressedLinear(torch.nn.Linear):
         config: compression config; None picks a scheme by dtype.
         device: device of the bias; the compressed buffers stay where the source weight was.
         dtype: container dtype the weight is compressed in.
-        forward_mode: "decode_then_gemm" (default) or "fused".
+        forward_mode: "decode_then_gemm" (default), "fused", or "fused_through_lds" (see `linear/fused.py`).
     """
 
     state_buffer_names: ClassVar[tuple[str, ...]] = ()
@@ -183,7 +186,7 @@ class CompressedLinear(torch.nn.Linear):
         return None if self.bias is None else self.bias.to(device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if self.forward_mode == "fused":
+        if self.forward_mode != "decode_then_gemm":
             from . import fused
             return fused.linear_forward(self, x)
         return F.linear(x, self._decoded_for(x).to(x.dtype), self._bias_on(x.device))

@@ -254,6 +254,67 @@ def linear_rows(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.
     return out.reshape(*x.shape[:-1], outer)
 
 
+def fused_batches(buffers: LatticeBuffers, info: dict) -> tuple[torch.Tensor, int, int]:
+    """(device table of ep_hip_fused_batch, number of batches, number of tiles) for decode-to-GEMM through LDS, built once
+    per container and kept on its `layout` tensor: ep_hip_fused_plan groups the tiles whose chains stay aligned in k."""
+    device = buffers.payload.device
+    key = (info["rows"], info["cols"], info["tile_elements"], device)
+    cached = getattr(buffers.layout, "_lattice_rans_hip_fused_batches", None)
+    if cached is not None and cached[0] == key:
+        return cached[1:]
+    lib = _hip.library()
+    count = ctypes.c_int(0)
+    _hip.check("ep_hip_fused_plan", lib.ep_hip_fused_plan(info["rows"], info["cols"], info["tile_elements"], None, 0, ctypes.byref(count)))
+    host = torch.zeros(count.value * ctypes.sizeof(_hip.FusedBatch), dtype=torch.uint8)
+    _hip.check("ep_hip_fused_plan", lib.ep_hip_fused_plan(info["rows"], info["cols"], info["tile_elements"], host.data_ptr(), count.value,
+                                                          ctypes.byref(count)))
+    table = host.to(device)
+    buffers.layout._lattice_rans_hip_fused_batches = (key, table, count.value, info["total_tiles"])
+    return table, count.value, info["total_tiles"]
+
+
+def mfma_linear_usable(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
+    """Can `linear_mfma` take this container and activation? bf16 activations, weight rows of a multiple of 16 and at least
+    256 columns, and a plan with the two-level tables of prob_bits 11 (what the default encoder settings give up to 7 bpp)."""
+    if not (x.dtype == torch.bfloat16 and x.numel() > 0 and shape[1] % 16 == 0 and shape[1] >= 256 and x.shape[-1] == shape[1]
+            and buffers.payload.device.type == "cuda"):
+        return False
+    info, _, _ = _checked_geometry(buffers, shape, torch.bfloat16)
+    with torch.cuda.device(buffers.payload.device):
+        plan = _plan_for(buffers, info)
+    return plan.desc.prob_bits == 11 and plan.desc.sym_offset != 0 and plan.desc.table_kind in (_hip.TABLE_LDS_BYTE, _hip.TABLE_LDS_SYM)
+
+
+def linear_mfma(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
+    """x[..., K] @ W.T (+ bias) for any number of activation rows, W = this bf16 container, the decoded weight going from the
+    rANS lanes to the matrix cores through LDS and never to memory (ep_hip_linear_fused_mfma_bf16).
+
+    The reference decodes the whole weight and calls F.linear (entropack/linear/linear.py:163-165).
+    """
+    device = buffers.payload.device
+    info, _, _ = _checked_geometry(buffers, shape, torch.bfloat16)
+    if not mfma_linear_usable(buffers, shape, x):
+        raise ValueError("linear_mfma takes bfloat16 activations, weight rows of a multiple of 16 (at least 256) columns and a "
+                         "container whose plan has the two-level tables (prob_bits 11, byte-valued symbols)")
+    flat = x.reshape(-1, x.shape[-1])
+    if flat.stride(-1) != 1 or flat.stride(0) % 8 or flat.data_ptr() % 16:
+        flat = flat.contiguous()
+    outer = info["rows"]
+    with torch.cuda.device(device):
+        plan = _plan_for(buffers, info)
+        table, batches, _ = fused_batches(buffers, info)
+        job = _job_of(buffers, info, plan, _hip.STORE_KINDS[torch.bfloat16])
+        out = torch.empty(flat.shape[0], outer, dtype=x.dtype, device=device)
+        workspace = torch.empty(_hip.library().ep_hip_linear_fused_mfma_workspace(outer, info["cols"], info["tile_elements"], flat.shape[0]),
+                                dtype=torch.uint8, device=device)
+        bias_ready = None if bias is None else bias.to(device=device, dtype=x.dtype).contiguous()
+        _hip.check("ep_hip_linear_fused_mfma_bf16", _hip.library().ep_hip_linear_fused_mfma_bf16(
+            ctypes.byref(job), table.data_ptr(), batches, flat.data_ptr(), flat.shape[0], flat.stride(0),
+            None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(), out.stride(0), _hip.FLOAT_KINDS[x.dtype],
+            workspace.data_ptr(), _hip.current_stream(device)))
+    return out.reshape(*x.shape[:-1], outer)
+
+
 class BatchDecoder:
     """Decodes many containers (a model's layers) in one pass: ep_hip_batch_plan / ep_hip_decode_lattice_batch.
 

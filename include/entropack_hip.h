@@ -264,6 +264,46 @@ int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev,
 int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, const void* x_dev, int64_t m_rows, int64_t ldx,
                                     const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* stream);
 
+/* Decode-to-GEMM through LDS ------------------------------------------------------------------------------------ *
+ *
+ * y[m_rows][rows] = x[m_rows][cols_padded] * W^T (+ bias) for any number of activation rows, W a compressed container,
+ * with the decoded weight handed from the rANS lanes to the matrix cores through LDS: the dense weight is never written
+ * to memory. A workgroup decodes up to EP_HIP_FUSED_SLOTS tiles whose first vectors lie at (nearly) the same position
+ * inside a weight row, because only such tiles supply many weight rows at one k, which is what a matrix-core operand is;
+ * ep_hip_fused_plan groups a container's tiles that way (host only, pure arithmetic on the geometry), the caller copies
+ * the batches to the device once per container and passes them to every product.
+ * Reference: CompressedLinear.forward / _reconstruct, entropack/linear/linear.py:125-130,163-165 (decode the whole weight,
+ * then F.linear); the reference has no fused form (its lattice_rans.cu:21-23 fuses decode, reconstruction and cast only). */
+#define EP_HIP_FUSED_SLOTS 32        /* tiles per batch: one per 32-lane half of sixteen waves */
+#define EP_HIP_FUSED_MAX_SKEW 31     /* largest distance, in vectors, between the in-row positions of a batch's tiles */
+
+typedef struct ep_hip_fused_batch {
+  int32_t base;                          /* in-row vector position (even) that aligned index 0 of this batch stands for */
+  int32_t reserved[3];
+  int32_t tile[EP_HIP_FUSED_SLOTS];      /* tile index, or -1 for an unused slot */
+  int32_t delta[EP_HIP_FUSED_SLOTS];     /* (tile * tile_vectors) mod vectors_per_row - base, 0 .. EP_HIP_FUSED_MAX_SKEW */
+} ep_hip_fused_batch;
+
+/* Groups the tiles of a rows x cols_padded container with `tile_elements` symbols per tile into batches. With
+ * batches_host NULL only counts them (*n_batches); else fills at most `capacity` batches. EP_HIP_EUNSUPPORTED for rows of
+ * fewer than 32 vectors or of an odd number of vectors (cols_padded not a multiple of 16). */
+int ep_hip_fused_plan(int64_t rows, int64_t cols_padded, int tile_elements, ep_hip_fused_batch* batches_host, int capacity,
+                      int* n_batches);
+
+/* The product. `weight` as for ep_hip_linear_fused_bf16 (store_kind EP_STORE_BF16; the decoded values are rounded to
+ * bf16 exactly as ep_hip_decode_lattice stores them); `batches_dev` = the device copy of ep_hip_fused_plan's output for
+ * the same geometry. x is bf16 with row stride `ldx` elements (a multiple of 8, 16-byte aligned base); bias (may be NULL)
+ * and y have type `out_kind`; `workspace_dev` (256-byte aligned) holds ep_hip_linear_fused_mfma_workspace(...) bytes and
+ * need not be cleared: the kernel writes every partial sum of an output (one per tile the weight row touches and half
+ * of the k steps) into a plane of its own with plain stores, and a second kernel adds them in a fixed order, then the
+ * bias, and rounds once, so results are the same from run to run. EP_HIP_EUNSUPPORTED unless the plan has the two-level
+ * tables of prob_bits 11 (byte-valued symbols), which is what the default encoder settings give up to 7 bpp: the caller
+ * then decodes and multiplies separately. */
+int ep_hip_linear_fused_mfma_bf16(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
+                                  const void* x_dev, int64_t m_rows, int64_t ldx, const void* bias_dev, void* y_dev, int64_t ldy,
+                                  int out_kind, float* workspace_dev, void* stream);
+size_t ep_hip_linear_fused_mfma_workspace(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows);
+
 /* Encoder (the step before the path) -------------------------------------------------------------------------- *
  *
  * The device form of the lattice_rans encoder, one entry point per kernel of the reference's CUDA lane. All pointers are
