@@ -148,6 +148,8 @@ static int fill_decode_args(const uint16_t* payload_dev, uint64_t payload_words,
   args.error = error_dev;
   args.lut_bytes = args.rank_val_offset = args.rank_rs_offset = args.rank_half = 0;
   args.sym_tables = nullptr;
+  args.store_cached = 0;
+  args.reserved = 0;
   args.m_rows = 0;
   args.x = nullptr;
   args.y32 = nullptr;
@@ -240,6 +242,14 @@ extern "C" int ep_hip_decode_lattice(const uint16_t* payload_dev, uint64_t paylo
   const int status = fill_decode_args(payload_dev, payload_words, offsets_dev, states_dev, scales_dev, tables_dev, desc, out_dev,
                                       store_kind, rows, cols_padded, tile_elements, error_dev, args, pairs);
   if (status != EP_HIP_OK) return status;
+  // Memory takes writes in pieces of 64 bytes = four bf16 vectors, and a group writes 32 consecutive vectors from the tile's
+  // first vector + a multiple of 32. When the tile length is no multiple of four vectors (the default tiles from 5 bpp up:
+  // 910 and 455 vectors), the piece at either end of a group is shared with the neighbouring group, which streams its part
+  // out microseconds apart; written through the cache the two parts meet in L2. With the container read from memory (a
+  // layer decoded once per forward) that is 7-8 % faster at 5, 6 and 8 bpp (8192 x 28672: 176 -> 161, 183 -> 168, 215 ->
+  // 200 us); whole tiles keep the streaming stores, which are the faster ones there (156 against 161 us at 4 bpp), and so
+  // do batches, where layers of both kinds share a launch (the 120-layer pass measured 2 % slower with mixed policies).
+  args.store_cached = store_kind == EP_STORE_BF16 && args.tile_vectors % 4 != 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (desc->table_kind == EP_TABLE_GLOBAL64) return launch_global64(args, pairs, s);
   return launch_lds_decode(args, *desc, kernel_kind_of(store_kind), pairs, s);

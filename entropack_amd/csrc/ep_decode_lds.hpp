@@ -493,6 +493,16 @@ __device__ __forceinline__ int window_pointer_b(const Pair& s) {
   return s.windowB - 64 * static_cast<int>(s.slid >> 23) + static_cast<int>(s.pos >> 16) - static_cast<int>(kPosBias);
 }
 
+// One 16-byte store of a bf16 vector, streaming or through the cache as the container's tile length asks. Written as
+// two instructions the compiler cannot merge: given two ordinary stores of one value to one address on the two sides of
+// a branch it keeps a single store and drops the streaming hint. (A store the compiler does not know about only makes
+// its later waits on the memory counter stricter.)
+typedef uint32_t lds_store_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_bf16_vector(lds_store_u32x4* to, lds_store_u32x4 value, bool through_cache) {
+  if (through_cache) asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(to), "v"(value) : "memory");
+  else asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(to), "v"(value) : "memory");
+}
+
 // ---- the kernel ------------------------------------------------------------------------------------------------------
 
 // A wave alternates between a chain of dependent symbol steps, where every instruction waits for the one before, and a
@@ -716,10 +726,10 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
         uint32_t packed[4];
         pack_bf16(w, scale, packed);
         // Streaming store: the dense weight is written once and not read back by this kernel, and waves must not
-        // queue behind write-allocate traffic when they next wait on their payload prefetch.
+        // queue behind write-allocate traffic when they next wait on their payload prefetch (store_cached: see below).
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
         const u32x4 quad = {packed[0], packed[1], packed[2], packed[3]};
-        __builtin_nontemporal_store(quad, reinterpret_cast<u32x4*>(a.out) + vector);
+        store_bf16_vector(reinterpret_cast<u32x4*>(a.out) + vector, quad, a.store_cached != 0);
       } else if constexpr (KIND == EP_STORE_I8) {
         store_vector_i8(a.out, vector, w);
       } else {
@@ -914,7 +924,10 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
           typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
           const u32x4 quad = {packed[0], packed[1], packed[2], packed[3]};
           uint8_t* lower_out = static_cast<uint8_t*>(a.out) + 16ull * lower_tile_of(j);
-          __builtin_nontemporal_store(quad, reinterpret_cast<u32x4*>(lower_out + at));
+          // Streaming stores, except for tiles whose length is no multiple of four vectors (store_cached): their groups
+          // share 64-byte pieces with the neighbouring groups, and pieces written through the cache meet there.
+          if (a.store_cached) asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(at), "v"(quad), "s"(lower_out) : "memory");
+          else asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(at), "v"(quad), "s"(lower_out) : "memory");
         } else if constexpr (KIND == EP_STORE_I8) {
           store_vector_i8(a.out, lower_tile_of(j) + (at >> 4), w);
         } else {

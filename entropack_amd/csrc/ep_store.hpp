@@ -27,6 +27,8 @@ struct DecodeArgs {
   uint32_t rank_rs_offset;
   uint32_t rank_half;       // LDS_RANK: the value table holds half-precision coordinates
   const uint8_t* sym_tables;   // the plan's two-level (LDS_SYM) section, or null
+  uint32_t store_cached;       // bf16 stores go through the cache instead of streaming (tiles that split 64-byte pieces between groups)
+  uint32_t reserved;
   // Multiply-on-the-fly kernels only: activations x[m_rows][ldx] (bf16) and the f32 accumulator y32[m_rows][ldy32].
   int m_rows;
   const uint16_t* x;
