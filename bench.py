@@ -261,7 +261,7 @@ def int8_linear_section(ep, steps):
     x = torch.randn(4096, 3072).to(torch.bfloat16).cuda()
     ops = 2.0 * 4096 * 3072 * 3072
     out = {"workload": "CompressedINT8Linear 3072x3072, codes @ 4.0 bpp, + bias, X [4096, 3072] bf16, seed 2", "ops": ops}
-    for mode in ("decode_then_gemm", "fused"):
+    for mode in ("decode_then_gemm", "fused", "fused_through_lds"):
         layer = ep.CompressedINT8Linear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
         y = layer(x)
         codes, (qa, sa) = layer.codes("cuda"), kernels.quantize_rows(x)

@@ -528,15 +528,20 @@ extern "C" int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, 
   return linear_fused_bf16(weight, x_dev, m_rows, ldx, bias_dev, y_dev, ldy, out_kind, accumulator, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int ep_hip_linear_fused_mfma_bf16(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
-                                             const void* x_dev, int64_t m_rows, int64_t ldx, const void* bias_dev, void* y_dev,
-                                             int64_t ldy, int out_kind, float* workspace_dev, void* stream) {
-  using namespace ep;
+namespace ep {
+
+// Shared by the two decode-to-GEMM entry points: argument checks, the kernels' argument block, the launch.
+static int linear_fused_mfma(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches, bool int8, const void* x_dev,
+                             int64_t m_rows, int64_t ldx, const float* scale_a_dev, const float* scale_b_dev, const void* bias_dev, void* y_dev,
+                             int64_t ldy, int out_kind, void* workspace_dev, hipStream_t stream) {
   if (weight == nullptr || batches_dev == nullptr || x_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
   if (out_kind < EP_FLOAT_BF16 || out_kind > EP_FLOAT_F32 || m_rows <= 0 || n_batches <= 0 || weight->desc == nullptr) return EP_HIP_EINVAL;
+  if (int8 && (scale_a_dev == nullptr || scale_b_dev == nullptr)) return EP_HIP_EINVAL;
   const int64_t outer = weight->rows, inner = weight->cols_padded;
-  if (ldx < inner || ldy < outer || reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || ldx % 8 != 0) return EP_HIP_EINVAL;
-  if (m_rows > 0x7FFFFFFF || weight->store_kind != EP_STORE_BF16 || weight->desc->table_kind == EP_TABLE_GLOBAL64) return EP_HIP_EUNSUPPORTED;
+  if (ldx < inner || ldy < outer || reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || ldx % (int8 ? 16 : 8) != 0) return EP_HIP_EINVAL;
+  if (m_rows > 0x7FFFFFFF || weight->store_kind != (int8 ? EP_STORE_I8 : EP_STORE_BF16) || weight->desc->table_kind == EP_TABLE_GLOBAL64) {
+    return EP_HIP_EUNSUPPORTED;
+  }
   DecodeArgs args;
   int pairs = 0;
   const int status = fill_decode_args(weight->payload_dev, weight->payload_words, weight->offsets_dev, weight->states_dev, weight->scales_dev,
@@ -549,11 +554,27 @@ extern "C" int ep_hip_linear_fused_mfma_bf16(const ep_hip_decode_job* weight, co
   args.m_rows = static_cast<int>(m_rows);
   args.x = static_cast<const uint16_t*>(x_dev);
   args.ldx = ldx;
-  args.y32 = workspace_dev;
-  return launch_fused_mfma(args, *weight->desc, batches_dev, n_batches, bias_dev, y_dev, ldy, out_kind, static_cast<hipStream_t>(stream));
+  args.y32 = static_cast<float*>(workspace_dev);
+  return launch_fused_mfma(args, *weight->desc, batches_dev, n_batches, int8, scale_a_dev, scale_b_dev, bias_dev, y_dev, ldy, out_kind, stream);
 }
 
-extern "C" size_t ep_hip_linear_fused_mfma_workspace(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows) {
+}  // namespace ep
+
+extern "C" int ep_hip_linear_fused_mfma_bf16(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
+                                             const void* x_dev, int64_t m_rows, int64_t ldx, const void* bias_dev, void* y_dev,
+                                             int64_t ldy, int out_kind, void* workspace_dev, void* stream) {
+  return ep::linear_fused_mfma(weight, batches_dev, n_batches, false, x_dev, m_rows, ldx, nullptr, nullptr, bias_dev, y_dev, ldy, out_kind,
+                               workspace_dev, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ep_hip_linear_fused_mfma_i8(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
+                                           const int8_t* a_dev, int64_t m_rows, int64_t lda, const float* scale_a_dev, const float* scale_b_dev,
+                                           const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* workspace_dev, void* stream) {
+  return ep::linear_fused_mfma(weight, batches_dev, n_batches, true, a_dev, m_rows, lda, scale_a_dev, scale_b_dev, bias_dev, y_dev, ldy, out_kind,
+                               workspace_dev, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t ep_hip_linear_fused_mfma_workspace(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows, int int8) {
   if (rows <= 0 || cols_padded < 8 || tile_elements <= 0 || m_rows <= 0) return 0;
-  return ep::fused_workspace_bytes(rows, cols_padded, tile_elements, m_rows);
+  return ep::fused_workspace_bytes(rows, cols_padded, tile_elements, m_rows, int8 ? 1 : 2);
 }

@@ -34,15 +34,20 @@
 namespace ep {
 
 constexpr int kFusedRingDepth = 128;                                  // vectors per tile kept in LDS
-constexpr uint32_t kFusedRowBytes = kFusedRingDepth * 16 + 16;        // 16 bytes of padding: 16 tiles at one position cover all banks
+// A ring row: 128 vectors of 16 bytes (bf16) or 8 bytes (int8 codes) + 16 bytes of padding, so that 16 tiles read at one
+// position cover all banks.
+constexpr uint32_t fused_row_bytes(bool int8) { return kFusedRingDepth * (int8 ? 8u : 16u) + 16u; }
 constexpr int kFusedWaves = 16;
 
 typedef __bf16 fused_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float fused_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t fused_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t fused_u32x2 __attribute__((ext_vector_type(2)));
+typedef int fused_i32x4 __attribute__((ext_vector_type(4)));
+typedef int fused_i32x16 __attribute__((ext_vector_type(16)));
 
-inline int fused_lds_bytes(int prob_bits) {
-  return sym_table_bytes(prob_bits) + kFusedWaves * 2 * kRingBytes + EP_HIP_FUSED_SLOTS * static_cast<int>(kFusedRowBytes);
+inline int fused_lds_bytes(int prob_bits, bool int8) {
+  return sym_table_bytes(prob_bits) + kFusedWaves * 2 * kRingBytes + EP_HIP_FUSED_SLOTS * static_cast<int>(fused_row_bytes(int8));
 }
 
 // The weights of the vector a lane just decoded with the two-level tables: (z + c / 2) * scale with one rounding,
@@ -80,13 +85,21 @@ __device__ __forceinline__ void fused_chain(Pair& s, const StepConsts& k, bool v
   emit_priority();
 }
 
-template <int PB, int F>
+// INT8: the container decodes to int8 codes (the int8 store's rounding and clamp), the activations are int8, the products
+// are v_mfma_i32_32x32x32_i8 (a step is 32 k = four vectors, a wave takes four of a window's eight) and the planes hold
+// exact int32 sums.
+template <int PB, int F, bool INT8>
 __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const ep_hip_fused_batch* __restrict__ batches) {
   extern __shared__ __align__(16) uint8_t smem[];
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
   typedef __attribute__((address_space(3))) fused_u32x4* lds_u4;
+  typedef __attribute__((address_space(3))) fused_u32x2* lds_u2;
   constexpr uint32_t kTables = static_cast<uint32_t>(sym_table_bytes(PB));
   constexpr uint32_t kTable = 1u << PB;
+  constexpr uint32_t kVectorBytes = INT8 ? 8u : 16u;
+  constexpr uint32_t kRowBytes = fused_row_bytes(INT8);
+  constexpr int kStepVectors = INT8 ? 4 : 2;           // vectors one matrix-core instruction multiplies (32 or 16 k)
+  constexpr int kWaveSteps = INT8 ? 4 : 8;             // steps of a window one wave takes (every second one)
   static_assert(F == 1 || F == 2 || F == 4 || F == 8, "32 F activation rows per workgroup, two waves per 32");
 
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
@@ -148,10 +161,12 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
     }
   }
   open_window(s, windows0 + static_cast<uint32_t>(slot) * kRingBytes, word_begin, word_end, s.count > 0, a.payload, a.payload_words, a.offsets, l32);
-  const uint32_t my_row = ring0 + static_cast<uint32_t>(slot) * kFusedRowBytes;
-  auto ring_store = [&](int aligned, fused_u32x4 value) {
+  const uint32_t my_row = ring0 + static_cast<uint32_t>(slot) * kRowBytes;
+  auto ring_store = [&](int aligned, fused_u32x4 value) {       // int8: the first two words
     if (aligned >= 0) {
-      *reinterpret_cast<lds_u4>(static_cast<uintptr_t>(my_row + (static_cast<uint32_t>(aligned) & (kFusedRingDepth - 1)) * 16u)) = value;
+      const uint32_t at = my_row + (static_cast<uint32_t>(aligned) & (kFusedRingDepth - 1)) * kVectorBytes;
+      if constexpr (INT8) *reinterpret_cast<lds_u2>(static_cast<uintptr_t>(at)) = fused_u32x2{value[0], value[1]};
+      else *reinterpret_cast<lds_u4>(static_cast<uintptr_t>(at)) = value;
     }
   };
 
@@ -159,11 +174,11 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
   const bool multiplies = wave < 2 * F;
   const int fragment = wave % F, parity = wave / F;        // 32 activation rows, and which of every two k steps
   const int m_first = static_cast<int>(blockIdx.y) * 32 * F + 32 * fragment;
-  // a.x = the activations repacked by pack_activations_kernel: [k / 16][activation row][16 values], so that the 32 rows x
-  // 16 k of a fragment are 1 KiB of consecutive memory (a.ldx = rows per k block, a multiple of 32 F).
-  const uint8_t* x_row = reinterpret_cast<const uint8_t*>(a.x) + (static_cast<int64_t>(m_first + l32) * 16 + half * 8) * 2;
+  // a.x = the activations repacked by pack_activations_kernel: [k step][activation row][32 bytes] (16 bf16 or 32 int8
+  // values), so that the 32 rows of a fragment are 1 KiB of consecutive memory (a.ldx = rows per k step, a multiple of 32 F).
+  const uint8_t* x_row = reinterpret_cast<const uint8_t*>(a.x) + static_cast<int64_t>(m_first + l32) * 32 + half * 16;
   const int64_t x_block_bytes = a.ldx * 32;
-  const uint32_t read_row = ring0 + static_cast<uint32_t>(l32) * kFusedRowBytes;
+  const uint32_t read_row = ring0 + static_cast<uint32_t>(l32) * kRowBytes;
   // The accumulator column l32 holds tile `l32` of the batch. row_now = the weight row that column is summing: that of
   // the position just above the first window, lowered by one at every row boundary the windows cross.
   const int column_tile = batch.tile[l32];
@@ -172,9 +187,10 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
   if (column_live) {
     row_now = static_cast<int>((static_cast<int64_t>(column_tile) * tv - batch.delta[l32] + 32 * groups + 32) / vpr);
   }
-  fused_f32x16 acc;
+  using Acc = typename std::conditional<INT8, fused_i32x16, fused_f32x16>::type;
+  Acc acc;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
   // A column's sums for one weight row are one of several partial sums of that row: a row touches up to `planes` tiles,
   // and two waves share a fragment's k steps. Every (tile of the row, wave parity) has its own plane of the workspace,
   // laid out [plane][weight row][activation row]: a lane's four consecutive activation rows are 16 contiguous bytes, a
@@ -188,20 +204,20 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
         const int plane = 2 * (column_tile - static_cast<int>(row_first / tv)) + parity;
         float* at = a.y32 + (static_cast<int64_t>(plane) * rows_total + row_now) * a.ldy32 + m_first + 4 * half;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          typedef float f32x4 __attribute__((ext_vector_type(4)));
-          *reinterpret_cast<f32x4*>(at + 8 * q) = f32x4{acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+        for (int q = 0; q < 4; ++q) {          // int8: the same cells hold int32 sums
+          typedef typename std::conditional<INT8, fused_i32x4, float __attribute__((ext_vector_type(4)))>::type Cell4;
+          *reinterpret_cast<Cell4*>(at + 8 * q) = Cell4{acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
         }
       }
     }
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
     row_now -= 1;
   };
 
   // In-row vector position of the window's first aligned index; windows go down by 32 per step.
   int q0 = __builtin_amdgcn_readfirstlane(static_cast<int>((static_cast<int64_t>(batch.base) + 32 * groups) % vpr));
-  if (q0 < 0 || (q0 & 1) != 0) {        // a batch table that is not ep_hip_fused_plan's: nothing below may index with it
+  if (q0 < 0 || (q0 & (kStepVectors - 1)) != 0) {        // a batch table that is not ep_hip_fused_plan's: nothing below may index with it
     if (threadIdx.x == 0) flag_error(a.error, EP_DECODE_BAD_OFFSETS);
     return;
   }
@@ -215,13 +231,13 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
   for (int g = groups - 1; g >= -1; --g) {
     // The activations of the window this step completes, aligned indices [32 (g + 1), 32 (g + 2)): 16 bytes per lane and
     // k step, requested now and used after the chain.
-    fused_u32x4 xa[8];
+    fused_u32x4 xa[kWaveSteps];
     if (multiplies) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        int q = q0 + 2 * (2 * j + parity);
+      for (int j = 0; j < kWaveSteps; ++j) {
+        int q = q0 + kStepVectors * (2 * j + parity);
         q = q >= vpr ? q - vpr : q;
-        xa[j] = *reinterpret_cast<const fused_u32x4*>(x_row + static_cast<int64_t>(q >> 1) * x_block_bytes);
+        xa[j] = *reinterpret_cast<const fused_u32x4*>(x_row + static_cast<int64_t>(q / kStepVectors) * x_block_bytes);
       }
     }
 
@@ -236,12 +252,19 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
       else fused_chain<PB, true>(s, k, valid_lane, valid);
       float w[8];
       sym_weights(s, scale, w);
+      if constexpr (INT8) {
+        uint32_t low, high;
+        codes_i8(w, low, high);
+        packed[0] = valid_lane ? low : 0u;
+        packed[1] = valid_lane ? high : 0u;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        typedef float float2v __attribute__((ext_vector_type(2)));
-        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        const float2v two = {w[2 * i], w[2 * i + 1]};
-        packed[i] = valid_lane ? __builtin_bit_cast(uint32_t, __builtin_convertvector(two, bf16x2)) : 0u;
+        for (int i = 0; i < 4; ++i) {
+          typedef float float2v __attribute__((ext_vector_type(2)));
+          typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+          const float2v two = {w[2 * i], w[2 * i + 1]};
+          packed[i] = valid_lane ? __builtin_bit_cast(uint32_t, __builtin_convertvector(two, bf16x2)) : 0u;
+        }
       }
     }
     ring_store(first + l32 + delta, packed);
@@ -251,23 +274,27 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
       const uint32_t window = static_cast<uint32_t>(32 * (g + 1));
       const bool crossing = q0 + 32 >= vpr;                 // a row ends inside this window, or exactly at its top
       const int boundary = crossing ? vpr - q0 : 64;        // window-relative index of the upper row's first vector
-      auto multiply = [&](int j) {
-        const uint32_t at = (window + static_cast<uint32_t>(2 * (2 * j + parity) + half)) & (kFusedRingDepth - 1);
-        const fused_u32x4 b = *reinterpret_cast<lds_u4>(static_cast<uintptr_t>(read_row + at * 16u));
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(fused_bf16x8, xa[j]), __builtin_bit_cast(fused_bf16x8, b), acc, 0, 0, 0);
+      auto multiply = [&](int j) {       // a lane's 16 bytes: one bf16 vector, or two consecutive vectors of int8 codes
+        const uint32_t at = (window + static_cast<uint32_t>(kStepVectors * (2 * j + parity) + (kStepVectors / 2) * half)) & (kFusedRingDepth - 1);
+        const fused_u32x4 b = *reinterpret_cast<lds_u4>(static_cast<uintptr_t>(read_row + at * kVectorBytes));
+        if constexpr (INT8) {
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(fused_i32x4, xa[j]), __builtin_bit_cast(fused_i32x4, b), acc, 0, 0, 0);
+        } else {
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(fused_bf16x8, xa[j]), __builtin_bit_cast(fused_bf16x8, b), acc, 0, 0, 0);
+        }
       };
       if (!crossing) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) multiply(j);
+        for (int j = 0; j < kWaveSteps; ++j) multiply(j);
       } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (2 * (2 * j + parity) >= boundary) multiply(j);
+        for (int j = 0; j < kWaveSteps; ++j) {
+          if (kStepVectors * (2 * j + parity) >= boundary) multiply(j);
         }
         flush();
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (2 * (2 * j + parity) < boundary) multiply(j);
+        for (int j = 0; j < kWaveSteps; ++j) {
+          if (kStepVectors * (2 * j + parity) < boundary) multiply(j);
         }
       }
     }
@@ -289,19 +316,20 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
   }
 }
 
-// x[m][k] (bf16, row stride ldx) -> packed[k / 16][m][16], rows m_rows .. m_padded - 1 zero. One thread per 32 bytes.
-__global__ __launch_bounds__(256) void pack_activations_kernel(const uint16_t* __restrict__ x, int64_t ldx, int m_rows, int64_t m_padded,
-                                                               int k_blocks, uint16_t* __restrict__ packed) {
+// x[m][32-byte steps of a row] (row stride in bytes) -> packed[step][m][32 bytes], rows m_rows .. m_padded - 1 zero: 16
+// bf16 or 32 int8 activations per step. One thread per 32 bytes.
+__global__ __launch_bounds__(256) void pack_activations_kernel(const uint8_t* __restrict__ x, int64_t row_bytes, int m_rows, int64_t m_padded,
+                                                               int k_steps, uint8_t* __restrict__ packed) {
   const int64_t index = blockIdx.x * int64_t{256} + threadIdx.x;
-  if (index >= m_padded * k_blocks) return;
-  const int64_t m = index % m_padded, block = index / m_padded;
+  if (index >= m_padded * k_steps) return;
+  const int64_t m = index % m_padded, step = index / m_padded;
   uint4 low = make_uint4(0, 0, 0, 0), high = low;
   if (m < m_rows) {
-    const uint4* from = reinterpret_cast<const uint4*>(x + m * ldx + block * 16);
+    const uint4* from = reinterpret_cast<const uint4*>(x + m * row_bytes + step * 32);
     low = from[0];
     high = from[1];
   }
-  uint4* to = reinterpret_cast<uint4*>(packed + index * 16);
+  uint4* to = reinterpret_cast<uint4*>(packed + index * 32);
   to[0] = low;
   to[1] = high;
 }
@@ -311,10 +339,14 @@ inline int fused_planes_per_row(int64_t vpr, int tv) { return 1 + static_cast<in
 
 // y[m][n] = cast(sum of the partial-sum planes of weight row n + bias[n]). Workspace layout [plane][n][m_padded]; row n
 // was written by tiles first_tile(n) .. last_tile(n), two planes (wave parities) each. A block transposes a 32 x 32 patch
-// through LDS so that both the reads (along m) and the writes (along n) are contiguous.
-__global__ __launch_bounds__(256) void finish_fused_planes_kernel(const float* __restrict__ y32, const void* __restrict__ bias, void* __restrict__ y,
-                                                                  int m_rows, int64_t m_padded, int outer, int vpr, int tv, int64_t ldy,
-                                                                  int out_kind) {
+// through LDS so that both the reads (along m) and the writes (along n) are contiguous. INT8: the planes hold int32 sums,
+// added exactly, then f32(sum) * scale_a[m] * scale_b[n] + bias[n] as three single-rounded operations (the epilogue of the
+// int8 GEMM kernels, entropack/linear/quant_kernels.py:15-54 of the reference).
+template <bool INT8>
+__global__ __launch_bounds__(256) void finish_fused_planes_kernel(const float* __restrict__ y32, const float* __restrict__ scale_a,
+                                                                  const float* __restrict__ scale_b, const void* __restrict__ bias,
+                                                                  void* __restrict__ y, int m_rows, int64_t m_padded, int outer, int vpr, int tv,
+                                                                  int64_t ldy, int out_kind) {
   __shared__ float patch[32][33];
   const int n0 = static_cast<int>(blockIdx.x) * 32, m0 = static_cast<int>(blockIdx.y) * 32;
   const int lane_m = threadIdx.x & 31, group = threadIdx.x >> 5;          // 8 groups of 32 threads
@@ -325,7 +357,15 @@ __global__ __launch_bounds__(256) void finish_fused_planes_kernel(const float* _
     if (n < outer && m0 + lane_m < m_padded) {
       const int64_t row_first = static_cast<int64_t>(n) * vpr;
       const int tiles = static_cast<int>((row_first + vpr - 1) / tv) - static_cast<int>(row_first / tv) + 1;
-      for (int plane = 0; plane < 2 * tiles; ++plane) sum += y32[(static_cast<int64_t>(plane) * outer + n) * m_padded + m0 + lane_m];
+      if constexpr (INT8) {
+        int total = 0;
+        for (int plane = 0; plane < 2 * tiles; ++plane) {
+          total += reinterpret_cast<const int*>(y32)[(static_cast<int64_t>(plane) * outer + n) * m_padded + m0 + lane_m];
+        }
+        sum = static_cast<float>(total);
+      } else {
+        for (int plane = 0; plane < 2 * tiles; ++plane) sum += y32[(static_cast<int64_t>(plane) * outer + n) * m_padded + m0 + lane_m];
+      }
     }
     patch[group * 4 + i][lane_m] = sum;
   }
@@ -335,6 +375,7 @@ __global__ __launch_bounds__(256) void finish_fused_planes_kernel(const float* _
     const int m = m0 + group * 4 + i, n = n0 + lane_m;
     if (m >= m_rows || n >= outer) continue;
     float v = patch[lane_m][group * 4 + i];
+    if constexpr (INT8) v = __fmul_rn(__fmul_rn(v, scale_a[m]), scale_b[n]);
     if (bias != nullptr) {
       float add;
       if (out_kind == EP_FLOAT_BF16) add = __uint_as_float(static_cast<uint32_t>(static_cast<const uint16_t*>(bias)[n]) << 16);
@@ -348,13 +389,13 @@ __global__ __launch_bounds__(256) void finish_fused_planes_kernel(const float* _
   }
 }
 
-template <int PB, int F>
+template <int PB, int F, bool INT8>
 static int launch_fused_one(const DecodeArgs& args, const ep_hip_fused_batch* batches, int n_batches, int m_blocks, hipStream_t stream) {
   static thread_local int configured_for = -1;
-  const int status = allow_full_lds(reinterpret_cast<const void*>(decode_mfma_kernel<PB, F>), configured_for);
+  const int status = allow_full_lds(reinterpret_cast<const void*>(decode_mfma_kernel<PB, F, INT8>), configured_for);
   if (status != EP_HIP_OK) return status;
-  hipLaunchKernelGGL((decode_mfma_kernel<PB, F>), dim3(static_cast<unsigned>(n_batches), static_cast<unsigned>(m_blocks)), dim3(1024),
-                     static_cast<size_t>(fused_lds_bytes(PB)), stream, args, batches);
+  hipLaunchKernelGGL((decode_mfma_kernel<PB, F, INT8>), dim3(static_cast<unsigned>(n_batches), static_cast<unsigned>(m_blocks)), dim3(1024),
+                     static_cast<size_t>(fused_lds_bytes(PB, INT8)), stream, args, batches);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }
@@ -370,15 +411,15 @@ static size_t fused_plane_bytes(int64_t rows, int64_t cols_padded, int tile_elem
                        static_cast<size_t>(fused_padded_rows(m_rows)) * 4;
   return (bytes + 255) / 256 * 256;
 }
-// The partial-sum planes, then the repacked activations.
-size_t fused_workspace_bytes(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows) {
-  return fused_plane_bytes(rows, cols_padded, tile_elements, m_rows) + static_cast<size_t>(fused_padded_rows(m_rows)) * static_cast<size_t>(cols_padded) * 2;
+// The partial-sum planes, then the repacked activations (`element_bytes` each: 2 for bf16, 1 for int8).
+size_t fused_workspace_bytes(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows, int element_bytes) {
+  return fused_plane_bytes(rows, cols_padded, tile_elements, m_rows) +
+         static_cast<size_t>(fused_padded_rows(m_rows)) * static_cast<size_t>(cols_padded) * static_cast<size_t>(element_bytes);
 }
 
-int launch_fused_mfma(DecodeArgs args, const ep_hip_plan_desc& desc, const ep_hip_fused_batch* batches, int n_batches, const void* bias,
-                      void* y, int64_t ldy, int out_kind, hipStream_t stream) {
-  if (desc.prob_bits != 11 || args.sym_tables == nullptr) return EP_HIP_EUNSUPPORTED;       // the two-level tables of prob_bits 11 plans
-  if (args.vecs_per_row < 32 || args.vecs_per_row % 2 != 0 || n_batches <= 0 || args.m_rows <= 0) return EP_HIP_EUNSUPPORTED;
+template <bool INT8>
+static int launch_fused_kind(DecodeArgs args, const ep_hip_fused_batch* batches, int n_batches, const float* scale_a, const float* scale_b,
+                             const void* bias, void* y, int64_t ldy, int out_kind, hipStream_t stream) {
   const int m = args.m_rows;
   const int per_block = fused_rows_per_block(m);
   const int m_blocks = (m + per_block - 1) / per_block;
@@ -386,30 +427,39 @@ int launch_fused_mfma(DecodeArgs args, const ep_hip_plan_desc& desc, const ep_hi
   args.ldy32 = static_cast<int64_t>(m_blocks) * per_block;          // activation rows per workspace row
   const int64_t cols_padded = static_cast<int64_t>(args.vecs_per_row) * 8;
   const int outer = static_cast<int>(args.num_vectors / args.vecs_per_row);
-  uint16_t* packed = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(args.y32) +
-                                                 fused_plane_bytes(outer, cols_padded, args.tile_vectors * 9, m));
+  uint8_t* packed = reinterpret_cast<uint8_t*>(args.y32) + fused_plane_bytes(outer, cols_padded, args.tile_vectors * 9, m);
   {
-    const int k_blocks = args.vecs_per_row / 2;
-    const int64_t threads = args.ldy32 * k_blocks;
-    hipLaunchKernelGGL(pack_activations_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, args.x, args.ldx, m,
-                       args.ldy32, k_blocks, packed);
+    const int element_bytes = INT8 ? 1 : 2;
+    const int k_steps = static_cast<int>(cols_padded * element_bytes / 32);
+    const int64_t threads = args.ldy32 * k_steps;
+    hipLaunchKernelGGL(pack_activations_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint8_t*>(args.x), args.ldx * element_bytes, m, args.ldy32, k_steps, packed);
     EP_HIP_TRY(hipGetLastError());
-    args.x = packed;
+    args.x = reinterpret_cast<const uint16_t*>(packed);
     args.ldx = args.ldy32;
   }
   int status;
   switch (per_block / 32) {
-    case 1: status = launch_fused_one<11, 1>(args, batches, n_batches, m_blocks, stream); break;
-    case 2: status = launch_fused_one<11, 2>(args, batches, n_batches, m_blocks, stream); break;
-    case 4: status = launch_fused_one<11, 4>(args, batches, n_batches, m_blocks, stream); break;
-    default: status = launch_fused_one<11, 8>(args, batches, n_batches, m_blocks, stream); break;
+    case 1: status = launch_fused_one<11, 1, INT8>(args, batches, n_batches, m_blocks, stream); break;
+    case 2: status = launch_fused_one<11, 2, INT8>(args, batches, n_batches, m_blocks, stream); break;
+    case 4: status = launch_fused_one<11, 4, INT8>(args, batches, n_batches, m_blocks, stream); break;
+    default: status = launch_fused_one<11, 8, INT8>(args, batches, n_batches, m_blocks, stream); break;
   }
   if (status != EP_HIP_OK) return status;
   const dim3 grid(static_cast<unsigned>((outer + 31) / 32), static_cast<unsigned>((m + 31) / 32));
-  hipLaunchKernelGGL(finish_fused_planes_kernel, grid, dim3(256), 0, stream, args.y32, bias, y, m, args.ldy32, outer, args.vecs_per_row,
-                     args.tile_vectors, ldy, out_kind);
+  hipLaunchKernelGGL(finish_fused_planes_kernel<INT8>, grid, dim3(256), 0, stream, args.y32, scale_a, scale_b, bias, y, m, args.ldy32, outer,
+                     args.vecs_per_row, args.tile_vectors, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
+}
+
+// args.x / args.ldx: the activations as the caller holds them (bf16, or int8 codes with scale_a / scale_b given).
+int launch_fused_mfma(const DecodeArgs& args, const ep_hip_plan_desc& desc, const ep_hip_fused_batch* batches, int n_batches, bool int8,
+                      const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t ldy, int out_kind, hipStream_t stream) {
+  if (desc.prob_bits != 11 || args.sym_tables == nullptr) return EP_HIP_EUNSUPPORTED;       // the two-level tables of prob_bits 11 plans
+  if (args.vecs_per_row < 32 || args.vecs_per_row % 4 != 0 || n_batches <= 0 || args.m_rows <= 0) return EP_HIP_EUNSUPPORTED;
+  if (int8) return launch_fused_kind<true>(args, batches, n_batches, scale_a, scale_b, bias, y, ldy, out_kind, stream);
+  return launch_fused_kind<false>(args, batches, n_batches, nullptr, nullptr, bias, y, ldy, out_kind, stream);
 }
 
 }  // namespace ep
@@ -422,14 +472,14 @@ extern "C" int ep_hip_fused_plan(int64_t rows, int64_t cols_padded, int tile_ele
   const int tv = tile_vectors_of(tile_elements);
   const int64_t vectors = rows * vpr;
   const int64_t tiles = (vectors + tv - 1) / tv;
-  if (vpr < 32 || vpr % 2 != 0 || vpr > 0x7FFFFFFF || vectors >= (int64_t{1} << 31) || tiles >= (int64_t{1} << 30)) return EP_HIP_EUNSUPPORTED;
+  if (vpr < 32 || vpr % 4 != 0 || vpr > 0x7FFFFFFF || vectors >= (int64_t{1} << 31) || tiles >= (int64_t{1} << 30)) return EP_HIP_EUNSUPPORTED;
   std::vector<std::pair<int32_t, int32_t>> order(static_cast<size_t>(tiles));      // (position of the tile's first vector in its row, tile)
   for (int64_t t = 0; t < tiles; ++t) order[static_cast<size_t>(t)] = {static_cast<int32_t>((t * tv) % vpr), static_cast<int32_t>(t)};
   std::sort(order.begin(), order.end());
   int count = 0;
   size_t at = 0;
   while (at < order.size()) {
-    const int32_t base = order[at].first & ~1;        // even: a 16-wide k step (two vectors) then never straddles a row boundary
+    const int32_t base = order[at].first & ~3;        // a multiple of 4: a k step (two vectors of bf16, four of int8 codes) never straddles a row boundary
     size_t end = at;
     while (end < order.size() && end - at < EP_HIP_FUSED_SLOTS && order[end].first - base <= EP_HIP_FUSED_MAX_SKEW) ++end;
     if (batches_host != nullptr) {

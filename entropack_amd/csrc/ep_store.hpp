@@ -99,7 +99,7 @@ __device__ __forceinline__ void stream_store8(void* at, uint32_t a, uint32_t b) 
 // Clamping first gives the same result (the bounds are integers). Adding 1.5 * 2^23 to a value in [-128, 127] rounds it
 // to an integer, ties to even, in the sum's mantissa, whose low byte is then the two's-complement code; the add writes
 // that byte straight into its place in the packed word (sub-dword destination select), so a weight costs a clamp and an add.
-__device__ __forceinline__ void store_vector_i8(void* out, int64_t vector, const float (&w)[8]) {
+__device__ __forceinline__ void codes_i8(const float (&w)[8], uint32_t& low, uint32_t& high) {
   float magic = 12582912.0f;
   asm volatile("" : "+v"(magic));          // a vector register: the sub-dword form takes no literal
   // Few vectors hold a value outside [-128, 127]: one magnitude test for all eight instead of eight clamps.
@@ -114,7 +114,6 @@ __device__ __forceinline__ void store_vector_i8(void* out, int64_t vector, const
 #pragma unroll
     for (int i = 0; i < 8; ++i) c[i] = __builtin_fminf(__builtin_fmaxf(w[i], -128.0f), 127.0f);
   }
-  uint32_t low, high;
   // The two words alternate: an instruction that keeps the other bytes of its destination must not directly follow
   // the one that wrote them (sub-dword writes need one instruction in between on this hardware).
 #define EP_I8_ADD(DST, SRC, BYTE, UNUSED) \
@@ -127,6 +126,11 @@ __device__ __forceinline__ void store_vector_i8(void* out, int64_t vector, const
       : "=&v"(low), "=&v"(high)
       : "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]), "v"(c[7]), "v"(magic));
 #undef EP_I8_ADD
+}
+
+__device__ __forceinline__ void store_vector_i8(void* out, int64_t vector, const float (&w)[8]) {
+  uint32_t low, high;
+  codes_i8(w, low, high);
   stream_store8(reinterpret_cast<uint2*>(out) + vector, low, high);
 }
 
@@ -270,8 +274,8 @@ int launch_sym(const LdsLaunch& cfg, const DecodeArgs& args, int num_pairs, cons
 int effective_table_kind(const ep_hip_plan_desc& desc, int kind, int64_t pairs, int cus);
 int launch_lds_decode(const DecodeArgs& args, const ep_hip_plan_desc& desc, int kind, int num_pairs, hipStream_t stream);
 // Decode-to-GEMM through LDS (ep_decode_mfma.hip): args.x / m_rows / y32 set, one workgroup per batch and block of rows.
-int launch_fused_mfma(DecodeArgs args, const ep_hip_plan_desc& desc, const ep_hip_fused_batch* batches, int n_batches, const void* bias, void* y,
-                      int64_t ldy, int out_kind, hipStream_t stream);
-size_t fused_workspace_bytes(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows);
+int launch_fused_mfma(const DecodeArgs& args, const ep_hip_plan_desc& desc, const ep_hip_fused_batch* batches, int n_batches, bool int8,
+                      const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t ldy, int out_kind, hipStream_t stream);
+size_t fused_workspace_bytes(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows, int element_bytes);
 
 }  // namespace ep

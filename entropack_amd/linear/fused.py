@@ -92,5 +92,14 @@ def linear_forward(layer, x: torch.Tensor) -> torch.Tensor:
 
 
 def int8_linear_forward(layer, activation: torch.Tensor, activation_scale: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    if layer.forward_mode == "fused_through_lds":
+        container = layer._container()
+        if container.compress_method == "lattice_rans" and container.encoded_dtype == torch.int8:
+            on_device = container.to(device=activation.device)
+            buffers = packed_buffers(on_device.buffers, LatticeBuffers)
+            if hip_lane.mfma_linear_usable(buffers, tuple(container.shape), activation):
+                return hip_lane.linear_mfma_i8(buffers, shape=tuple(container.shape), activation=activation, activation_scale=activation_scale,
+                                               weight_scale=layer._scale(activation.device), bias=layer._bias_on(activation.device),
+                                               out_dtype=out_dtype)
     codes = layer._decoded_for(activation)
     return kernels.int8_gemm(activation, codes, activation_scale, layer._scale(codes.device), layer._bias_on(activation.device), out_dtype)

@@ -408,7 +408,7 @@ class CompressedINT8Linear(QuantizedLinear):
             activation, activation_scale = kernels.rotate_quantize_rows(flat.detach(), self._convrot_group)
         else:
             activation, activation_scale = kernels.quantize_rows(flat.detach())
-        if self.forward_mode == "fused":
+        if self.forward_mode != "decode_then_gemm":
             from . import fused
             out = fused.int8_linear_forward(self, activation, activation_scale, x.dtype)
         else:

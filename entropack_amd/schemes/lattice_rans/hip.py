@@ -274,15 +274,38 @@ def fused_batches(buffers: LatticeBuffers, info: dict) -> tuple[torch.Tensor, in
 
 
 def mfma_linear_usable(buffers: LatticeBuffers, shape, x: torch.Tensor) -> bool:
-    """Can `linear_mfma` take this container and activation? bf16 activations, weight rows of a multiple of 16 and at least
-    256 columns, and a plan with the two-level tables of prob_bits 11 (what the default encoder settings give up to 7 bpp)."""
-    if not (x.dtype == torch.bfloat16 and x.numel() > 0 and shape[1] % 16 == 0 and shape[1] >= 256 and x.shape[-1] == shape[1]
+    """Can `linear_mfma` (bfloat16 activations) or `linear_mfma_i8` (int8 activation codes) take this container and
+    activation? Weight rows of a multiple of 32 and at least 256 columns, and a plan with the two-level tables of prob_bits
+    11 (what the default encoder settings give up to 7 bpp)."""
+    if not (x.dtype in (torch.bfloat16, torch.int8) and x.numel() > 0 and shape[1] % 32 == 0 and shape[1] >= 256 and x.shape[-1] == shape[1]
             and buffers.payload.device.type == "cuda"):
         return False
-    info, _, _ = _checked_geometry(buffers, shape, torch.bfloat16)
+    info, _, _ = _checked_geometry(buffers, shape, x.dtype)
     with torch.cuda.device(buffers.payload.device):
         plan = _plan_for(buffers, info)
     return plan.desc.prob_bits == 11 and plan.desc.sym_offset != 0 and plan.desc.table_kind in (_hip.TABLE_LDS_BYTE, _hip.TABLE_LDS_SYM)
+
+
+def _mfma_call(buffers: LatticeBuffers, shape, flat: torch.Tensor, weight_dtype: torch.dtype, out_dtype: torch.dtype, bias, extra):
+    """Common part of the two decode-to-GEMM calls: plan, batches, job, output, workspace; `extra(job, table, batches, out,
+    workspace, bias pointer, stream)` makes the C call."""
+    device = buffers.payload.device
+    info, _, _ = _checked_geometry(buffers, shape, weight_dtype)
+    if not mfma_linear_usable(buffers, shape, flat):
+        raise ValueError("decode-to-GEMM through LDS takes bfloat16 or int8 activations, weight rows of a multiple of 32 (at least 256) "
+                         "columns and a container whose plan has the two-level tables (prob_bits 11, byte-valued symbols)")
+    outer = info["rows"]
+    with torch.cuda.device(device):
+        plan = _plan_for(buffers, info)
+        table, batches, _ = fused_batches(buffers, info)
+        job = _job_of(buffers, info, plan, _hip.STORE_KINDS[weight_dtype])
+        out = torch.empty(flat.shape[0], outer, dtype=out_dtype, device=device)
+        workspace = torch.empty(_hip.library().ep_hip_linear_fused_mfma_workspace(outer, info["cols"], info["tile_elements"], flat.shape[0],
+                                                                                   1 if weight_dtype == torch.int8 else 0),
+                                dtype=torch.uint8, device=device)
+        bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
+        extra(job, table, batches, out, workspace, None if bias_ready is None else bias_ready.data_ptr(), _hip.current_stream(device))
+    return out
 
 
 def linear_mfma(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
@@ -291,28 +314,38 @@ def linear_mfma(buffers: LatticeBuffers, *, shape, x: torch.Tensor, bias: torch.
 
     The reference decodes the whole weight and calls F.linear (entropack/linear/linear.py:163-165).
     """
-    device = buffers.payload.device
-    info, _, _ = _checked_geometry(buffers, shape, torch.bfloat16)
-    if not mfma_linear_usable(buffers, shape, x):
-        raise ValueError("linear_mfma takes bfloat16 activations, weight rows of a multiple of 16 (at least 256) columns and a "
-                         "container whose plan has the two-level tables (prob_bits 11, byte-valued symbols)")
     flat = x.reshape(-1, x.shape[-1])
     if flat.stride(-1) != 1 or flat.stride(0) % 8 or flat.data_ptr() % 16:
         flat = flat.contiguous()
-    outer = info["rows"]
-    with torch.cuda.device(device):
-        plan = _plan_for(buffers, info)
-        table, batches, _ = fused_batches(buffers, info)
-        job = _job_of(buffers, info, plan, _hip.STORE_KINDS[torch.bfloat16])
-        out = torch.empty(flat.shape[0], outer, dtype=x.dtype, device=device)
-        workspace = torch.empty(_hip.library().ep_hip_linear_fused_mfma_workspace(outer, info["cols"], info["tile_elements"], flat.shape[0]),
-                                dtype=torch.uint8, device=device)
-        bias_ready = None if bias is None else bias.to(device=device, dtype=x.dtype).contiguous()
+
+    def call(job, table, batches, out, workspace, bias_pointer, stream):
         _hip.check("ep_hip_linear_fused_mfma_bf16", _hip.library().ep_hip_linear_fused_mfma_bf16(
-            ctypes.byref(job), table.data_ptr(), batches, flat.data_ptr(), flat.shape[0], flat.stride(0),
-            None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(), out.stride(0), _hip.FLOAT_KINDS[x.dtype],
-            workspace.data_ptr(), _hip.current_stream(device)))
-    return out.reshape(*x.shape[:-1], outer)
+            ctypes.byref(job), table.data_ptr(), batches, flat.data_ptr(), flat.shape[0], flat.stride(0), bias_pointer, out.data_ptr(),
+            out.stride(0), _hip.FLOAT_KINDS[x.dtype], workspace.data_ptr(), stream))
+
+    out = _mfma_call(buffers, shape, flat, torch.bfloat16, x.dtype, bias, call)
+    return out.reshape(*x.shape[:-1], out.shape[-1])
+
+
+def linear_mfma_i8(buffers: LatticeBuffers, *, shape, activation: torch.Tensor, activation_scale: torch.Tensor, weight_scale: torch.Tensor,
+                   bias: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
+    """W8A8 with the int8 weight codes decoded inside the product (ep_hip_linear_fused_mfma_i8): `activation` int8 [M, K] with
+    `activation_scale` f32[M] (ep_hip_quantize_rows), `weight_scale` f32[N]; the same bits as the int8 GEMM on decoded codes.
+
+    The reference decodes the codes and calls its Triton int8 GEMM (entropack/linear/linear.py:362-385,485-490).
+    """
+    flat = activation.reshape(-1, activation.shape[-1])
+    if flat.stride(-1) != 1 or flat.stride(0) % 16 or flat.data_ptr() % 16:
+        flat = flat.contiguous()
+    scale_a = activation_scale.to(device=flat.device, dtype=torch.float32).contiguous()
+    scale_b = weight_scale.to(device=flat.device, dtype=torch.float32).contiguous()
+
+    def call(job, table, batches, out, workspace, bias_pointer, stream):
+        _hip.check("ep_hip_linear_fused_mfma_i8", _hip.library().ep_hip_linear_fused_mfma_i8(
+            ctypes.byref(job), table.data_ptr(), batches, flat.data_ptr(), flat.shape[0], flat.stride(0), scale_a.data_ptr(), scale_b.data_ptr(),
+            bias_pointer, out.data_ptr(), out.stride(0), _hip.FLOAT_KINDS[out_dtype], workspace.data_ptr(), stream))
+
+    return _mfma_call(buffers, shape, flat, torch.int8, out_dtype, bias, call)
 
 
 class BatchDecoder:

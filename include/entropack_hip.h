@@ -278,7 +278,7 @@ int ep_hip_linear_fused_bf16_static(const ep_hip_decode_job* weight, const void*
 #define EP_HIP_FUSED_MAX_SKEW 31     /* largest distance, in vectors, between the in-row positions of a batch's tiles */
 
 typedef struct ep_hip_fused_batch {
-  int32_t base;                          /* in-row vector position (even) that aligned index 0 of this batch stands for */
+  int32_t base;                          /* in-row vector position (a multiple of 4) that aligned index 0 of this batch stands for */
   int32_t reserved[3];
   int32_t tile[EP_HIP_FUSED_SLOTS];      /* tile index, or -1 for an unused slot */
   int32_t delta[EP_HIP_FUSED_SLOTS];     /* (tile * tile_vectors) mod vectors_per_row - base, 0 .. EP_HIP_FUSED_MAX_SKEW */
@@ -286,23 +286,35 @@ typedef struct ep_hip_fused_batch {
 
 /* Groups the tiles of a rows x cols_padded container with `tile_elements` symbols per tile into batches. With
  * batches_host NULL only counts them (*n_batches); else fills at most `capacity` batches. EP_HIP_EUNSUPPORTED for rows of
- * fewer than 32 vectors or of an odd number of vectors (cols_padded not a multiple of 16). */
+ * fewer than 32 vectors or whose number of vectors is no multiple of four (cols_padded not a multiple of 32). */
 int ep_hip_fused_plan(int64_t rows, int64_t cols_padded, int tile_elements, ep_hip_fused_batch* batches_host, int capacity,
                       int* n_batches);
 
 /* The product. `weight` as for ep_hip_linear_fused_bf16 (store_kind EP_STORE_BF16; the decoded values are rounded to
  * bf16 exactly as ep_hip_decode_lattice stores them); `batches_dev` = the device copy of ep_hip_fused_plan's output for
  * the same geometry. x is bf16 with row stride `ldx` elements (a multiple of 8, 16-byte aligned base); bias (may be NULL)
- * and y have type `out_kind`; `workspace_dev` (256-byte aligned) holds ep_hip_linear_fused_mfma_workspace(...) bytes and
- * need not be cleared: the kernel writes every partial sum of an output (one per tile the weight row touches and half
+ * and y have type `out_kind`; `workspace_dev` (256-byte aligned) holds ep_hip_linear_fused_mfma_workspace(..., 0) bytes
+ * and need not be cleared: the kernel writes every partial sum of an output (one per tile the weight row touches and half
  * of the k steps) into a plane of its own with plain stores, and a second kernel adds them in a fixed order, then the
  * bias, and rounds once, so results are the same from run to run. EP_HIP_EUNSUPPORTED unless the plan has the two-level
- * tables of prob_bits 11 (byte-valued symbols), which is what the default encoder settings give up to 7 bpp: the caller
- * then decodes and multiplies separately. */
+ * tables of prob_bits 11 (byte-valued symbols), which is what the default encoder settings give up to 7 bpp, and
+ * cols_padded is a multiple of 32: the caller then decodes and multiplies separately. */
 int ep_hip_linear_fused_mfma_bf16(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
                                   const void* x_dev, int64_t m_rows, int64_t ldx, const void* bias_dev, void* y_dev, int64_t ldy,
-                                  int out_kind, float* workspace_dev, void* stream);
-size_t ep_hip_linear_fused_mfma_workspace(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows);
+                                  int out_kind, void* workspace_dev, void* stream);
+
+/* The same for W8A8: `weight` is a container of int8 codes (store_kind EP_STORE_I8, decoded with the rounding and clamp of
+ * the int8 store), a_dev the int8 activation codes of ep_hip_quantize_rows with row stride `lda` bytes (a multiple of 16),
+ * scale_a_dev[m_rows] / scale_b_dev[rows] the activation and weight row scales:
+ *   y[m][n] = cast(f32(sum_k a[m][k] * w[n][k]) * scale_a[m] * scale_b[n] + bias[n]),
+ * the int32 sums exact (partial sums are added as integers), the epilogue three single-rounded float operations: the same
+ * bits as ep_hip_gemm_i8 on the decoded codes. Workspace: ep_hip_linear_fused_mfma_workspace(..., 1) bytes.
+ * Reference: CompressedINT8Linear._forward8 / _gemm, entropack/linear/linear.py:362-385,485-490 (decode the codes, then the
+ * Triton int8 GEMM of entropack/linear/quant_kernels.py:15-54). */
+int ep_hip_linear_fused_mfma_i8(const ep_hip_decode_job* weight, const ep_hip_fused_batch* batches_dev, int n_batches,
+                                const int8_t* a_dev, int64_t m_rows, int64_t lda, const float* scale_a_dev, const float* scale_b_dev,
+                                const void* bias_dev, void* y_dev, int64_t ldy, int out_kind, void* workspace_dev, void* stream);
+size_t ep_hip_linear_fused_mfma_workspace(int64_t rows, int64_t cols_padded, int tile_elements, int64_t m_rows, int int8);
 
 /* Encoder (the step before the path) -------------------------------------------------------------------------- *
  *

@@ -32,7 +32,7 @@ def _plan(rows, cols, tile_elements):
 
 
 @pytest.mark.parametrize("rows,cols,tile_elements", [
-    (3072, 3072, 16384), (3072, 3072, 4096), (8192, 28672, 16384), (3840, 10240, 8192), (64, 272, 288), (1, 256, 16384), (300, 4112, 4100),
+    (3072, 3072, 16384), (3072, 3072, 4096), (8192, 28672, 16384), (3840, 10240, 8192), (64, 288, 288), (1, 256, 16384), (300, 4128, 4100),
 ])
 def test_fused_plan_covers_every_tile_once_with_aligned_chains(rows, cols, tile_elements):
     status, batches = _plan(rows, cols, tile_elements)
@@ -42,7 +42,7 @@ def test_fused_plan_covers_every_tile_once_with_aligned_chains(rows, cols, tile_
     tiles = -(-rows * vectors_per_row // tile_vectors)
     seen = []
     for batch in batches:
-        assert batch.base % 2 == 0 and 0 <= batch.base < vectors_per_row
+        assert batch.base % 4 == 0 and 0 <= batch.base < vectors_per_row
         used = [slot for slot in range(hip_backend.FUSED_SLOTS) if batch.tile[slot] >= 0]
         assert used and used == list(range(len(used)))                   # used slots come first
         for slot in used:
@@ -54,6 +54,7 @@ def test_fused_plan_covers_every_tile_once_with_aligned_chains(rows, cols, tile_
 
 def test_fused_plan_refuses_rows_it_cannot_align():
     assert _plan(64, 264, 16384)[0] == hip_backend.EUNSUPPORTED            # 33 vectors per row: odd
+    assert _plan(64, 272, 16384)[0] == hip_backend.EUNSUPPORTED            # 34 vectors per row: no multiple of four
     assert _plan(64, 128, 16384)[0] == hip_backend.EUNSUPPORTED            # 16 vectors per row: shorter than a group
     assert _plan(0, 256, 16384)[0] == hip_backend.EINVAL
     count = ctypes.c_int(0)
@@ -97,9 +98,9 @@ CASES = [
     # rows, cols, bpp, tile_elements (None = default), activation rows
     (3072, 3072, 4.0, None, (1, 5, 33, 100, 256, 300)),
     (512, 1024, 4.0, 4096, (7, 64)),
-    (256, 272, 3.5, 288, (3, 40)),              # 34 vectors per row, tiles of 32 vectors: a row boundary in almost every window
+    (256, 288, 3.5, 288, (3, 40)),              # 36 vectors per row, tiles of 32 vectors: a row boundary in almost every window
     (1000, 2048, 2.0, None, (16, 129)),         # tiles of 3640 vectors, a short last tile
-    (130, 4112, 6.0, 4100, (2, 96)),            # 514 vectors per row, odd tile length (455 vectors)
+    (130, 4128, 6.0, 4100, (2, 96)),            # 516 vectors per row, odd tile length (455 vectors)
 ]
 
 
@@ -185,3 +186,36 @@ def test_config_3_layer_in_fused_through_lds_mode_never_materialises_its_weight(
         if m == 256:
             # output + partial-sum planes + repacked activations: less than the 18.9 MB a dense copy of the weight would take
             assert peak - before < 3072 * 3072 * 2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols,tile_elements,activation_rows", [(768, 1024, None, (5, 100, 300)), (96, 288, 288, (33,)), (512, 3072, 4096, (64, 257))])
+def test_int8_layer_in_fused_through_lds_mode_gives_the_bits_of_decode_then_gemm(rows, cols, tile_elements, activation_rows):
+    """W8A8: the int8 codes are decoded inside the product (ep_hip_linear_fused_mfma_i8). Integer partial sums are exact and the
+    epilogue is the int8 GEMM's, so the output must equal the decode_then_gemm layer's bit for bit, and both must equal the
+    layer's definition f32(sum) * sa * sw + b (entropack/linear/quant_kernels.py:15-54 of the reference) rounded once."""
+    from entropack_amd.linear import kernels
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    torch.manual_seed(rows)
+    dense = torch.nn.Linear(cols, rows, dtype=torch.bfloat16)
+    dense.weight.data.copy_((torch.randn(rows, cols) * 0.02).to(torch.bfloat16))
+    dense.bias.data.copy_((torch.randn(rows) * 0.01).to(torch.bfloat16))
+    options = {} if tile_elements is None else {"tile_elements": tile_elements}
+    config = ep.EntroPackLossyConfig(target_bpp=4.0, execution_backend="eager", **options)
+    layers = {mode: ep.CompressedINT8Linear.from_linear(dense, config=config, forward_mode=mode).cuda() for mode in ("decode_then_gemm", "fused_through_lds")}
+    layers["fused_through_lds"].load_state_dict(layers["decode_then_gemm"].state_dict())
+    codes = layers["decode_then_gemm"].codes("cuda")
+    for m in activation_rows:
+        print("case int8 fused through LDS", (rows, cols, tile_elements), "M =", m, flush=True)
+        x = torch.randn(m, cols).to(torch.bfloat16).cuda()
+        expect = layers["decode_then_gemm"](x)
+        got = layers["fused_through_lds"](x)
+        torch.cuda.synchronize()
+        assert got.shape == (m, rows) and got.dtype == torch.bfloat16
+        assert torch.equal(got, expect), (m, (got.float() - expect.float()).abs().max().item())
+        qa, sa = kernels.quantize_rows(x)
+        exact = (qa.double() @ codes.double().T).float()
+        definition = exact * sa.unsqueeze(1) * layers["decode_then_gemm"].weight_quant_scale.cuda().unsqueeze(0) + dense.bias.data.cuda().float()
+        assert torch.equal(got, definition.to(torch.bfloat16))
+    container = layers["fused_through_lds"]._container().to(device="cuda")
+    hip_lane.check_errors(packed_buffers(container.buffers, LatticeBuffers))
