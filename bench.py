@@ -281,6 +281,7 @@ def int8_linear_section(ep, steps):
     # with two arenas every pass decodes every layer. `beside` = on a second stream while the previous group multiplies,
     # `in_line` = on the layers' own stream between two groups (one arena).
     import copy
+    layer.forward_mode = "decode_then_gemm"                # the stack is the layer in its default mode
     stack = [copy.deepcopy(layer).cuda() for _ in range(48)]
 
     def forward():

@@ -31,6 +31,8 @@ constexpr int kRingBytes = kRingWords * 2;
 constexpr int kChunkWords = 64;
 
 void set_runtime_error(hipError_t e);
+// Address of the current device's static accumulator (ep_hip_linear_fused_bf16_static), resolved on first use per device.
+int static_accumulator(float** address);
 
 #define EP_HIP_TRY(expr)                         \
   do {                                           \

@@ -480,14 +480,16 @@ static int linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev,
 }
 
 // The accumulator of ep_hip_linear_fused_bf16_static: one copy per GPU, held until the process ends. In host code the
-// array's name is only a handle; its device address comes from hipGetSymbolAddress, once per device.
+// array's name is only a handle; its device address comes from hipGetSymbolAddress, once per device: by
+// ep_hip_device_query for the device that is current then (the library's set-up call, outside any stream capture), else by
+// the entry point's first call on the device.
 static __device__ __align__(256) float scratch[EP_HIP_STATIC_ACCUMULATOR_FLOATS];
 
 constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_lock;
 static float* g_scratch_of_device[kMaxDevices];      // device ordinal -> address of that device's `scratch`
 
-static int static_accumulator(float** address) {
+int static_accumulator(float** address) {
   int device = 0;
   EP_HIP_TRY(hipGetDevice(&device));
   if (device < 0 || device >= kMaxDevices) return EP_HIP_EUNSUPPORTED;

@@ -641,6 +641,8 @@ extern "C" int ep_hip_encode_offsets(const uint32_t* tile_words_dev, int64_t til
 extern "C" int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int64_t stride_words,
                                     uint16_t* payload_dev, void* stream) {
   if (scratch_dev == nullptr || offsets_dev == nullptr || payload_dev == nullptr || tiles <= 0 || stride_words <= 0) return EP_HIP_EINVAL;
+  // The kernel stores pairs of words: the payload must start on four bytes.
+  if (reinterpret_cast<uintptr_t>(payload_dev) % 4 != 0) return EP_HIP_EINVAL;
   int blocks = 0;
   const int status = ep::grid_for(tiles, 1, &blocks);
   if (status != EP_HIP_OK) return status;

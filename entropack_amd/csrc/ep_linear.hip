@@ -236,6 +236,67 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const void* __restri
   if (threadIdx.x == 0) scales[row] = scale;
 }
 
+// Plain quantisation of two-byte activations, one wave per row (four rows per block): no LDS, no barrier, the row read
+// once with fully coalesced 16-byte loads (chunk c of lane l holds elements 8 (64 c + l) .. + 8) and kept packed in
+// registers between the absmax and the codes. The codes are rint(v / scale) with IEEE division by definition; dividing
+// 12 M activations costs more vector instructions than everything else in this kernel together, so a chunk first forms
+// t = v * (1 / scale), which lies within 127.5 * 2^-23 of the true quotient, as does the correctly rounded quotient itself:
+// unless t is closer than 2^-14 to a half-integer the two round to the same integer. Chunks in which some lane's value is
+// that close (about one in sixteen) are redone with the division; the result is the definition's, bit for bit, either way.
+template <int IN_KIND, int CHUNKS>
+__global__ __launch_bounds__(256) void quantize_rows_wave_kernel(const uint16_t* __restrict__ x, int64_t ldx, int K, int rows,
+                                                                 int8_t* __restrict__ codes, float* __restrict__ scales) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63;
+  const int64_t row = blockIdx.x * int64_t{4} + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint16_t* from = x + row * ldx;
+  auto value = [](uint32_t word, int high) -> float {
+    const uint32_t bits = high ? word >> 16 : word & 0xFFFFu;
+    if constexpr (IN_KIND == kOutBF16) return __uint_as_float(bits << 16);
+    else return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
+  };
+  u32x4 held[CHUNKS];
+  float top = 0.0f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int k = 8 * (64 * c + lane);
+    held[c] = u32x4{0u, 0u, 0u, 0u};
+    if (k < K) held[c] = *reinterpret_cast<const u32x4*>(from + k);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) top = __builtin_fmaxf(top, __builtin_fabsf(value(held[c][i >> 1], i & 1)));
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) top = __builtin_fmaxf(top, __shfl_xor(top, offset));
+  const float scale = __builtin_fmaxf(top / 127.0f, 1.1920928955078125e-07f);
+  const float inverse = 1.0f / scale;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int k = 8 * (64 * c + lane);
+    float code[8];
+    float nearest_half = 0.0f;               // the largest |t - rint(t)| of the chunk: 0.5 at a half-integer
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float t = __fmul_rn(value(held[c][i >> 1], i & 1), inverse);
+      code[i] = __builtin_rintf(t);
+      nearest_half = __builtin_fmaxf(nearest_half, __builtin_fabsf(t - code[i]));
+    }
+    if (__builtin_amdgcn_ballot_w64(nearest_half > 0.5f - 0.00006103515625f) != 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) code[i] = __builtin_rintf(value(held[c][i >> 1], i & 1) / scale);
+    }
+    u32x2 packed = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = static_cast<int>(__builtin_fminf(__builtin_fmaxf(code[i], -127.0f), 127.0f));
+      packed[i >> 2] |= (static_cast<uint32_t>(q) & 0xFFu) << (8 * (i & 3));
+    }
+    if (k < K) *reinterpret_cast<u32x2*>(codes + row * K + k) = packed;
+  }
+  if (lane == 0) scales[row] = scale;
+}
+
 // The same with an optional block rotation in front (entropack/linear/convrot.py:34-53 of the reference: activations
 // are multiplied, group by group, with the Kronecker power of the 4 x 4 matrix 1 - 2 * antidiagonal, divided by
 // sqrt(group), the product rounded to the activation dtype, and then quantised). The matrix is symmetric and every
@@ -1158,6 +1219,27 @@ int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K
   using namespace ep;
   if (x_dev == nullptr || codes_dev == nullptr || scales_dev == nullptr) return EP_HIP_EINVAL;
   if (rows <= 0 || K <= 0 || rows > 0x7FFFFFFF || K > 0x7FFFFFFF || ldx < K || !out_kind_valid(in_kind)) return EP_HIP_EINVAL;
+  // Two-byte activations in whole 16-byte pieces: one wave per row.
+  if (in_kind != kOutF32 && K % 8 == 0 && K <= 8192 && ldx % 8 == 0 && reinterpret_cast<uintptr_t>(x_dev) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(codes_dev) % 8 == 0) {
+    const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint16_t* x = static_cast<const uint16_t*>(x_dev);
+    const int k = static_cast<int>(K), m = static_cast<int>(rows);
+#define EP_QUANTISE_WAVE(KIND, CHUNKS) hipLaunchKernelGGL((quantize_rows_wave_kernel<KIND, CHUNKS>), grid, dim3(256), 0, s, x, ldx, k, m, codes_dev, scales_dev)
+    if (in_kind == kOutBF16) {
+      if (K <= 2048) EP_QUANTISE_WAVE(kOutBF16, 4);
+      else if (K <= 4096) EP_QUANTISE_WAVE(kOutBF16, 8);
+      else EP_QUANTISE_WAVE(kOutBF16, 16);
+    } else {
+      if (K <= 2048) EP_QUANTISE_WAVE(kOutF16, 4);
+      else if (K <= 4096) EP_QUANTISE_WAVE(kOutF16, 8);
+      else EP_QUANTISE_WAVE(kOutF16, 16);
+    }
+#undef EP_QUANTISE_WAVE
+    EP_HIP_TRY(hipGetLastError());
+    return EP_HIP_OK;
+  }
   if (rows_take_wide_loads(x_dev, in_kind, K, ldx, codes_dev)) return launch_rotate_quantize(x_dev, in_kind, rows, K, ldx, 0, codes_dev, scales_dev, stream);
   hipLaunchKernelGGL(quantize_rows_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      x_dev, in_kind, ldx, static_cast<int>(K), codes_dev, scales_dev);

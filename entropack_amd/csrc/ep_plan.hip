@@ -252,7 +252,17 @@ int ep_hip_device_query(int device, ep_hip_device_info* info) {
   info->lds_bytes_per_block = lds;
   strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
   info->is_gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
-  return info->is_gfx950 ? EP_HIP_OK : EP_HIP_ENODEVICE;
+  if (!info->is_gfx950) return EP_HIP_ENODEVICE;
+  // Set-up for the entry point that allocates nothing: its accumulator's address on this device is looked up here, outside
+  // any stream capture, when the queried device is the current one (a symbol lookup may load the code object, which a
+  // capture in progress does not survive).
+  int current = -1;
+  if (hipGetDevice(&current) == hipSuccess && current == device) {
+    float* unused = nullptr;
+    const int status = ep::static_accumulator(&unused);
+    if (status != EP_HIP_OK) return status;
+  }
+  return EP_HIP_OK;
 }
 
 int ep_hip_plan_describe(const int32_t* meta, const uint16_t* freq, size_t n_freq, int prob_bits, int tile_elements,

@@ -12,6 +12,7 @@ validation walks that list.
 import dataclasses
 import numbers
 import typing
+import weakref
 
 __all__ = ["CompressionConfig", "OneOf", "Range", "RawConfig", "validate_config"]
 
@@ -111,15 +112,22 @@ def _rules(config_class: type) -> tuple:
     return _compiled[config_class]
 
 
-_last_valid: list = [None, None]      # the config object validated last and the field values it had then
+_last_valid: tuple = (None, None)      # (a weak reference to the config object validated last, the field values it had then)
 
 
 def validate_config(config) -> None:
-    # A layer validates the same config object on every forward: skip the rules while its fields are unchanged.
+    # A layer validates the same config object on every forward: skip the rules while its fields are unchanged. The pair
+    # is one tuple, read and replaced in one step, so two threads validating different configs can never pair one config's
+    # identity with the other's fields; the config itself is held weakly.
+    global _last_valid
     fields = getattr(config, "__dict__", None)
-    if fields is not None and _last_valid[0] is config and _last_valid[1] == fields:
+    seen, seen_fields = _last_valid
+    if fields is not None and seen is not None and seen() is config and seen_fields == fields:
         return
     for rule in _rules(type(config)):
         rule.apply(getattr(config, rule.name))
     if fields is not None:
-        _last_valid[0], _last_valid[1] = config, dict(fields)
+        try:
+            _last_valid = (weakref.ref(config), dict(fields))
+        except TypeError:          # a config type without weak references: validated every time
+            pass

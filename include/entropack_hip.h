@@ -257,7 +257,9 @@ int ep_hip_linear_fused_bf16(const ep_hip_decode_job* weight, const void* x_dev,
  * until the process ends) instead of a caller's workspace. Nothing is allocated or freed, here or in any routine it
  * calls. m_rows * weight->rows above EP_HIP_STATIC_ACCUMULATOR_FLOATS returns EP_HIP_ETOOLARGE. Every call on a GPU
  * uses that GPU's one array (cleared by a kernel at the start of each call): calls that overlap on one GPU, from
- * different streams or threads, race; calls on one stream, or otherwise ordered, are safe.
+ * different streams or threads, race; calls on one stream, or otherwise ordered, are safe. The array's address on a
+ * device is looked up by ep_hip_device_query (when that device is current) or by the first call on the device: one of
+ * the two must have happened before a call is captured into a HIP graph.
  * No counterpart in the reference, whose lane allocates its outputs with torch.empty
  * (entropack/schemes/lattice_rans/cuda.py:794). */
 #define EP_HIP_STATIC_ACCUMULATOR_FLOATS (1 << 18)
@@ -372,7 +374,8 @@ int ep_hip_encode_rans(const int8_t* coset_dev, const int32_t* fields_dev, int64
 int ep_hip_encode_offsets(const uint32_t* tile_words_dev, int64_t tiles, uint32_t* offsets_dev, uint64_t* total_words_dev, void* stream);
 
 /* payload_dev[offsets_dev[t] ..) = the words stream t left at scratch_dev[t * stride_words ..): stride_words =
- * tile_vectors * 9 after ep_hip_encode_rans, the scratch stride after ep_hip_tile_ans_encode. Replaces cuda.py:552-557
+ * tile_vectors * 9 after ep_hip_encode_rans, the scratch stride after ep_hip_tile_ans_encode; payload_dev 4-byte
+ * aligned (EP_HIP_EINVAL otherwise: words are stored in pairs). Replaces cuda.py:552-557
  * (e8_compact_kernel, lattice_rans.cu:467) and tile_ans/cuda.py:110-115 (tile_ans_compact_kernel, tile_ans.cu:157). */
 int ep_hip_encode_gather(const uint16_t* scratch_dev, const uint32_t* offsets_dev, int64_t tiles, int64_t stride_words,
                          uint16_t* payload_dev, void* stream);

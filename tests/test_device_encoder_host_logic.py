@@ -97,9 +97,24 @@ def test_entry_points_refuse_bad_arguments_before_touching_a_device():
     assert lib.ep_hip_encode_offsets(a, 0, a, a, None) == hip.EINVAL
     assert lib.ep_hip_encode_offsets(a, 4, a, a + 4, None) == hip.EINVAL
     assert lib.ep_hip_encode_gather(a, a, 4, 0, a, None) == hip.EINVAL
+    assert lib.ep_hip_encode_gather(a, a, 4, 8, a + 2, None) == hip.EINVAL            # a payload that starts on two bytes
     assert lib.ep_hip_tile_ans_histogram(a, 16, 3, a, None) == hip.EUNSUPPORTED
     assert lib.ep_hip_tile_ans_histogram(a + 1, 16, 2, a, None) == hip.EINVAL
     raw = (ctypes.c_uint8 * 2)(1, 0)
     assert lib.ep_hip_tile_ans_encode(a, 16, 2, 8, 10, a, raw, None, a, a, 8, a, None) == hip.EINVAL       # a coded lane needs states
     assert lib.ep_hip_tile_ans_encode(a, 16, 2, 8, 10, a, raw, a, a, a, 4, a, None) == hip.EINVAL          # stride below the tile
     assert lib.ep_hip_tile_ans_encode(a, 16, 5, 8, 10, a, raw, a, a, a, 8, a, None) == hip.EUNSUPPORTED
+
+
+def test_both_encoder_lanes_price_with_the_cpu_lanes_size_model():
+    """The device lane drives the CPU lane's scale search (`eager.resolve_scale`) and therefore its size model: coded bytes
+    + 4 bytes per row + 64 (layout) + 408 (stream_meta) + 384 (slack), the constants of the reference's eager lane
+    (entropack/schemes/lattice_rans/eager.py:102-107 there). The reference's CUDA lane prices without the last two
+    (cuda.py:224), so a device-encoded container follows the CPU lane, not the reference's device lane; on small layers the
+    settled rate differs by (408 + 384) * 8 / weights bits per weight."""
+    import inspect
+
+    from entropack_amd.schemes.lattice_rans import eager, hip_encode
+    assert (eager.MODEL_LAYOUT_BYTES, eager.MODEL_STREAM_META_BYTES, eager.MODEL_SLACK_BYTES) == (64, 408, 384)
+    assert "resolve_scale" in inspect.getsource(hip_encode)            # the device lane has no size model of its own
+    assert "MODEL_" not in inspect.getsource(hip_encode)

@@ -354,6 +354,35 @@ def test_rotate_quantize_rows_on_exactly_representable_sums(group, rows, inner, 
     assert torch.equal(codes.cpu(), expect_codes)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_quantize_rows_of_two_byte_activations_is_the_divisions_answer_for_every_value(dtype):
+    """The kernel for bfloat16 / float16 rows multiplies by 1 / scale and falls back to the division only where the product
+    lies within 2^-14 of a half-integer. Rows whose maxima give scales that are no powers of two, filled with every value
+    of the dtype up to the row's maximum (bfloat16: all of them; float16: every fourth), must come out as IEEE division,
+    rint and clamp say, code for code."""
+    bits = torch.arange(0, 0x7F80 if dtype == torch.bfloat16 else 0x7C00, 1 if dtype == torch.bfloat16 else 4, dtype=torch.int32)
+    values = bits.to(torch.int16).view(dtype)
+    tops = torch.tensor([0.37, 1.0, 3.1, 200.0, 1000.0, 4.4e-3, 77.0, 130.0, 513.0, 2.0e4], dtype=torch.float32).to(dtype)
+    inner = 8192
+    rows = []
+    for top in tops:
+        below = values[values.float() <= top.float()]
+        signed = torch.cat([below, -below])
+        pad = (-signed.numel()) % (inner - 1)
+        signed = torch.cat([signed, signed.repeat(pad // signed.numel() + 1)[:pad]])
+        block = signed.view(-1, inner - 1)
+        rows.append(torch.cat([top.expand(block.shape[0], 1), block], dim=1))          # column 0 pins the row's maximum
+    x = torch.cat(rows).contiguous().cuda()
+    codes, scale = kernels.quantize_rows(x)
+    flat = x.float().cpu()
+    expect_scale = (flat.abs().amax(dim=1) / torch.tensor(127.0)).clamp(min=torch.finfo(torch.float32).eps)
+    expect_codes = (flat / expect_scale.unsqueeze(1)).round().clamp(-127, 127).to(torch.int8)
+    assert torch.equal(scale.cpu(), expect_scale)
+    assert torch.equal(codes.cpu(), expect_codes)
+    naive = (flat * (1.0 / expect_scale).unsqueeze(1)).round().clamp(-127, 127).to(torch.int8)
+    print("values a reciprocal multiply alone gets wrong:", int((naive != expect_codes).sum()), "of", naive.numel(), flush=True)
+
+
 @pytest.mark.parametrize("group,rows,inner,dtype", [(256, 4096, 3072, torch.bfloat16), (64, 17, 3136, torch.bfloat16), (16, 9, 1008, torch.float16),
                                                     (4, 3, 4100, torch.float32), (256, 128, 28672, torch.bfloat16)])
 def test_rotate_quantize_rows_on_gaussian_rows_with_outliers(group, rows, inner, dtype):

@@ -98,3 +98,36 @@ def test_static_accumulator_entry_point_rejects_what_does_not_fit():
     job.rows = 256
     assert call(256, 4) == hip.OK
     torch.cuda.synchronize()
+
+
+def test_static_accumulator_entry_point_inside_a_hip_graph():
+    """The entry point's advertised use: captured into a graph (kernel nodes only, nothing allocated), replayed with eager
+    work in between; every replay gives the eager call's result. The library's device query has looked the accumulator's
+    address up beforehand (`hip.device_info`), so the first call may already be the captured one."""
+    print("case static accumulator under graph capture: 512x1024 m=3", flush=True)
+    packed, dense = _container(512, 1024, seed=47)
+    job, keep = _job(packed)
+    hip.device_info(torch.cuda.current_device())
+    library = hip.library()
+    x = torch.randn(3, 1024, device="cuda").to(torch.bfloat16)
+    y = torch.zeros(3, 512, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            hip.check("ep_hip_linear_fused_bf16_static", library.ep_hip_linear_fused_bf16_static(
+                ctypes.byref(job), x.data_ptr(), 3, x.stride(0), None, y.data_ptr(), y.stride(0), hip.FLOAT_KINDS[torch.bfloat16],
+                hip.current_stream(x.device)))
+    torch.cuda.current_stream().wait_stream(side)
+    expect = F.linear(x.float(), dense.float()).to(torch.bfloat16)
+    for replay in range(3):
+        y.zero_()
+        x.copy_(torch.randn(3, 1024, device="cuda").to(torch.bfloat16))
+        expect = F.linear(x.float(), dense.float())
+        graph.replay()
+        torch.cuda.synchronize()
+        error = ((y.double() - expect.to(torch.bfloat16).double()).norm() / expect.double().norm()).item()
+        assert error <= REL_L2, (replay, error)
+        _ = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")       # eager work between the replays
+    lane.check_errors(keep[0])
