@@ -830,6 +830,146 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(
   store_wave_tile<INT8, false, NJ, Acc, RAGGED>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
 }
 
+// ---- 128 x 128 tiles with four stages: products of few blocks whose operands come from memory ---------------------------
+//
+// The two-stage 128 x 128 kernel above keeps one K step of loads (32 KB) in flight per block, which covers the L2's latency
+// but not memory's: on a weight that has just been decoded (it is in no cache) 256 x 3072 x 3072 took 46 us where the same
+// product on cached operands took 25 us. When a product has at most one such block per CU there is no second block for
+// the LDS anyway, so this variant spends it on depth: four stages of 32 KB, the tile three steps ahead requested while a
+// step is multiplied (96 KB in flight per block). The wait before the barrier that publishes a stage is counted: the 16
+// loads issued after that stage's own may still be in flight. Everything else (piece permutation, fragment reads a slice
+// ahead, slab epilogue) is the two-stage kernel's.
+// SPLIT: the grid's z blocks share a tile, each taking gridDim.z-th of K; the sums go, as they are (f32, or int32 for int8), to
+// slab blockIdx.z of `y` ([slice][M][N]) for the kernel that adds the slices, and scales, bias and out_kind are not used.
+template <bool INT8, bool RAGGED, bool SPLIT>
+__global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                          const float* __restrict__ scale_a, const float* __restrict__ scale_b,
+                                                          const void* __restrict__ bias, void* __restrict__ y, int M, int N, int64_t k_bytes,
+                                                          int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind) {
+  constexpr int BM = 128, BN = 128, kWaves = 4, WN = 64, NJ = 2;
+  constexpr int kRowBytes = kTileBytesK;
+  constexpr int kStage = (BM + BN) * kRowBytes;              // 32 KB
+  __shared__ __align__(1024) uint8_t stage0[kStage];
+  __shared__ __align__(1024) uint8_t stage1[kStage];
+  __shared__ __align__(1024) uint8_t stage2[kStage];
+  __shared__ __align__(1024) uint8_t stage3[kStage];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int kLoadsA = BM / (8 * kWaves), kLoadsB = BN / (8 * kWaves), kLoads = kLoadsA + kLoadsB;      // 4 + 4 pieces of 1 KiB per wave and tile
+  const int wave_m = wave / 2, wave_n = wave % 2;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int64_t steps = k_bytes / kTileBytesK / (SPLIT ? gridDim.z : 1);           // this block's
+  const int64_t k_first = SPLIT ? blockIdx.z * steps * kTileBytesK : 0;
+
+  const uint8_t* source[kLoads];
+#pragma unroll
+  for (int c = 0; c < kLoads; ++c) {
+    const bool of_a = c < kLoadsA;
+    const int row = 8 * (wave + kWaves * (of_a ? c : c - kLoadsA)) + (lane >> 3);
+    const int piece = (lane & 7) ^ ((row >> 1) & 7);
+    int from_row = (of_a ? m0 : n0) + row;
+    if (RAGGED && from_row >= (of_a ? M : N)) from_row = (of_a ? M : N) - 1;
+    source[c] = (of_a ? a + from_row * lda_bytes + 16 * piece : b + from_row * ldb_bytes + 16 * piece) + k_first;
+  }
+  auto load_one = [&](uint8_t* stage, int64_t kb, int c) {
+    const bool of_a = c < kLoadsA;
+    const int first_row = (of_a ? 0 : BM) + 8 * (wave + kWaves * (of_a ? c : c - kLoadsA));
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(source[c] + kb),
+                                     (__attribute__((address_space(3))) void*)(stage + first_row * kRowBytes), 16, 0, 0);
+  };
+
+  using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
+  using Frag = typename std::conditional<INT8, i32x4, bf16x8>::type;
+  Acc acc[2][NJ] = {};
+  constexpr int kReads = 2 + NJ, kMultiplies = 2 * NJ;
+  Frag frag[2][kReads];
+  const int frag_row = lane & 31;
+  const int turn = (frag_row >> 1) & 7;
+  const uint32_t frag_a_at = static_cast<uint32_t>((wave_m * 64 + frag_row) * kRowBytes);
+  const uint32_t frag_b_at = static_cast<uint32_t>((BM + wave_n * WN + frag_row) * kRowBytes);
+  auto read_one = [&](int set, const uint8_t* stage, int kk, int t) {
+    const uint32_t place = static_cast<uint32_t>(((2 * kk + (lane >> 5)) ^ turn) * 16);
+    const uint32_t at = place + (t < 2 ? frag_a_at + t * 32 * kRowBytes : frag_b_at + (t - 2) * 32 * kRowBytes);
+    frag[set][t] = *reinterpret_cast<const Frag*>(stage + at);
+  };
+  auto multiply_one = [&](int set, int m) {
+    const int i = m / NJ, j = m % NJ;
+    if constexpr (INT8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+    else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+  };
+
+  auto tile_at = [&](int64_t t) { return (t < steps ? t : steps - 1) * kTileBytesK; };
+  // One K step on `here`; `there` is read next; `fill` (read in the step before this one) takes the tile three steps ahead,
+  // three, three and two of its eight pieces per slice. Past the last tile the loads repeat the last one, which nobody reads.
+  auto k_step = [&](uint8_t* here, uint8_t* there, uint8_t* fill, int64_t step) {
+    const int64_t ahead = tile_at(step + 3);
+#pragma unroll
+    for (int slice = 0; slice < 3; ++slice) {
+#pragma unroll
+      for (int m = 0; m < kMultiplies; ++m) {
+        multiply_one(slice & 1, m);
+        const int piece = 3 * slice + m;
+        if (m < 3 && piece < kLoads) load_one(fill, ahead, piece);
+        if (m < kReads) read_one((slice & 1) ^ 1, here, slice + 1, m);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // `there` holds the tile of the next step, requested two steps ago: the 16 loads issued since may still be in flight.
+    // A bare barrier: the fence of __syncthreads() makes the compiler wait for every load into LDS, which would empty the
+    // pipeline at each step. This wave's fragment reads of `here` are complete (lgkmcnt 0) before it arrives, so no wave
+    // can overwrite a stage that another still reads.
+    __builtin_amdgcn_s_waitcnt(0x4070);                     // vmcnt(16), lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int m = 0; m < kMultiplies; ++m) {
+      multiply_one(1, m);
+      if (m < kReads) read_one(0, there, 0, m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+#pragma unroll
+  for (int c = 0; c < kLoads; ++c) load_one(stage0, 0, c);
+#pragma unroll
+  for (int c = 0; c < kLoads; ++c) load_one(stage1, tile_at(1), c);
+#pragma unroll
+  for (int c = 0; c < kLoads; ++c) load_one(stage2, tile_at(2), c);
+  __builtin_amdgcn_s_waitcnt(0x4F70);                       // vmcnt(16): the first tile has landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int t = 0; t < kReads; ++t) read_one(0, stage0, 0, t);
+  for (int64_t step = 0; step < steps; step += 4) {
+    k_step(stage0, stage1, stage3, step);            // the launcher takes only K of a whole number of four steps: a branch
+    k_step(stage1, stage2, stage0, step + 1);        // between the steps would make the compiler's wait-count pass forget which
+    k_step(stage2, stage3, stage1, step + 2);        // stage each load in flight fills, and wait for all of them
+    k_step(stage3, stage0, stage2, step + 3);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();     // every load has landed and every fragment is read before the slabs below reuse a stage
+
+  if constexpr (SPLIT) {
+    // Register r of lane l holds row 8 (r / 4) + 4 (l / 32) + r % 4 and column l % 32 of its 32 x 32 tile.
+    using Cell = typename std::conditional<INT8, int32_t, float>::type;
+    Cell* out = static_cast<Cell*>(y) + static_cast<int64_t>(blockIdx.z) * M * N;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int n = n0 + wave_n * WN + j * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wave_m * 64 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+          if (!RAGGED || (m < M && n < N)) out[static_cast<int64_t>(m) * N + n] = acc[i][j][r];
+        }
+      }
+    }
+  } else {
+    static_assert(4 * 32 * WN * 4 <= kStage, "four slabs fit into one stage");
+    float* slab = reinterpret_cast<float*>(stage0) + wave * (32 * WN);
+    store_wave_tile<INT8, false, NJ, Acc, RAGGED>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
+  }
+}
+
 template <bool INT8, bool GUARD, int BN>
 static int launch_big_variant(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                       int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
@@ -893,6 +1033,21 @@ template <bool INT8>
 static int launch_direct_small(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                                int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>((N + 127) / 128), static_cast<unsigned>((M + 127) / 128));
+  // At most one block per CU (the deep kernel holds 128 KB of LDS) and K a whole number of four steps, which is what its loop runs.
+  int device = 0, cus = 0;
+  if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
+#ifndef EP_NO_DEEP_TILES
+  if (static_cast<int64_t>(grid.x) * grid.y <= cus && k_bytes % (4 * kTileBytesK) == 0) {
+    if (M % 128 == 0 && N % 128 == 0)
+      hipLaunchKernelGGL((gemm_deep_kernel<INT8, false, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                         scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
+    else
+      hipLaunchKernelGGL((gemm_deep_kernel<INT8, true, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                         scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
+    EP_HIP_TRY(hipGetLastError());
+    return EP_HIP_OK;
+  }
+#endif
   if (M % 128 == 0 && N % 128 == 0)
     hipLaunchKernelGGL((gemm_direct_kernel<INT8, 128, 128, 2, 2, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a),
                        static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
@@ -1047,6 +1202,68 @@ __global__ __launch_bounds__(256) void gemm_skinny_finish_kernel(const void* __r
   store_out(y, out_kind, static_cast<int64_t>(m) * ldy + n, v);
 }
 
+// The same sums and roundings, four consecutive cells of a row per thread (16-byte loads of the slabs, one store of the
+// four results): for N and ldy multiples of 4 and y aligned to four outputs.
+template <bool INT8>
+__global__ __launch_bounds__(256) void gemm_finish_quads_kernel(const void* __restrict__ partial, int slices, const float* __restrict__ scale_a,
+                                                                const float* __restrict__ scale_b, const void* __restrict__ bias,
+                                                                void* __restrict__ y, int M, int N, int64_t ldy, int out_kind) {
+  const int64_t cell = 4 * (blockIdx.x * int64_t{256} + threadIdx.x);
+  const int64_t cells = static_cast<int64_t>(M) * N;
+  if (cell >= cells) return;
+  const int m = static_cast<int>(cell / N), n = static_cast<int>(cell % N);
+  float v[4];
+  if constexpr (INT8) {
+    int4 sum = make_int4(0, 0, 0, 0);
+    for (int s = 0; s < slices; ++s) {
+      const int4 p = *reinterpret_cast<const int4*>(static_cast<const int32_t*>(partial) + static_cast<int64_t>(s) * cells + cell);
+      sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+    }
+    const int32_t sums[4] = {sum.x, sum.y, sum.z, sum.w};
+    const float sa = scale_a[m];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = __fmul_rn(__fmul_rn(static_cast<float>(sums[i]), sa), scale_b[n + i]);
+      if (bias != nullptr) v[i] = __fadd_rn(v[i], load_bias(bias, out_kind, n + i));
+    }
+  } else {
+    float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int s = 0; s < slices; ++s) {
+      const float4 p = *reinterpret_cast<const float4*>(static_cast<const float*>(partial) + static_cast<int64_t>(s) * cells + cell);
+      sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+    }
+    v[0] = sum.x; v[1] = sum.y; v[2] = sum.z; v[3] = sum.w;
+    if (bias != nullptr) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] += load_bias(bias, out_kind, n + i);
+    }
+  }
+  const int64_t at = static_cast<int64_t>(m) * ldy + n;
+  if (out_kind == kOutF32) {
+    *reinterpret_cast<float4*>(static_cast<float*>(y) + at) = make_float4(v[0], v[1], v[2], v[3]);
+  } else if (out_kind == kOutBF16) {
+    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + at) =
+        make_uint2(bf16_bits_of(v[0]) | bf16_bits_of(v[1]) << 16, bf16_bits_of(v[2]) | bf16_bits_of(v[3]) << 16);
+  } else {
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    half4 h = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1]), static_cast<_Float16>(v[2]), static_cast<_Float16>(v[3])};
+    *reinterpret_cast<half4*>(static_cast<_Float16*>(y) + at) = h;
+  }
+}
+
+template <bool INT8>
+static void launch_finish(const void* partial, int slices, const float* scale_a, const float* scale_b, const void* bias, void* y, int M, int N,
+                          int64_t ldy, int out_kind, hipStream_t s) {
+  const int64_t cells = static_cast<int64_t>(M) * N;
+  const uintptr_t four_outputs = out_kind == kOutF32 ? 16 : 8;
+  if (N % 4 == 0 && ldy % 4 == 0 && reinterpret_cast<uintptr_t>(y) % four_outputs == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0)
+    hipLaunchKernelGGL(gemm_finish_quads_kernel<INT8>, dim3(static_cast<unsigned>((cells / 4 + 255) / 256)), dim3(256), 0, s, partial, slices,
+                       scale_a, scale_b, bias, y, M, N, ldy, out_kind);
+  else
+    hipLaunchKernelGGL(gemm_skinny_finish_kernel<INT8>, dim3(static_cast<unsigned>((cells + 255) / 256)), dim3(256), 0, s, partial, slices,
+                       scale_a, scale_b, bias, y, M, N, ldy, out_kind);
+}
+
 // K slices for an M x N product with `k_bytes` bytes per row on `cus` compute units: enough blocks for about four
 // per CU, at least one chunk each.
 static int skinny_slices(int64_t N, int64_t k_bytes, int cus) {
@@ -1076,9 +1293,47 @@ static int launch_skinny(const void* x, const void* w, const float* scale_a, con
   else if (M <= 96) hipLaunchKernelGGL((gemm_skinny_kernel<3, INT8>), grid, dim3(256), 0, s, xb, wb, workspace, m, n, k_bytes, ldx_bytes, ldw_bytes, per);
   else hipLaunchKernelGGL((gemm_skinny_kernel<4, INT8>), grid, dim3(256), 0, s, xb, wb, workspace, m, n, k_bytes, ldx_bytes, ldw_bytes, per);
   EP_HIP_TRY(hipGetLastError());
-  const int64_t cells = M * N;
-  hipLaunchKernelGGL(gemm_skinny_finish_kernel<INT8>, dim3(static_cast<unsigned>((cells + 255) / 256)), dim3(256), 0, s, workspace, slices,
-                     scale_a, scale_b, bias, y, m, n, ldy, out_kind);
+  launch_finish<INT8>(workspace, slices, scale_a, scale_b, bias, y, m, n, ldy, out_kind, s);
+  EP_HIP_TRY(hipGetLastError());
+  return EP_HIP_OK;
+}
+
+// ---- a few hundred activation rows: 128 x 128 tiles with K split over blocks ----------------------------------------------
+//
+// A CU moves operand bytes into its LDS at a bounded rate (about 80 GB/s when they come from the last-level cache and 55-60
+// GB/s from memory on an MI355X: a bounded number of requests in flight, over the latency). A 128 x 128 tile of a product
+// with K = 3072 takes 1.5 MB of operands, 19 us at the first rate and 27-32 us at the second, whatever the pipeline's
+// depth, and a product of 48 such tiles leaves four CUs in five idle meanwhile. So when the tiles are at most half as many
+// as the CUs, K is divided over `slices` blocks per tile (the four-stage kernel above with SPLIT), each CU moves 1 / slices
+// of the bytes, and the kernel that adds the skinny product's slices adds these.
+static int split_slices(int64_t M, int64_t N, int64_t k_bytes, int cus) {
+  if (M <= 128 || k_bytes % kTileBytesK != 0) return 0;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  const int64_t steps = k_bytes / kTileBytesK;
+  int64_t most = cus / tiles;
+  most = most > 8 ? 8 : most;
+  for (int64_t slices = most; slices >= 2; --slices)
+    if (steps % (4 * slices) == 0 && steps / slices >= 8) return static_cast<int>(slices);   // whole rounds of the kernel's four-step loop
+  return 0;
+}
+
+template <bool INT8>
+static int launch_split(const void* x, const void* w, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
+                        int64_t N, int64_t k_bytes, int64_t ldx_bytes, int64_t ldw_bytes, int64_t ldy, int out_kind, int slices,
+                        void* workspace, size_t workspace_bytes, hipStream_t s) {
+  if (workspace_bytes < static_cast<size_t>(slices) * static_cast<size_t>(M) * static_cast<size_t>(N) * 4) return EP_HIP_EINVAL;
+  const dim3 grid(static_cast<unsigned>((N + 127) / 128), static_cast<unsigned>((M + 127) / 128), static_cast<unsigned>(slices));
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  const uint8_t* wb = static_cast<const uint8_t*>(w);
+  const int m = static_cast<int>(M), n = static_cast<int>(N);
+  if (M % 128 == 0 && N % 128 == 0)
+    hipLaunchKernelGGL((gemm_deep_kernel<INT8, false, true>), grid, dim3(256), 0, s, xb, wb, nullptr, nullptr, nullptr, workspace, m, n, k_bytes,
+                       ldx_bytes, ldw_bytes, int64_t{0}, 0);
+  else
+    hipLaunchKernelGGL((gemm_deep_kernel<INT8, true, true>), grid, dim3(256), 0, s, xb, wb, nullptr, nullptr, nullptr, workspace, m, n, k_bytes,
+                       ldx_bytes, ldw_bytes, int64_t{0}, 0);
+  EP_HIP_TRY(hipGetLastError());
+  launch_finish<INT8>(workspace, slices, scale_a, scale_b, bias, y, m, n, ldy, out_kind, s);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
 }
@@ -1153,7 +1408,8 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
 size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units) {
   using namespace ep;
   if (M <= 0 || N <= 0 || k_bytes <= 0 || compute_units <= 0) return 0;
-  return static_cast<size_t>(skinny_slices(N, k_bytes, compute_units)) * static_cast<size_t>(M) * static_cast<size_t>(N) * 4;
+  const int slices = M <= 128 ? skinny_slices(N, k_bytes, compute_units) : split_slices(M, N, k_bytes, compute_units);
+  return static_cast<size_t>(slices) * static_cast<size_t>(M) * static_cast<size_t>(N) * 4;
 }
 
 int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
@@ -1161,12 +1417,17 @@ int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bi
                             void* workspace_dev, size_t workspace_bytes, void* stream) {
   using namespace ep;
   if (x_dev == nullptr || w_dev == nullptr || y_dev == nullptr || workspace_dev == nullptr) return EP_HIP_EINVAL;
-  if (M <= 0 || N <= 0 || K <= 0 || N > 0x7FFFFFFF || K > 0x3FFFFFFF || compute_units <= 0) return EP_HIP_EINVAL;
-  if (M > 128) return EP_HIP_EUNSUPPORTED;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x3FFFFFFF || compute_units <= 0) return EP_HIP_EINVAL;
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  if (M > 128) {
+    const int slices = split_slices(M, N, K * 2, compute_units);
+    if (slices == 0) return EP_HIP_EUNSUPPORTED;
+    return launch_split<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, slices,
+                               workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+  }
   return launch_skinny<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, compute_units,
                               workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
 }
@@ -1177,12 +1438,17 @@ int ep_hip_gemm_i8_skinny(const int8_t* a_dev, const int8_t* b_dev, const float*
   using namespace ep;
   if (a_dev == nullptr || b_dev == nullptr || scale_a_dev == nullptr || scale_b_dev == nullptr || y_dev == nullptr ||
       workspace_dev == nullptr) return EP_HIP_EINVAL;
-  if (M <= 0 || N <= 0 || K <= 0 || N > 0x7FFFFFFF || K > 0x7FFFFFFF || compute_units <= 0) return EP_HIP_EINVAL;
-  if (M > 128) return EP_HIP_EUNSUPPORTED;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF || compute_units <= 0) return EP_HIP_EINVAL;
   if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
+  if (M > 128) {
+    const int slices = split_slices(M, N, K, compute_units);
+    if (slices == 0) return EP_HIP_EUNSUPPORTED;
+    return launch_split<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, slices,
+                              workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+  }
   return launch_skinny<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, compute_units,
                              workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
 }

@@ -42,11 +42,13 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
     if rows == 0:
         return out.reshape(*x.shape[:-1], outer)
     bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
-    if rows <= SKINNY_MAX_ROWS:
+    with torch.cuda.device(device):
+        lib = _hip.library()
+        cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
+        split_bytes = lib.ep_hip_gemm_skinny_workspace(rows, outer, inner * 2, cus)      # 0: not a product for the K-split kernels
+    if rows <= SKINNY_MAX_ROWS or split_bytes:
         with torch.cuda.device(device):
-            lib = _hip.library()
-            cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
-            workspace = torch.empty(lib.ep_hip_gemm_skinny_workspace(rows, outer, inner * 2, cus), dtype=torch.uint8, device=device)
+            workspace = torch.empty(split_bytes, dtype=torch.uint8, device=device)
             _hip.check("ep_hip_gemm_bf16_skinny", lib.ep_hip_gemm_bf16_skinny(
                 flat.data_ptr(), w.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(), out.data_ptr(),
                 rows, outer, inner, flat.stride(0), w.stride(0), out.stride(0), _hip.FLOAT_KINDS[out_dtype], cus,
@@ -131,11 +133,13 @@ def int8_gemm(activation: torch.Tensor, codes: torch.Tensor, activation_scale: t
         return out
     bias_ready = None if bias is None else bias.to(device=device, dtype=out_dtype).contiguous()
     scale_a, scale_b = activation_scale.float().contiguous(), weight_scale.float().contiguous()
-    if rows <= SKINNY_MAX_ROWS:
+    with torch.cuda.device(device):
+        lib = _hip.library()
+        cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
+        split_bytes = lib.ep_hip_gemm_skinny_workspace(rows, outer, a.shape[1], cus)     # 0: not a product for the K-split kernels
+    if rows <= SKINNY_MAX_ROWS or split_bytes:
         with torch.cuda.device(device):
-            lib = _hip.library()
-            cus = _hip.device_info(device.index if device.index is not None else torch.cuda.current_device()).compute_units
-            workspace = torch.empty(lib.ep_hip_gemm_skinny_workspace(rows, outer, a.shape[1], cus), dtype=torch.uint8, device=device)
+            workspace = torch.empty(split_bytes, dtype=torch.uint8, device=device)
             _hip.check("ep_hip_gemm_i8_skinny", lib.ep_hip_gemm_i8_skinny(
                 a.data_ptr(), b.data_ptr(), scale_a.data_ptr(), scale_b.data_ptr(), None if bias_ready is None else bias_ready.data_ptr(),
                 out.data_ptr(), rows, outer, a.shape[1], a.stride(0), b.stride(0), out.stride(0), _hip.FLOAT_KINDS[out_dtype], cus,

@@ -197,12 +197,18 @@ enum ep_hip_float_kind { EP_FLOAT_BF16 = 0, EP_FLOAT_F16 = 1, EP_FLOAT_F32 = 2 }
 int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
                      int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, void* stream);
 
-/* The same products for at most 128 activation rows, where reading W once bounds the time: K is split over blocks so
- * that every CU streams weights, partial sums (f32, or exact int32 for the int8 product) go to `workspace_dev`
- * (16-byte aligned, at least ep_hip_gemm_skinny_workspace(M, N, bytes of one row of K, compute_units) bytes, contents
- * irrelevant on entry) and a second kernel adds them, applies the same epilogue as ep_hip_gemm_bf16 / ep_hip_gemm_i8
- * and rounds once. Same operand rules as those; M > 128 returns EP_HIP_EUNSUPPORTED. Reference: the F.linear call of
- * CompressedLinear.forward and the int8 GEMM of CompressedINT8Linear at small batch, entropack/linear/linear.py:163-165,
+/* The same products with K split over blocks, for products too small to occupy the device otherwise; partial sums (f32,
+ * or exact int32 for the int8 product) go to `workspace_dev` (16-byte aligned, at least
+ * ep_hip_gemm_skinny_workspace(M, N, bytes of one row of K, compute_units) bytes, contents irrelevant on entry) and a second
+ * kernel adds them, applies the same epilogue as ep_hip_gemm_bf16 / ep_hip_gemm_i8 and rounds once.
+ *  - M <= 128: reading W once bounds the time; blocks of 128 weight rows, K split so that every CU streams weights.
+ *  - M > 128: 128 x 128 tiles (operand tiles loaded straight into LDS, four stages), K split over 2..8 blocks per tile when
+ *    the tiles number at most half the CUs and each block keeps a whole number of four 128-byte K steps, at least eight.
+ *    Where no such split exists ep_hip_gemm_skinny_workspace returns 0 and the entry points EP_HIP_EUNSUPPORTED: the
+ *    product then belongs to ep_hip_gemm_bf16 / ep_hip_gemm_i8.
+ * f32 sums are added in the order of the slices, so a bf16 product can differ from ep_hip_gemm_bf16's in the last bit of
+ * the f32 sum; the int8 product is the same bits. Same operand rules as those entry points. Reference: the F.linear call
+ * of CompressedLinear.forward and the int8 GEMM of CompressedINT8Linear at small batch, entropack/linear/linear.py:163-165,
  * 485-490. */
 size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units);
 int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,

@@ -37,7 +37,9 @@ def within_one_ulp(got, rounded):
                                    (768, 3072, 320), (3072, 3000, 264), (512, 3072, 128),     # 48 whole tiles; 192 ragged ones; too few
                                    (256, 256, 64), (384, 640, 192), (1024, 3072, 320),        # whole 128 x 128 tiles
                                    (300, 1000, 1024), (130, 136, 64), (1000, 3000, 320), (300, 1001, 128),   # overhanging ones
-                                   (3000, 3100, 192)])                                          # overhanging 256 x 192 tiles
+                                   (3000, 3100, 192),                                           # overhanging 256 x 192 tiles
+                                   (256, 3072, 3072), (1024, 3072, 1024), (640, 3072, 256),    # one 128 x 128 tile per CU at most and
+                                   (200, 3000, 2048)])                                          # K of 4n steps: the four-stage kernel
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
     print("case", shape, with_bias, flush=True)
@@ -146,7 +148,8 @@ def test_quantize_rows_is_exact_next_to_rounding_boundaries():
 @pytest.mark.parametrize("shape", [(4096, 3072, 3072), (5, 70, 48), (129, 130, 1040), (4100, 4200, 528), (1, 300, 4112), (128, 1000, 28672),
                                    (33, 257, 16), (4096, 3000, 272), (4096, 4096, 896), (4096, 3072, 128), (4096, 3072, 384),
                                    (768, 3072, 640), (3072, 3000, 272), (256, 128, 128), (384, 640, 384), (1024, 3072, 640),
-                                   (300, 1000, 1024), (130, 129, 128), (3000, 3100, 256)])
+                                   (300, 1000, 1024), (130, 129, 128), (3000, 3100, 256),
+                                   (256, 3072, 3072), (1024, 3072, 512), (200, 3000, 4096)])    # the four-stage kernel, whole and ragged
 def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
     print("case", shape, flush=True)
     m, n, k = shape
