@@ -1,6 +1,6 @@
 """Headline benchmark: lossy (lattice_rans) decode throughput on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|fused_lds|encode|tile_ans_encode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|c2|c5a|c5b|c4|tile_ans|gemm|gemm_phases|fused_lds|encode|tile_ans_encode]
 
 One "step" = one decode of the whole container (entropy decode + E8 reconstruction + BF16 store) from buffers
 already resident in HBM. Prints ONE JSON line. `value` = algorithmic bytes (container bytes read + dense bytes
@@ -702,6 +702,48 @@ def gemm_workload(args, ep):
     return 0
 
 
+def gemm_phases_workload(args, ep):
+    """`--workload gemm_phases [--rows M]`: the N = K = 3072 bf16 product with M activation rows in a fixed dispatch order,
+    for counter and trace runs that have to tell the launches apart. For this library's product, then for the vendor
+    library's: 4 launches on weight 0, 24 on 24 different weights (untimed), then **16 on weight 0** (launches 28..43 of that
+    kernel: operands in the caches), then **24 on the 24 weights in turn** (launches 44..67: the weight comes from memory,
+    453 MB of weights pass between two uses of one). Each timed phase sits between one pair of events."""
+    from torch.nn import functional as F
+    from entropack_amd.linear import kernels
+    torch.manual_seed(0)
+    weights = [(torch.randn(3072, 3072, device="cuda") * 0.02).to(torch.bfloat16) for _ in range(24)]
+    x = torch.randn(args.rows, 3072, device="cuda").to(torch.bfloat16)
+    out = {}
+    for name, product in (("own", lambda w: kernels.gemm_bf16(x, w, None)), ("library", lambda w: F.linear(x, w))):
+        for _ in range(4):
+            product(weights[0])
+        for w in weights:
+            product(w)
+        torch.cuda.synchronize()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        marks[0].record()
+        for _ in range(16):
+            product(weights[0])
+        marks[1].record()
+        torch.cuda.synchronize()
+        marks[2].record()
+        for w in weights:
+            product(w)
+        marks[3].record()
+        torch.cuda.synchronize()
+        out[name] = {"same_weight_us": round(marks[0].elapsed_time(marks[1]) / 16 * 1e3, 2),
+                     "rotating_weights_us": round(marks[2].elapsed_time(marks[3]) / 24 * 1e3, 2)}
+    own = out["own"]["rotating_weights_us"]
+    flops = 2.0 * args.rows * 3072 * 3072
+    print(json.dumps({
+        "metric": f"bf16 GEMM TFLOP/s, {args.rows} x 3072 x 3072, weight from memory, clocks not settled", "value": round(flops / own / 1e6, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": 24, "warmup": 28, "ms_per_step": round(own / 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"y = x W^T, M = {args.rows}, N = K = 3072, bf16: 16 launches on one weight, 24 on 24 weights, own then library",
+                   "phases": out}}))
+    return 0
+
+
 def fused_lds_workload(args, ep):
     """`--workload fused_lds`: configuration 3's layer (W 3072 x 3072 @ 4 bpp + bias, seed 2) in `fused_through_lds` mode, the
     one kernel in which the matrix cores multiply decoded tiles taken from LDS, beside the two other modes, for M = 16,
@@ -1094,7 +1136,8 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "fused_lds", "encode", "tile_ans_encode"])
+    parser.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["c4", "tile_ans", "gemm", "gemm_phases", "fused_lds", "encode", "tile_ans_encode"])
+    parser.add_argument("--rows", type=int, default=256, help="activation rows of the gemm_phases workload")
     parser.add_argument("--stack-blocks", type=int, default=30, help="blocks of the c4 layer stack (30 = the full 120 layers)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity check")
     parser.add_argument("--no-linear", action="store_true", help="skip the CompressedLinear (config 3) section")
@@ -1118,6 +1161,8 @@ def main():
         return lossless_workload(args, ep)
     if args.workload == "gemm":
         return gemm_workload(args, ep)
+    if args.workload == "gemm_phases":
+        return gemm_phases_workload(args, ep)
     if args.workload == "fused_lds":
         return fused_lds_workload(args, ep)
     if args.workload == "encode":

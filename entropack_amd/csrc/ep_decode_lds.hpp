@@ -926,12 +926,8 @@ __device__ __forceinline__ void decode_lds_body(const DecodeArgs& a, int pair_be
           uint8_t* lower_out = static_cast<uint8_t*>(a.out) + 16ull * lower_tile_of(j);
           // Streaming stores, except for tiles whose length is no multiple of four vectors (store_cached): their groups
           // share 64-byte pieces with the neighbouring groups, and pieces written through the cache meet there.
-#ifdef EP_PROBE_NO_STORE
-          asm volatile("" ::"v"(at), "v"(quad), "s"(lower_out));
-#else
           if (a.store_cached) asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(at), "v"(quad), "s"(lower_out) : "memory");
           else asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(at), "v"(quad), "s"(lower_out) : "memory");
-#endif
         } else if constexpr (KIND == EP_STORE_I8) {
           store_vector_i8(a.out, lower_tile_of(j) + (at >> 4), w);
         } else {

@@ -833,12 +833,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(
 // ---- 128 x 128 tiles with four stages: products of few blocks whose operands come from memory ---------------------------
 //
 // The two-stage 128 x 128 kernel above keeps one K step of loads (32 KB) in flight per block, which covers the L2's latency
-// but not memory's: on a weight that has just been decoded (it is in no cache) 256 x 3072 x 3072 took 46 us where the same
-// product on cached operands took 25 us. When a product has at most one such block per CU there is no second block for
-// the LDS anyway, so this variant spends it on depth: four stages of 32 KB, the tile three steps ahead requested while a
-// step is multiplied (96 KB in flight per block). The wait before the barrier that publishes a stage is counted: the 16
-// loads issued after that stage's own may still be in flight. Everything else (piece permutation, fragment reads a slice
-// ahead, slab epilogue) is the two-stage kernel's.
+// but not memory's. When a product has at most one such block per CU there is no second block for the LDS anyway, so this
+// variant spends it on depth: four stages of 32 KB, the tile three steps ahead requested while a step is multiplied (96 KB
+// in flight per block). The wait before the barrier that publishes a stage is counted: the 16 loads issued after that
+// stage's own may still be in flight. The barrier is a bare s_barrier, and the loop body has no branch: after the fence of
+// __syncthreads(), and after any join of two paths, the compiler's wait-count pass waits for every load into LDS, which
+// empties the pipeline (visible as `s_waitcnt vmcnt(0)` at each step in the code it emits). Everything else (piece
+// permutation, fragment reads a slice ahead, slab epilogue) is the two-stage kernel's.
+// Measured on N = K = 3072 bf16, weight in the last-level cache / weight from memory: M = 256 (48 blocks) 21.6 / 43.0 us
+// with two stages, 18.9 / 31.7 us with four; M = 1024 (192 blocks) 32.0 / 43.1 -> 23.2 / 31.5 us (vendor library 18.8 /
+// 19.2 and 25.6 / 28.7 us). What remains from memory is not depth: a fifth wave that touched the weight rows two groups of
+// steps ahead in 512-byte runs changed nothing, nor did starting each column of blocks at its own K offset. It is the rate at
+// which one CU takes operand bytes, 1.5 MB per block here whatever M is (see the K split below).
 // SPLIT: the grid's z blocks share a tile, each taking gridDim.z-th of K; the sums go, as they are (f32, or int32 for int8), to
 // slab blockIdx.z of `y` ([slice][M][N]) for the kernel that adds the slices, and scales, bias and out_kind are not used.
 template <bool INT8, bool RAGGED, bool SPLIT>
@@ -1036,7 +1042,6 @@ static int launch_direct_small(const void* a, const void* b, const float* scale_
   // At most one block per CU (the deep kernel holds 128 KB of LDS) and K a whole number of four steps, which is what its loop runs.
   int device = 0, cus = 0;
   if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
-#ifndef EP_NO_DEEP_TILES
   if (static_cast<int64_t>(grid.x) * grid.y <= cus && k_bytes % (4 * kTileBytesK) == 0) {
     if (M % 128 == 0 && N % 128 == 0)
       hipLaunchKernelGGL((gemm_deep_kernel<INT8, false, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
@@ -1047,7 +1052,6 @@ static int launch_direct_small(const void* a, const void* b, const float* scale_
     EP_HIP_TRY(hipGetLastError());
     return EP_HIP_OK;
   }
-#endif
   if (M % 128 == 0 && N % 128 == 0)
     hipLaunchKernelGGL((gemm_direct_kernel<INT8, 128, 128, 2, 2, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a),
                        static_cast<const uint8_t*>(b), scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes,
