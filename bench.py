@@ -30,8 +30,8 @@ ROTATING_INPUT_BYTES = 640 << 20
 #: named profile was taken. `csrc_sha16` names those sources; when the kernels have changed since, the figure is not
 #: reported (`traffic` is null and `traffic_source` says why) instead of going stale silently.
 MEASURED_TRAFFIC = {
-    "target": {"bytes": 599_800_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "c15e64bcd7fec39f"},
-    "tile_ans": {"bytes": 819_000_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "0f34596f8f8863b4"},
+    "target": {"bytes": 599_800_000, "profile": "profiles/decode_sym_target_4bpp_hbm_traffic.md", "csrc_sha16": "afaa16960905fbe8"},
+    "tile_ans": {"bytes": 819_000_000, "profile": "profiles/decode_tile_ans_bf16_8192x28672_bench.md", "csrc_sha16": "f3f46eef72554c3a"},
 }
 #: The kernel sources a traffic figure depends on, per workload.
 TRAFFIC_SOURCES = {
