@@ -29,6 +29,7 @@
 #include "ep_decode_lds.hpp"
 
 #include <algorithm>
+#include <exception>
 #include <vector>
 
 namespace ep {
@@ -114,6 +115,19 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
   const uint32_t windows0 = kTables;
   const uint32_t ring0 = windows0 + kFusedWaves * 2 * kRingBytes;
 
+  const ep_hip_fused_batch& batch = batches[blockIdx.x];
+  const int vpr = a.vecs_per_row;
+  const int tv = a.tile_vectors;
+  const int groups = (tv + 31) >> 5;
+  const int rows_total = static_cast<int>(a.num_vectors / vpr);
+  // In-row vector position of the window's first aligned index; windows go down by 32 per step. Checked before anything
+  // is in flight into LDS: a workgroup must not end with loads on their way into memory that is no longer its own.
+  int q0 = __builtin_amdgcn_readfirstlane(static_cast<int>((static_cast<int64_t>(batch.base) + 32 * groups) % vpr));
+  if (q0 < 0 || (q0 & (kStepVectors - 1)) != 0) {        // a batch table that is not ep_hip_fused_plan's: nothing below may index with it
+    if (threadIdx.x == 0) flag_error(a.error, EP_DECODE_BAD_OFFSETS);
+    return;
+  }
+
   // Tables: memory -> LDS without registers in between, left in flight during the set-up below.
   for (uint32_t kib = static_cast<uint32_t>(wave); kib < kTables / 1024u; kib += kFusedWaves) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a.sym_tables + kib * 1024u + static_cast<uint32_t>(lane) * 16u),
@@ -127,12 +141,6 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
   k.ktab = static_cast<uint32_t>(kSymFbStreamBytes);
   k.shv = half ? 16u : 0u;
   asm volatile("" : "+v"(k.f0v), "+v"(k.f1v), "+v"(k.ktab), "+v"(k.shv));
-
-  const ep_hip_fused_batch& batch = batches[blockIdx.x];
-  const int vpr = a.vecs_per_row;
-  const int tv = a.tile_vectors;
-  const int groups = (tv + 31) >> 5;
-  const int rows_total = static_cast<int>(a.num_vectors / vpr);
 
   // ---- this half's tile ------------------------------------------------------------------------------------------
   const int slot = 2 * wave + half;
@@ -214,13 +222,6 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeArgs a, const e
     for (int r = 0; r < 16; ++r) acc[r] = 0;
     row_now -= 1;
   };
-
-  // In-row vector position of the window's first aligned index; windows go down by 32 per step.
-  int q0 = __builtin_amdgcn_readfirstlane(static_cast<int>((static_cast<int64_t>(batch.base) + 32 * groups) % vpr));
-  if (q0 < 0 || (q0 & (kStepVectors - 1)) != 0) {        // a batch table that is not ep_hip_fused_plan's: nothing below may index with it
-    if (threadIdx.x == 0) flag_error(a.error, EP_DECODE_BAD_OFFSETS);
-    return;
-  }
 
   // Positions above the tile's top group (read by the first window) start as zeros.
   ring_store(32 * groups + l32 + delta, fused_u32x4{0, 0, 0, 0});
@@ -473,7 +474,12 @@ extern "C" int ep_hip_fused_plan(int64_t rows, int64_t cols_padded, int tile_ele
   const int64_t vectors = rows * vpr;
   const int64_t tiles = (vectors + tv - 1) / tv;
   if (vpr < 32 || vpr % 4 != 0 || vpr > 0x7FFFFFFF || vectors >= (int64_t{1} << 31) || tiles >= (int64_t{1} << 30)) return EP_HIP_EUNSUPPORTED;
-  std::vector<std::pair<int32_t, int32_t>> order(static_cast<size_t>(tiles));      // (position of the tile's first vector in its row, tile)
+  std::vector<std::pair<int32_t, int32_t>> order;      // (position of the tile's first vector in its row, tile)
+  try {
+    order.resize(static_cast<size_t>(tiles));
+  } catch (const std::exception&) {                   // no exception leaves the C ABI
+    return EP_HIP_EINVAL;
+  }
   for (int64_t t = 0; t < tiles; ++t) order[static_cast<size_t>(t)] = {static_cast<int32_t>((t * tv) % vpr), static_cast<int32_t>(t)};
   std::sort(order.begin(), order.end());
   int count = 0;

@@ -130,6 +130,42 @@ def test_linear_mfma_matches_f_linear_on_the_oracle_weight(rows, cols, bpp, tile
 
 
 @pytest.mark.gpu
+def test_linear_mfma_on_randomly_drawn_containers():
+    """24 containers from a fixed seed: rows 1..700, 32..640 vectors per row (multiples of four), rates 1.5..7 bpp, tile sizes
+    from one group to the default, outlier rows, 1..200 activation rows; every draw against the float64 product on the CPU
+    oracle's weight."""
+    from entropack_amd.schemes.lattice_rans import hip as hip_lane
+    rng = np.random.default_rng(20240611)
+    done = 0
+    while done < 24:
+        rows = int(rng.integers(1, 701))
+        cols = 8 * 4 * int(rng.integers(8, 161))
+        bpp = float(rng.choice([1.5, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0]))
+        tile_elements = [None, 288, 300, 1000, 2304, 4096, 4100, 8192][int(rng.integers(0, 8))]
+        m = int(rng.integers(1, 201))
+        torch.manual_seed(int(rng.integers(0, 1 << 30)))
+        weight = torch.randn(rows, cols) * 0.02
+        if rng.random() < 0.3:
+            weight[int(rng.integers(0, rows))] *= 30.0
+        weight = weight.to(torch.bfloat16)
+        options = {} if tile_elements is None else {"tile_elements": tile_elements}
+        container = ep.compress(weight, ep.EntroPackLossyConfig(target_bpp=bpp, execution_backend="eager", **options))
+        on_gpu = container.to("cuda")
+        buffers = packed_buffers(on_gpu.buffers, LatticeBuffers)
+        x = torch.randn(m, cols).to(torch.bfloat16).cuda()
+        if not hip_lane.mfma_linear_usable(buffers, (rows, cols), x):      # e.g. a rate whose tables are not the two-level form
+            continue
+        print("draw", done, (rows, cols, bpp, tile_elements), "M =", m, flush=True)
+        oracle = _oracle_weight(container)[:, :cols].cuda()
+        bias = (torch.randn(rows) * 0.01).to(torch.bfloat16).cuda() if rng.random() < 0.5 else None
+        y = hip_lane.linear_mfma(buffers, shape=(rows, cols), x=x, bias=bias)
+        torch.cuda.synchronize()
+        hip_lane.check_errors(buffers)
+        _check(y, x, oracle, bias, (rows, cols, bpp, tile_elements, m))
+        done += 1
+
+
+@pytest.mark.gpu
 def test_linear_mfma_flags_a_corrupt_stream_and_refuses_other_tables():
     from entropack_amd.schemes.lattice_rans import hip as hip_lane
     torch.manual_seed(5)
