@@ -199,6 +199,30 @@ def test_compressed_linear_forward_config_3(mode):
     assert 3.9 < layer.compressed_bits < 4.1
 
 
+@pytest.mark.parametrize("m", [256, 1024, 4096])
+def test_fused_mode_with_this_librarys_tiled_product(m, monkeypatch):
+    """`fused.TILED_PRODUCT = "own"`: more than 128 rows are multiplied by this library's kernels (K split over blocks at 256 rows,
+    four-stage 128 x 128 tiles at 1024, 256 x 192 tiles at 4096) and the vendor library is not called."""
+    from entropack_amd.linear import fused as fused_mode
+    print("case own tiled product, M =", m, flush=True)
+    layer, _, bias = _c3_layer("fused")
+    torch.manual_seed(12)
+    x = torch.randn(m, 3072).to(torch.bfloat16).cuda()
+    decoded = layer.dequantize("cuda")
+    expect = F.linear(x.float(), decoded.float(), bias.cuda().float())
+    monkeypatch.setattr(fused_mode, "TILED_PRODUCT", "own")
+
+    def no_library(*args, **kwargs):
+        raise AssertionError("the vendor product was called")
+
+    monkeypatch.setattr(fused_mode.F, "linear", no_library)
+    y = layer(x)
+    monkeypatch.undo()
+    assert y.shape == (m, 3072) and y.dtype == torch.bfloat16
+    assert rel_l2(y, expect) <= REL_L2
+    assert within_one_ulp(y, expect.to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("m", [1, 16, 128])
 def test_compressed_linear_small_m_both_modes_agree(m):
     layer_a, _, bias = _c3_layer("decode_then_gemm", rows=512, cols=2048)
