@@ -248,49 +248,65 @@ __global__ __launch_bounds__(256) void quantize_rows_wave_kernel(const uint16_t*
                                                                  int8_t* __restrict__ codes, float* __restrict__ scales) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
   const int lane = threadIdx.x & 63;
   const int64_t row = blockIdx.x * int64_t{4} + (threadIdx.x >> 6);
   if (row >= rows) return;
   const uint16_t* from = x + row * ldx;
-  auto value = [](uint32_t word, int high) -> float {
-    const uint32_t bits = high ? word >> 16 : word & 0xFFFFu;
+  auto value_of_bits = [](uint32_t bits) -> float {       // bits: a two-byte pattern in the low half
     if constexpr (IN_KIND == kOutBF16) return __uint_as_float(bits << 16);
     else return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
   };
+  auto value = [&](uint32_t word, int high) -> float {
+    if constexpr (IN_KIND == kOutBF16) return __uint_as_float(high ? word & 0xFFFF0000u : word << 16);
+    else return value_of_bits(high ? word >> 16 : word & 0xFFFFu);
+  };
+  // The row's largest magnitude, found on the bit patterns: without its sign bit a bf16 or f16 pattern grows with the
+  // magnitude it stands for (a NaN counts as larger than every number), two elements per instruction.
   u32x4 held[CHUNKS];
-  float top = 0.0f;
+  u16x2 top2 = {0, 0};
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
     const int k = 8 * (64 * c + lane);
     held[c] = u32x4{0u, 0u, 0u, 0u};
     if (k < K) held[c] = *reinterpret_cast<const u32x4*>(from + k);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) top = __builtin_fmaxf(top, __builtin_fabsf(value(held[c][i >> 1], i & 1)));
+    for (int i = 0; i < 4; ++i) top2 = __builtin_elementwise_max(top2, __builtin_bit_cast(u16x2, held[c][i] & 0x7FFF7FFFu));
   }
+  uint32_t top_bits = top2[0] > top2[1] ? top2[0] : top2[1];
 #pragma unroll
-  for (int offset = 32; offset > 0; offset >>= 1) top = __builtin_fmaxf(top, __shfl_xor(top, offset));
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(top_bits), offset));
+    top_bits = other > top_bits ? other : top_bits;
+  }
+  const float top = value_of_bits(top_bits);
   const float scale = __builtin_fmaxf(top / 127.0f, 1.1920928955078125e-07f);
   const float inverse = 1.0f / scale;
+  // code = rint(x / scale), |code| <= 127. Adding 1.5 * 2^23 rounds to the nearest integer, ties to even, as rint does, and
+  // leaves the code as the low byte of the sum's bit pattern. t = x * (1 / scale) is within 2^-14 of the quotient; where it
+  // is no closer than that to a half-integer both round alike, and a chunk with a lane that is closer takes the division.
+  constexpr float kMagic = 12582912.0f;
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
     const int k = 8 * (64 * c + lane);
-    float code[8];
+    float shifted[8];
     float nearest_half = 0.0f;               // the largest |t - rint(t)| of the chunk: 0.5 at a half-integer
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float t = __fmul_rn(value(held[c][i >> 1], i & 1), inverse);
-      code[i] = __builtin_rintf(t);
-      nearest_half = __builtin_fmaxf(nearest_half, __builtin_fabsf(t - code[i]));
+      shifted[i] = __fadd_rn(t, kMagic);
+      nearest_half = __builtin_fmaxf(nearest_half, __builtin_fabsf(__fsub_rn(t, __fsub_rn(shifted[i], kMagic))));
     }
     if (__builtin_amdgcn_ballot_w64(nearest_half > 0.5f - 0.00006103515625f) != 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) code[i] = __builtin_rintf(value(held[c][i >> 1], i & 1) / scale);
+      for (int i = 0; i < 8; ++i) shifted[i] = __fadd_rn(__fdiv_rn(value(held[c][i >> 1], i & 1), scale), kMagic);
     }
-    u32x2 packed = {0u, 0u};
+    u32x2 packed;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int q = static_cast<int>(__builtin_fminf(__builtin_fmaxf(code[i], -127.0f), 127.0f));
-      packed[i >> 2] |= (static_cast<uint32_t>(q) & 0xFFu) << (8 * (i & 3));
+    for (int h = 0; h < 2; ++h) {            // the low bytes of four sums into one word
+      const uint32_t low = __builtin_amdgcn_perm(__float_as_uint(shifted[4 * h + 1]), __float_as_uint(shifted[4 * h]), 0x0C0C0400u);
+      const uint32_t high = __builtin_amdgcn_perm(__float_as_uint(shifted[4 * h + 3]), __float_as_uint(shifted[4 * h + 2]), 0x04000C0Cu);
+      packed[h] = low | high;
     }
     if (k < K) *reinterpret_cast<u32x2*>(codes + row * K + k) = packed;
   }
@@ -1497,15 +1513,20 @@ int ep_hip_quantize_rows(const void* x_dev, int in_kind, int64_t rows, int64_t K
     const uint16_t* x = static_cast<const uint16_t*>(x_dev);
     const int k = static_cast<int>(K), m = static_cast<int>(rows);
 #define EP_QUANTISE_WAVE(KIND, CHUNKS) hipLaunchKernelGGL((quantize_rows_wave_kernel<KIND, CHUNKS>), grid, dim3(256), 0, s, x, ldx, k, m, codes_dev, scales_dev)
+    // A chunk is 512 elements of the row: no more of them than the row has.
+#define EP_QUANTISE_WAVE_KIND(KIND)                      \
+    if (K <= 1024) EP_QUANTISE_WAVE(KIND, 2);            \
+    else if (K <= 2048) EP_QUANTISE_WAVE(KIND, 4);       \
+    else if (K <= 3072) EP_QUANTISE_WAVE(KIND, 6);       \
+    else if (K <= 4096) EP_QUANTISE_WAVE(KIND, 8);       \
+    else if (K <= 6144) EP_QUANTISE_WAVE(KIND, 12);      \
+    else EP_QUANTISE_WAVE(KIND, 16)
     if (in_kind == kOutBF16) {
-      if (K <= 2048) EP_QUANTISE_WAVE(kOutBF16, 4);
-      else if (K <= 4096) EP_QUANTISE_WAVE(kOutBF16, 8);
-      else EP_QUANTISE_WAVE(kOutBF16, 16);
+      EP_QUANTISE_WAVE_KIND(kOutBF16);
     } else {
-      if (K <= 2048) EP_QUANTISE_WAVE(kOutF16, 4);
-      else if (K <= 4096) EP_QUANTISE_WAVE(kOutF16, 8);
-      else EP_QUANTISE_WAVE(kOutF16, 16);
+      EP_QUANTISE_WAVE_KIND(kOutF16);
     }
+#undef EP_QUANTISE_WAVE_KIND
 #undef EP_QUANTISE_WAVE
     EP_HIP_TRY(hipGetLastError());
     return EP_HIP_OK;
