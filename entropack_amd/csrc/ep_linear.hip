@@ -467,8 +467,8 @@ __global__ __launch_bounds__(256) void rotate_quantize_rows_kernel(const void* _
 // stores whole row pieces, 16 bytes per lane. In the slab, rows with bit 2 set keep their columns rotated by 32: the
 // two lane halves of an accumulator register (rows 4 apart) then write to different banks. The arithmetic and the
 // rounding are those of the element-wise path, which ragged products and outputs with unaligned rows take.
-template <bool INT8, bool GUARD, int NJ, typename Acc, bool EDGE = false>    // EDGE: whole row pieces, but the tile may overhang M and N
-__device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, const float* __restrict__ scale_a,
+template <bool INT8, bool GUARD, int NJ, typename Acc, bool EDGE = false, int NI = 2>    // EDGE: whole row pieces, but the tile may overhang M and N; NI: 32-row tiles of the wave (from the argument)
+__device__ __forceinline__ void store_wave_tile(Acc (&acc)[NI][NJ], float* slab, const float* __restrict__ scale_a,
                                                 const float* __restrict__ scale_b, const void* __restrict__ bias,
                                                 void* __restrict__ y, int M, int N, int64_t ldy, int out_kind, int row0, int col0,
                                                 int lane) {
@@ -479,7 +479,7 @@ __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, 
                          (!EDGE || N % (16 / out_bytes) == 0);      // a 16-byte piece is then all inside the row or all outside
   if (wide_rows) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NI; ++i) {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         int n = col0 + j * 32 + (lane & 31);
@@ -542,7 +542,7 @@ __device__ __forceinline__ void store_wave_tile(Acc (&acc)[2][NJ], float* slab, 
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < NI; ++i) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int n = col0 + j * 32 + (lane & 31);
@@ -863,14 +863,17 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(
 // which one CU takes operand bytes, 1.5 MB per block here whatever M is (see the K split below).
 // SPLIT: the grid's z blocks share a tile, each taking gridDim.z-th of K; the sums go, as they are (f32, or int32 for int8), to
 // slab blockIdx.z of `y` ([slice][M][N]) for the kernel that adds the slices, and scales, bias and out_kind are not used.
-template <bool INT8, bool RAGGED, bool SPLIT>
+// TILE = 64: blocks of 64 x 64 (four waves of 32 x 32, four stages of 16 KB) for products whose 128 x 128 tiles would leave most
+// CUs idle.
+template <bool INT8, bool RAGGED, bool SPLIT, int TILE = 128>
 __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                           const float* __restrict__ scale_a, const float* __restrict__ scale_b,
                                                           const void* __restrict__ bias, void* __restrict__ y, int M, int N, int64_t k_bytes,
                                                           int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind) {
-  constexpr int BM = 128, BN = 128, kWaves = 4, WN = 64, NJ = 2;
+  static_assert(TILE == 128 || TILE == 64, "2 x 2 waves of 64 x 64 or 32 x 32");
+  constexpr int BM = TILE, BN = TILE, kWaves = 4, WN = TILE / 2, NJ = WN / 32, NI = NJ;
   constexpr int kRowBytes = kTileBytesK;
-  constexpr int kStage = (BM + BN) * kRowBytes;              // 32 KB
+  constexpr int kStage = (BM + BN) * kRowBytes;              // 32 KB (16 KB)
   __shared__ __align__(1024) uint8_t stage0[kStage];
   __shared__ __align__(1024) uint8_t stage1[kStage];
   __shared__ __align__(1024) uint8_t stage2[kStage];
@@ -878,7 +881,7 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  constexpr int kLoadsA = BM / (8 * kWaves), kLoadsB = BN / (8 * kWaves), kLoads = kLoadsA + kLoadsB;      // 4 + 4 pieces of 1 KiB per wave and tile
+  constexpr int kLoadsA = BM / (8 * kWaves), kLoadsB = BN / (8 * kWaves), kLoads = kLoadsA + kLoadsB;      // 4 + 4 (2 + 2) pieces of 1 KiB per wave and tile
   const int wave_m = wave / 2, wave_n = wave % 2;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int64_t steps = k_bytes / kTileBytesK / (SPLIT ? gridDim.z : 1);           // this block's
@@ -903,22 +906,22 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
 
   using Acc = typename std::conditional<INT8, i32x16, f32x16>::type;
   using Frag = typename std::conditional<INT8, i32x4, bf16x8>::type;
-  Acc acc[2][NJ] = {};
-  constexpr int kReads = 2 + NJ, kMultiplies = 2 * NJ;
+  Acc acc[NI][NJ] = {};
+  constexpr int kReads = NI + NJ, kMultiplies = NI * NJ;
   Frag frag[2][kReads];
   const int frag_row = lane & 31;
   const int turn = (frag_row >> 1) & 7;
-  const uint32_t frag_a_at = static_cast<uint32_t>((wave_m * 64 + frag_row) * kRowBytes);
+  const uint32_t frag_a_at = static_cast<uint32_t>((wave_m * 32 * NI + frag_row) * kRowBytes);
   const uint32_t frag_b_at = static_cast<uint32_t>((BM + wave_n * WN + frag_row) * kRowBytes);
   auto read_one = [&](int set, const uint8_t* stage, int kk, int t) {
     const uint32_t place = static_cast<uint32_t>(((2 * kk + (lane >> 5)) ^ turn) * 16);
-    const uint32_t at = place + (t < 2 ? frag_a_at + t * 32 * kRowBytes : frag_b_at + (t - 2) * 32 * kRowBytes);
+    const uint32_t at = place + (t < NI ? frag_a_at + t * 32 * kRowBytes : frag_b_at + (t - NI) * 32 * kRowBytes);
     frag[set][t] = *reinterpret_cast<const Frag*>(stage + at);
   };
   auto multiply_one = [&](int set, int m) {
     const int i = m / NJ, j = m % NJ;
-    if constexpr (INT8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
-    else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[set][i], frag[set][2 + j], acc[i][j], 0, 0, 0);
+    if constexpr (INT8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[set][i], frag[set][NI + j], acc[i][j], 0, 0, 0);
+    else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[set][i], frag[set][NI + j], acc[i][j], 0, 0, 0);
   };
 
   auto tile_at = [&](int64_t t) { return (t < steps ? t : steps - 1) * kTileBytesK; };
@@ -926,13 +929,15 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
   // three, three and two of its eight pieces per slice. Past the last tile the loads repeat the last one, which nobody reads.
   auto k_step = [&](uint8_t* here, uint8_t* there, uint8_t* fill, int64_t step) {
     const int64_t ahead = tile_at(step + 3);
+    constexpr int kPerSlice = (kLoads + 2) / 3;             // loads a slice issues: 3, 3, 2 of eight; 2, 2, 0 of four
+    constexpr int kSlots = kMultiplies > kReads ? (kMultiplies > kPerSlice ? kMultiplies : kPerSlice) : (kReads > kPerSlice ? kReads : kPerSlice);
 #pragma unroll
     for (int slice = 0; slice < 3; ++slice) {
 #pragma unroll
-      for (int m = 0; m < kMultiplies; ++m) {
-        multiply_one(slice & 1, m);
-        const int piece = 3 * slice + m;
-        if (m < 3 && piece < kLoads) load_one(fill, ahead, piece);
+      for (int m = 0; m < kSlots; ++m) {
+        if (m < kMultiplies) multiply_one(slice & 1, m);
+        const int piece = kPerSlice * slice + m;
+        if (m < kPerSlice && piece < kLoads) load_one(fill, ahead, piece);
         if (m < kReads) read_one((slice & 1) ^ 1, here, slice + 1, m);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -941,11 +946,11 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
     // A bare barrier: the fence of __syncthreads() makes the compiler wait for every load into LDS, which would empty the
     // pipeline at each step. This wave's fragment reads of `here` are complete (lgkmcnt 0) before it arrives, so no wave
     // can overwrite a stage that another still reads.
-    __builtin_amdgcn_s_waitcnt(0x4070);                     // vmcnt(16), lgkmcnt(0)
+    __builtin_amdgcn_s_waitcnt(kLoads == 8 ? 0x4070 : 0x0078);      // vmcnt(2 kLoads), lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int m = 0; m < kMultiplies; ++m) {
-      multiply_one(1, m);
+    for (int m = 0; m < (kMultiplies > kReads ? kMultiplies : kReads); ++m) {
+      if (m < kMultiplies) multiply_one(1, m);
       if (m < kReads) read_one(0, there, 0, m);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -956,7 +961,7 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
   for (int c = 0; c < kLoads; ++c) load_one(stage1, tile_at(1), c);
 #pragma unroll
   for (int c = 0; c < kLoads; ++c) load_one(stage2, tile_at(2), c);
-  __builtin_amdgcn_s_waitcnt(0x4F70);                       // vmcnt(16): the first tile has landed
+  __builtin_amdgcn_s_waitcnt(kLoads == 8 ? 0x4F70 : 0x0F78);       // vmcnt(2 kLoads): the first tile has landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int t = 0; t < kReads; ++t) read_one(0, stage0, 0, t);
@@ -974,13 +979,13 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
     using Cell = typename std::conditional<INT8, int32_t, float>::type;
     Cell* out = static_cast<Cell*>(y) + static_cast<int64_t>(blockIdx.z) * M * N;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NI; ++i) {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const int n = n0 + wave_n * WN + j * 32 + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wave_m * 64 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+          const int m = m0 + wave_m * 32 * NI + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
           if (!RAGGED || (m < M && n < N)) out[static_cast<int64_t>(m) * N + n] = acc[i][j][r];
         }
       }
@@ -988,7 +993,7 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
   } else {
     static_assert(4 * 32 * WN * 4 <= kStage, "four slabs fit into one stage");
     float* slab = reinterpret_cast<float*>(stage0) + wave * (32 * WN);
-    store_wave_tile<INT8, false, NJ, Acc, RAGGED>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 64, n0 + wave_n * WN, lane);
+    store_wave_tile<INT8, false, NJ, Acc, RAGGED>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 32 * NI, n0 + wave_n * WN, lane);
   }
 }
 
@@ -1051,6 +1056,15 @@ static bool small_tiles_in_one_round(int64_t M, int64_t N, int64_t k_bytes) {
   return small_whole_tiles<INT8>(M, N, k_bytes) && ((M + 127) / 128) * ((N + 127) / 128) <= kSmallTileSlots;
 }
 
+// Products whose 128 x 128 tiles would occupy at most half the CUs while 64 x 64 tiles still fit them in one round: what
+// bounds such a product is the rate at which one CU takes operand bytes (see the K split further down), and a 64 x 64 block
+// takes half of a 128 x 128 block's. 256 x 3072 x 3072 bf16, weight cached / from memory: 48 blocks of 128 x 128 18.9 / 31.7 us,
+// the same split four ways over K 20.1 / 20.6 us (two kernels), 192 blocks of 64 x 64 see the figures in the commit that added them.
+static bool few_tiles_take_small_blocks(int64_t M, int64_t N, int64_t k_bytes, int cus) {
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+  return 2 * tiles128 <= cus && tiles64 <= cus && k_bytes % (4 * kTileBytesK) == 0 && k_bytes >= 8 * kTileBytesK;
+}
+
 template <bool INT8>
 static int launch_direct_small(const void* a, const void* b, const float* scale_a, const float* scale_b, const void* bias, void* y, int64_t M,
                                int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
@@ -1058,6 +1072,17 @@ static int launch_direct_small(const void* a, const void* b, const float* scale_
   // At most one block per CU (the deep kernel holds 128 KB of LDS) and K a whole number of four steps, which is what its loop runs.
   int device = 0, cus = 0;
   if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
+  if (few_tiles_take_small_blocks(M, N, k_bytes, cus)) {
+    const dim3 small(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>((M + 63) / 64));
+    if (M % 64 == 0 && N % 64 == 0)
+      hipLaunchKernelGGL((gemm_deep_kernel<INT8, false, false, 64>), small, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                         scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
+    else
+      hipLaunchKernelGGL((gemm_deep_kernel<INT8, true, false, 64>), small, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                         scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
+    EP_HIP_TRY(hipGetLastError());
+    return EP_HIP_OK;
+  }
   if (static_cast<int64_t>(grid.x) * grid.y <= cus && k_bytes % (4 * kTileBytesK) == 0) {
     if (M % 128 == 0 && N % 128 == 0)
       hipLaunchKernelGGL((gemm_deep_kernel<INT8, false, false>), grid, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
@@ -1328,6 +1353,9 @@ static int launch_skinny(const void* x, const void* w, const float* scale_a, con
 // of the bytes, and the kernel that adds the skinny product's slices adds these.
 static int split_slices(int64_t M, int64_t N, int64_t k_bytes, int cus) {
   if (M <= 128 || k_bytes % kTileBytesK != 0) return 0;
+#ifndef EP_SPLIT_BEFORE_SMALL_BLOCKS
+  if (few_tiles_take_small_blocks(M, N, k_bytes, cus)) return 0;       // one kernel of 64 x 64 blocks does better than two
+#endif
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   const int64_t steps = k_bytes / kTileBytesK;
   int64_t most = cus / tiles;

@@ -315,25 +315,30 @@ def test_skinny_gemm_workspace_matches_its_split():
 def test_split_gemm_workspace_is_zero_unless_the_tiles_leave_half_the_cus_idle():
     """More than 128 rows: 128 x 128 tiles with K divided over the largest number of blocks per tile (at most 8, at most the
     CUs over the tiles) that leaves each a whole number of four 128-byte steps and at least eight; 0 where no such split
-    exists, which is how a caller learns that the product takes the unsplit kernels."""
+    exists, and 0 where 64 x 64 blocks fit the CUs in one round (one kernel then does better than two), which is how a
+    caller learns that the product takes the unsplit kernels."""
     size = hip_backend.library().ep_hip_gemm_skinny_workspace
 
     def expect(m, n, k_bytes, cus):
         if k_bytes % 128:
             return 0
         tiles, steps = -(-m // 128) * -(-n // 128), k_bytes // 128
+        small = -(-m // 64) * -(-n // 64)
+        if 2 * tiles <= cus and small <= cus and steps % 4 == 0 and steps >= 8:
+            return 0
         for slices in range(min(cus // tiles, 8), 1, -1):
             if steps % (4 * slices) == 0 and steps // slices >= 8:
                 return slices * m * n * 4
         return 0
 
-    assert size(256, 3072, 6144, 256) == 4 * 256 * 3072 * 4                    # 48 tiles, 48 steps: 5 does not divide, 4 does
-    assert size(256, 3072, 3072, 256) == 3 * 256 * 3072 * 4                    # int8 rows of the same layer: 24 steps
+    assert size(384, 3072, 6144, 256) == 3 * 384 * 3072 * 4                    # 72 tiles, 48 steps: three slices of 16
+    assert size(384, 3072, 2048, 256) == 2 * 384 * 3072 * 4                    # 16 steps: two slices of 8
+    assert size(256, 3072, 6144, 256) == 0                                     # 192 blocks of 64 x 64 fit the CUs
     assert size(1024, 3072, 6144, 256) == 0                                    # 192 tiles: nothing to gain
-    assert size(256, 3072, 6144 + 16, 256) == 0                                # K not of whole steps
-    assert size(256, 3072, 512, 256) == 0                                      # four steps: too short to split
+    assert size(384, 3072, 6144 + 16, 256) == 0                                # K not of whole steps
+    assert size(384, 3072, 512, 256) == 0                                      # four steps: too short to split
     for case in [(200, 3000, 4096, 256), (300, 1000, 2048, 256), (640, 3072, 6144, 256), (129, 128, 1 << 16, 256), (256, 3072, 6144, 64),
-                 (384, 640, 8192, 304)]:
+                 (384, 640, 8192, 304), (520, 2000, 4096, 256), (129, 4000, 2048, 256)]:
         assert size(*case) == expect(*case), case
 
 

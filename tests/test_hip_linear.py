@@ -39,7 +39,8 @@ def within_one_ulp(got, rounded):
                                    (300, 1000, 1024), (130, 136, 64), (1000, 3000, 320), (300, 1001, 128),   # overhanging ones
                                    (3000, 3100, 192),                                           # overhanging 256 x 192 tiles
                                    (256, 3072, 3072), (1024, 3072, 1024), (640, 3072, 256),    # one 128 x 128 tile per CU at most and
-                                   (200, 3000, 2048)])                                          # K of 4n steps: the four-stage kernel
+                                   (200, 3000, 2048),                                           # K of 4n steps: the four-stage kernel
+                                   (384, 3072, 1024), (520, 2000, 2048), (129, 4000, 1024)])    # ... with K split over blocks
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
     print("case", shape, with_bias, flush=True)
@@ -149,7 +150,8 @@ def test_quantize_rows_is_exact_next_to_rounding_boundaries():
                                    (33, 257, 16), (4096, 3000, 272), (4096, 4096, 896), (4096, 3072, 128), (4096, 3072, 384),
                                    (768, 3072, 640), (3072, 3000, 272), (256, 128, 128), (384, 640, 384), (1024, 3072, 640),
                                    (300, 1000, 1024), (130, 129, 128), (3000, 3100, 256),
-                                   (256, 3072, 3072), (1024, 3072, 512), (200, 3000, 4096)])    # the four-stage kernel, whole and ragged
+                                   (256, 3072, 3072), (1024, 3072, 512), (200, 3000, 4096),     # the four-stage kernel, whole and ragged
+                                   (384, 3072, 2048), (520, 2000, 4096)])                        # ... with K split over blocks
 def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
     print("case", shape, flush=True)
     m, n, k = shape
