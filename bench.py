@@ -183,11 +183,12 @@ def linear_section(ep, steps):
     out = {"workload": "CompressedLinear 3072x3072 @ 4.0 bpp + bias, X [4096, 3072] bf16, seed 2", "flops": flops}
     from entropack_amd.linear import fused as fused_mode
     reference = None
-    # `fused_own_gemm` = the fused mode made to multiply with this library's tiled kernel instead of the vendor library's
-    # (fused.TILED_PRODUCT = "own"); the mode's default is the faster of the two on a freshly decoded weight.
+    # `fused` multiplies with the mode's default (fused.TILED_PRODUCT = "auto": this library's kernel where it runs blocks of
+    # 64 x 64, e.g. 256 rows of this layer, the vendor library's otherwise); `fused_own_gemm` = the mode made to multiply with
+    # this library's tiled kernels whatever the shape ("own").
     # `fused_through_lds` = the one kernel in which the matrix cores multiply decoded tiles taken from LDS (the dense weight is
     # never written); selected by name only, because it is the slower one.
-    variants = (("decode_then_gemm", "decode_then_gemm", "library"), ("fused", "fused", "library"), ("fused_own_gemm", "fused", "own"),
+    variants = (("decode_then_gemm", "decode_then_gemm", "library"), ("fused", "fused", "auto"), ("fused_own_gemm", "fused", "own"),
                 ("fused_through_lds", "fused_through_lds", "library"))
     for name, mode, product in variants:
         layer = ep.CompressedLinear.from_linear(dense, config=ep.EntroPackLossyConfig(target_bpp=4.0), forward_mode=mode).cuda()
@@ -214,7 +215,7 @@ def linear_section(ep, steps):
             entry[name] = {"ms": round(_median_ms(lambda: layer(part), steps), 5),
                            "rel_l2_vs_f32_reference": ((got - reference[:rows]).norm() / reference[:rows].norm()).item()}
         out["fewer_rows"][f"M={rows}"] = entry
-    fused_mode.TILED_PRODUCT = "library"
+    fused_mode.TILED_PRODUCT = "auto"
     # The same layer encoded with tiles a quarter and an eighth of the default size (`tile_elements`, a field of the
     # reference's config): a tile's chain of dependent steps, which is all a single layer's decode waits for, shortens
     # in proportion, for a per-tile header that costs 1-3 % more stored bits.
@@ -380,7 +381,7 @@ def stack_linear_section(ep, steps, layers_total=48, distinct=4):
             ahead.check_errors()
         out["decode_ahead_group_16_in_line_own_gemm"] = entry
     finally:
-        fused_mode.TILED_PRODUCT = "library"
+        fused_mode.TILED_PRODUCT = "auto"
         for layer in layers:
             layer.forward_mode = "decode_then_gemm"
     return out

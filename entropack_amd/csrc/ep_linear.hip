@@ -864,16 +864,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void gemm_direct_kernel(
 // SPLIT: the grid's z blocks share a tile, each taking gridDim.z-th of K; the sums go, as they are (f32, or int32 for int8), to
 // slab blockIdx.z of `y` ([slice][M][N]) for the kernel that adds the slices, and scales, bias and out_kind are not used.
 // TILE = 64: blocks of 64 x 64 (four waves of 32 x 32, four stages of 16 KB) for products whose 128 x 128 tiles would leave most
-// CUs idle.
+// CUs idle. TILE = 96: blocks of 128 x 96 (four waves of 32 x 96 one above the other, four stages of 28 KB) for products whose
+// 128 x 128 tiles leave some CUs idle: a block then takes 224 instead of 256 operand rows.
 template <bool INT8, bool RAGGED, bool SPLIT, int TILE = 128>
 __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                           const float* __restrict__ scale_a, const float* __restrict__ scale_b,
                                                           const void* __restrict__ bias, void* __restrict__ y, int M, int N, int64_t k_bytes,
                                                           int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind) {
-  static_assert(TILE == 128 || TILE == 64, "2 x 2 waves of 64 x 64 or 32 x 32");
-  constexpr int BM = TILE, BN = TILE, kWaves = 4, WN = TILE / 2, NJ = WN / 32, NI = NJ;
+  static_assert(TILE == 128 || TILE == 64 || TILE == 96, "2 x 2 waves of 64 x 64 or 32 x 32, or 4 x 1 waves of 32 x 96");
+  constexpr int BM = TILE == 64 ? 64 : 128, BN = TILE, kWaves = 4, kWavesN = TILE == 96 ? 1 : 2, kWavesM = kWaves / kWavesN;
+  constexpr int WN = BN / kWavesN, NJ = WN / 32, NI = BM / (32 * kWavesM);
   constexpr int kRowBytes = kTileBytesK;
-  constexpr int kStage = (BM + BN) * kRowBytes;              // 32 KB (16 KB)
+  constexpr int kStage = (BM + BN) * kRowBytes;              // 32 KB (16 KB, 28 KB)
   __shared__ __align__(1024) uint8_t stage0[kStage];
   __shared__ __align__(1024) uint8_t stage1[kStage];
   __shared__ __align__(1024) uint8_t stage2[kStage];
@@ -882,7 +884,7 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int kLoadsA = BM / (8 * kWaves), kLoadsB = BN / (8 * kWaves), kLoads = kLoadsA + kLoadsB;      // 4 + 4 (2 + 2) pieces of 1 KiB per wave and tile
-  const int wave_m = wave / 2, wave_n = wave % 2;
+  const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int64_t steps = k_bytes / kTileBytesK / (SPLIT ? gridDim.z : 1);           // this block's
   const int64_t k_first = SPLIT ? blockIdx.z * steps * kTileBytesK : 0;
@@ -946,7 +948,8 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
     // A bare barrier: the fence of __syncthreads() makes the compiler wait for every load into LDS, which would empty the
     // pipeline at each step. This wave's fragment reads of `here` are complete (lgkmcnt 0) before it arrives, so no wave
     // can overwrite a stage that another still reads.
-    __builtin_amdgcn_s_waitcnt(kLoads == 8 ? 0x4070 : 0x0078);      // vmcnt(2 kLoads), lgkmcnt(0)
+    constexpr int kInFlight = 2 * kLoads;                   // s_waitcnt: vmcnt in bits 0-3 and 14-15, expcnt (not waited for) 4-6, lgkmcnt 8-11
+    __builtin_amdgcn_s_waitcnt((kInFlight & 15) | ((kInFlight >> 4) << 14) | 0x0070);      // vmcnt(2 kLoads), lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int m = 0; m < (kMultiplies > kReads ? kMultiplies : kReads); ++m) {
@@ -961,7 +964,7 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
   for (int c = 0; c < kLoads; ++c) load_one(stage1, tile_at(1), c);
 #pragma unroll
   for (int c = 0; c < kLoads; ++c) load_one(stage2, tile_at(2), c);
-  __builtin_amdgcn_s_waitcnt(kLoads == 8 ? 0x4F70 : 0x0F78);       // vmcnt(2 kLoads): the first tile has landed
+  __builtin_amdgcn_s_waitcnt(((2 * kLoads) & 15) | (((2 * kLoads) >> 4) << 14) | 0x0F70);       // vmcnt(2 kLoads): the first tile has landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int t = 0; t < kReads; ++t) read_one(0, stage0, 0, t);
@@ -991,8 +994,9 @@ __global__ __launch_bounds__(256, 1) void gemm_deep_kernel(const uint8_t* __rest
       }
     }
   } else {
-    static_assert(4 * 32 * WN * 4 <= kStage, "four slabs fit into one stage");
-    float* slab = reinterpret_cast<float*>(stage0) + wave * (32 * WN);
+    static_assert(TILE == 96 ? 32 * WN * 4 <= kStage : 4 * 32 * WN * 4 <= kStage, "the waves' slabs fit into one stage, or one stage each");
+    float* slab = TILE == 96 ? reinterpret_cast<float*>(wave == 0 ? stage0 : (wave == 1 ? stage1 : (wave == 2 ? stage2 : stage3)))
+                             : reinterpret_cast<float*>(stage0) + wave * (32 * WN);
     store_wave_tile<INT8, false, NJ, Acc, RAGGED>(acc, slab, scale_a, scale_b, bias, y, M, N, ldy, out_kind, m0 + wave_m * 32 * NI, n0 + wave_n * WN, lane);
   }
 }
@@ -1059,7 +1063,7 @@ static bool small_tiles_in_one_round(int64_t M, int64_t N, int64_t k_bytes) {
 // Products whose 128 x 128 tiles would occupy at most half the CUs while 64 x 64 tiles still fit them in one round: what
 // bounds such a product is the rate at which one CU takes operand bytes (see the K split further down), and a 64 x 64 block
 // takes half of a 128 x 128 block's. 256 x 3072 x 3072 bf16, weight cached / from memory: 48 blocks of 128 x 128 18.9 / 31.7 us,
-// the same split four ways over K 20.1 / 20.6 us (two kernels), 192 blocks of 64 x 64 see the figures in the commit that added them.
+// the same split four ways over K 20.1 / 20.6 us (two kernels), 192 blocks of 64 x 64 16.7 / 16.9 us (the vendor library 19.0 / 19.4).
 static bool few_tiles_take_small_blocks(int64_t M, int64_t N, int64_t k_bytes, int cus) {
   const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
   return 2 * tiles128 <= cus && tiles64 <= cus && k_bytes % (4 * kTileBytesK) == 0 && k_bytes >= 8 * kTileBytesK;
@@ -1079,6 +1083,19 @@ static int launch_direct_small(const void* a, const void* b, const float* scale_
                          scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
     else
       hipLaunchKernelGGL((gemm_deep_kernel<INT8, true, false, 64>), small, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                         scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
+    EP_HIP_TRY(hipGetLastError());
+    return EP_HIP_OK;
+  }
+  // One round of blocks either way: 128 x 96 blocks are more, and each takes fewer operand bytes (1024 x 3072 x 3072 bf16, weight
+  // cached / from memory: 23.4 / 31.8 us with 192 blocks of 128 x 128, 23.1 / 28.4 us with 256 of 128 x 96; vendor 26.2 / 29.5).
+  if (static_cast<int64_t>(grid.x) * grid.y <= cus && ((N + 95) / 96) * static_cast<int64_t>(grid.y) <= cus && k_bytes % (4 * kTileBytesK) == 0) {
+    const dim3 narrow(static_cast<unsigned>((N + 95) / 96), grid.y);
+    if (M % 128 == 0 && N % 96 == 0)
+      hipLaunchKernelGGL((gemm_deep_kernel<INT8, false, false, 96>), narrow, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                         scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
+    else
+      hipLaunchKernelGGL((gemm_deep_kernel<INT8, true, false, 96>), narrow, dim3(256), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
                          scale_a, scale_b, bias, y, static_cast<int>(M), static_cast<int>(N), k_bytes, lda_bytes, ldb_bytes, ldy, out_kind);
     EP_HIP_TRY(hipGetLastError());
     return EP_HIP_OK;
@@ -1353,9 +1370,7 @@ static int launch_skinny(const void* x, const void* w, const float* scale_a, con
 // of the bytes, and the kernel that adds the skinny product's slices adds these.
 static int split_slices(int64_t M, int64_t N, int64_t k_bytes, int cus) {
   if (M <= 128 || k_bytes % kTileBytesK != 0) return 0;
-#ifndef EP_SPLIT_BEFORE_SMALL_BLOCKS
   if (few_tiles_take_small_blocks(M, N, k_bytes, cus)) return 0;       // one kernel of 64 x 64 blocks does better than two
-#endif
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   const int64_t steps = k_bytes / kTileBytesK;
   int64_t most = cus / tiles;
@@ -1451,6 +1466,11 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
                      static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), ldx, ldw, ldy, out_kind);
   EP_HIP_TRY(hipGetLastError());
   return EP_HIP_OK;
+}
+
+int ep_hip_gemm_takes_small_blocks(int64_t M, int64_t N, int64_t k_bytes, int compute_units) {
+  if (M <= 0 || N <= 0 || k_bytes <= 0 || compute_units <= 0) return 0;
+  return ep::small_tiles_in_one_round<false>(M, N, k_bytes) && ep::few_tiles_take_small_blocks(M, N, k_bytes, compute_units) ? 1 : 0;
 }
 
 size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units) {

@@ -10,9 +10,10 @@
   throughput)
   up to 128         yes, once                   decode, then this package's split-K skinny product (`ep_hip_gemm_bf16_skinny`),
                                                 which streams the weight at 75 % of the memory bandwidth
-  more              yes, once                   decode, then a tiled product on the matrix cores: the vendor library's
-                                                (`TILED_PRODUCT = "library"`, the default) or this package's
-                                                (`"own"`, `ep_hip_gemm_bf16`)
+  more              yes, once                   decode, then a tiled product on the matrix cores: this package's
+                                                (`ep_hip_gemm_bf16`) where it runs blocks of 64 x 64, the vendor library's
+                                                otherwise (`TILED_PRODUCT = "auto"`, the default; `"own"` and `"library"`
+                                                force one of them)
 
 "fused_through_lds": any M, weight never written. One kernel (`ep_hip_linear_fused_mfma_bf16`) in which every workgroup
 decodes 32 tiles whose chains stay aligned in k, passes each group of decoded vectors through an LDS ring and multiplies
@@ -27,10 +28,12 @@ from L2 at M = 4096 where the GEMM needs 0.7 GB); gathering 32 aligned tiles on 
 SIMD, which lengthens each chain step from 138 to 219 ns; and for M > 256 the same tiles are decoded once per block of
 256 activation rows. It stays in the package as the built and measured form of the idea, selected only by name.
 
-The default for the tiled product is the library because its kernel is the faster one wherever the weight has just been
-decoded, i.e. is not in any cache: 3072 x 3072 weight, 256 / 1024 / 4096 rows: 20 / 31 / 63 us against 46 / 46 / 67 us for
-this package's kernel, which keeps less than one K step of loads in flight (with both operands cache-resident the two
-are within 5 % of each other at 4096 rows). The reference has one path for every M: decode, then `F.linear`
+Which tiled product, measured on an MI355X with the weight coming from memory, as a weight that has just been decoded
+does (3072 x 3072 weight, this package's kernels / the vendor library's): 256 rows 16.9 / 19.4 us, 1024 rows 28.4 / 29.5 us,
+4096 rows 67.3 / 63.2 us. A product of few tiles is bounded by the rate at which one compute unit takes operand bytes, and
+this package's kernel for it (blocks of 64 x 64, four stages of loads in flight) is the faster one on every layer shape
+tried (13-35 %); from there on the two are within 10 % of each other, one ahead here and the other there, and the
+default leaves those to the library. The reference has one path for every M: decode, then `F.linear`
 (entropack/linear/linear.py:163-165).
 
 The forward is differentiable with respect to the activations (like the reference's `F.linear` on a constant weight):
@@ -45,8 +48,9 @@ from ..schemes.lattice_rans import hip as hip_lane
 from ..schemes.lattice_rans.format import LatticeBuffers
 from . import kernels
 
-#: Which tiled GEMM multiplies more than `kernels.SKINNY_MAX_ROWS` activation rows in fused mode: "library" or "own".
-TILED_PRODUCT = "library"
+#: Which tiled GEMM multiplies more than `kernels.SKINNY_MAX_ROWS` activation rows in fused mode: "auto" (this package's where
+#: it runs its blocks of 64 x 64, else the library's), "library" or "own".
+TILED_PRODUCT = "auto"
 
 
 def _forward_kernels(layer, x: torch.Tensor) -> torch.Tensor:
@@ -62,8 +66,9 @@ def _forward_kernels(layer, x: torch.Tensor) -> torch.Tensor:
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("the fused forward runs in bfloat16; use forward_mode='decode_then_gemm' for other dtypes")
     rows = x.numel() // x.shape[-1] if x.shape[-1] else 0
-    if rows > kernels.SKINNY_MAX_ROWS and TILED_PRODUCT == "library":
-        return F.linear(x, weight, layer._bias_on(x.device))
+    if rows > kernels.SKINNY_MAX_ROWS and TILED_PRODUCT != "own":
+        if TILED_PRODUCT == "library" or not kernels.takes_small_blocks(rows, weight.shape[0], x.shape[-1] * 2, x.device):
+            return F.linear(x, weight, layer._bias_on(x.device))
     return kernels.gemm_bf16(x, weight, layer._bias_on(x.device), out_dtype=x.dtype)
 
 

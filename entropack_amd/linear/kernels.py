@@ -28,6 +28,13 @@ def _rows(tensor: torch.Tensor) -> torch.Tensor:
     return flat if flat.stride(-1) == 1 and flat.data_ptr() % 16 == 0 and flat.stride(0) % 16 == 0 else flat.contiguous()
 
 
+def takes_small_blocks(rows: int, outer: int, row_bytes: int, device: torch.device) -> bool:
+    """Whether this package's tiled product runs `rows` x `outer` with rows of `row_bytes` bytes of K in blocks of 64 x 64: the
+    products on which it is ahead of the vendor library's (host-side rule of the C library)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return bool(_hip.library().ep_hip_gemm_takes_small_blocks(rows, outer, row_bytes, _hip.device_info(index).compute_units))
+
+
 def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """x[..., K] @ weight[N, K].T (+ bias): bf16 operands, f32 accumulation on the matrix cores."""
     device = _require_device(x, weight)

@@ -211,6 +211,14 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
  * of CompressedLinear.forward and the int8 GEMM of CompressedINT8Linear at small batch, entropack/linear/linear.py:163-165,
  * 485-490. */
 size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units);
+
+/* 1 when ep_hip_gemm_bf16 / ep_hip_gemm_i8 multiply this product with blocks of 64 x 64: its 128 x 128 tiles would occupy at
+ * most half of `compute_units`, its 64 x 64 tiles fit them in one round, and a row of K (`k_bytes` bytes) is a whole number of
+ * four 128-byte steps, at least eight. These are the products on which this library's kernel is ahead of the vendor
+ * library's on an MI355X (256 x 3072 x 3072 bf16: 16.9 us against 19.4 us with the weight coming from memory), which is what
+ * a caller that has both may want to know; 0 otherwise. Host only. No counterpart in the reference (it has one product,
+ * F.linear, entropack/linear/linear.py:163-165). */
+int ep_hip_gemm_takes_small_blocks(int64_t M, int64_t N, int64_t k_bytes, int compute_units);
 int ep_hip_gemm_bf16_skinny(const void* x_dev, const void* w_dev, const void* bias_dev, void* y_dev, int64_t M, int64_t N,
                             int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int out_kind, int compute_units,
                             void* workspace_dev, size_t workspace_bytes, void* stream);

@@ -40,7 +40,8 @@ def within_one_ulp(got, rounded):
                                    (3000, 3100, 192),                                           # overhanging 256 x 192 tiles
                                    (256, 3072, 3072), (1024, 3072, 1024), (640, 3072, 256),    # one 128 x 128 tile per CU at most and
                                    (200, 3000, 2048),                                           # K of 4n steps: the four-stage kernel
-                                   (384, 3072, 1024), (520, 2000, 2048), (129, 4000, 1024)])    # ... with K split over blocks
+                                   (384, 3072, 1024), (520, 2000, 2048), (129, 4000, 1024),     # ... with K split over blocks
+                                   (900, 2900, 1024), (640, 3072, 2048)])                        # ... with 128 x 96 blocks
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
     print("case", shape, with_bias, flush=True)
@@ -151,7 +152,8 @@ def test_quantize_rows_is_exact_next_to_rounding_boundaries():
                                    (768, 3072, 640), (3072, 3000, 272), (256, 128, 128), (384, 640, 384), (1024, 3072, 640),
                                    (300, 1000, 1024), (130, 129, 128), (3000, 3100, 256),
                                    (256, 3072, 3072), (1024, 3072, 512), (200, 3000, 4096),     # the four-stage kernel, whole and ragged
-                                   (384, 3072, 2048), (520, 2000, 4096)])                        # ... with K split over blocks
+                                   (384, 3072, 2048), (520, 2000, 4096),                         # ... with K split over blocks
+                                   (900, 2900, 2048)])                                           # ... with 128 x 96 blocks
 def test_int8_gemm_is_exact_in_f32_and_rounds_once(shape):
     print("case", shape, flush=True)
     m, n, k = shape
@@ -203,8 +205,9 @@ def test_compressed_linear_forward_config_3(mode):
 
 @pytest.mark.parametrize("m", [256, 1024, 4096])
 def test_fused_mode_with_this_librarys_tiled_product(m, monkeypatch):
-    """`fused.TILED_PRODUCT = "own"`: more than 128 rows are multiplied by this library's kernels (K split over blocks at 256 rows,
-    four-stage 128 x 128 tiles at 1024, 256 x 192 tiles at 4096) and the vendor library is not called."""
+    """`fused.TILED_PRODUCT = "own"`: more than 128 rows are multiplied by this library's kernels (blocks of 64 x 64 at 256 rows,
+    of 128 x 96 at 1024, of 256 x 192 at 4096) and the vendor library is not called. The default, "auto", does the same at 256
+    rows and calls the library at 4096."""
     from entropack_amd.linear import fused as fused_mode
     print("case own tiled product, M =", m, flush=True)
     layer, _, bias = _c3_layer("fused")
@@ -219,6 +222,12 @@ def test_fused_mode_with_this_librarys_tiled_product(m, monkeypatch):
 
     monkeypatch.setattr(fused_mode.F, "linear", no_library)
     y = layer(x)
+    monkeypatch.setattr(fused_mode, "TILED_PRODUCT", "auto")
+    if m == 256:
+        assert torch.equal(layer(x), y)
+    elif m == 4096:
+        with pytest.raises(AssertionError, match="vendor product"):
+            layer(x)
     monkeypatch.undo()
     assert y.shape == (m, 3072) and y.dtype == torch.bfloat16
     assert rel_l2(y, expect) <= REL_L2
