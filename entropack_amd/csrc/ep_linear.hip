@@ -1043,27 +1043,25 @@ static int launch_big(const void* a, const void* b, const float* scale_a, const 
                   : launch_big_variant<INT8, true, BN>(a, b, scale_a, scale_b, bias, y, M, N, k_bytes, lda_bytes, ldb_bytes, ldy, out_kind, stream);
 }
 
-// Products of whole 128 x 128 tiles: the direct-load kernel with four waves of 64 x 64 per block and two blocks per CU
-// (64 KB of LDS each). While all blocks are resident at once (at most 512 on the 256 CUs of an MI355X) this is the
-// fastest of the tiled kernels here: 256 x 3072 x 3072 bf16 24 us (the single-stage 128 x 128 kernel below 52 us, the
-// vendor library 25 us), 1024 x 3072 x 3072 35 us (256 x 192 tiles 49 us), 2560 x 3072 x 3072, 480 blocks, 51 us (57 us).
-// With more blocks than that a second round starts and the 256-row tiles win: 3072 x 3072 x 3072 80 us against 62 us.
-constexpr int64_t kSmallTileSlots = 512;
-
+// Products of whole 128 x 128 tiles: the direct-load kernels with four waves per block. The two-stage kernel runs two blocks
+// per CU (64 KB of LDS each): 2560 x 3072 x 3072 bf16, 480 blocks in one round, 51 us (256 x 192 tiles 57 us); with more
+// blocks than two per CU a second round starts and the 256-row tiles win: 3072 x 3072 x 3072 80 us against 62 us
+// (whole_k_tiling below weighs the rounds). Products of at most one block per CU take the four-stage kernels.
 template <bool INT8>
 static bool small_whole_tiles(int64_t M, int64_t N, int64_t k_bytes) {       // whole in K; M and N may overhang
   return k_bytes % kTileBytesK == 0 && (M + 127) / 128 <= 65535;
-}
-
-template <bool INT8>
-static bool small_tiles_in_one_round(int64_t M, int64_t N, int64_t k_bytes) {
-  return small_whole_tiles<INT8>(M, N, k_bytes) && ((M + 127) / 128) * ((N + 127) / 128) <= kSmallTileSlots;
 }
 
 // Products whose 128 x 128 tiles would occupy at most half the CUs while 64 x 64 tiles still fit them in one round: what
 // bounds such a product is the rate at which one CU takes operand bytes (see the K split further down), and a 64 x 64 block
 // takes half of a 128 x 128 block's. 256 x 3072 x 3072 bf16, weight cached / from memory: 48 blocks of 128 x 128 18.9 / 31.7 us,
 // the same split four ways over K 20.1 / 20.6 us (two kernels), 192 blocks of 64 x 64 16.7 / 16.9 us (the vendor library 19.0 / 19.4).
+static int current_compute_units() {
+  int device = 0, cus = 0;
+  if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
+  return cus;
+}
+
 static bool few_tiles_take_small_blocks(int64_t M, int64_t N, int64_t k_bytes, int cus) {
   const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
   return 2 * tiles128 <= cus && tiles64 <= cus && k_bytes % (4 * kTileBytesK) == 0 && k_bytes >= 8 * kTileBytesK;
@@ -1074,8 +1072,7 @@ static int launch_direct_small(const void* a, const void* b, const float* scale_
                                int64_t N, int64_t k_bytes, int64_t lda_bytes, int64_t ldb_bytes, int64_t ldy, int out_kind, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>((N + 127) / 128), static_cast<unsigned>((M + 127) / 128));
   // At most one block per CU (the deep kernel holds 128 KB of LDS) and K a whole number of four steps, which is what its loop runs.
-  int device = 0, cus = 0;
-  if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) cus = 0;
+  const int cus = current_compute_units();
   if (few_tiles_take_small_blocks(M, N, k_bytes, cus)) {
     const dim3 small(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>((M + 63) / 64));
     if (M % 64 == 0 && N % 64 == 0)
@@ -1122,20 +1119,36 @@ static int launch_direct_small(const void* a, const void* b, const float* scale_
   return EP_HIP_OK;
 }
 
-// Which block tile a product takes: 256 x 256 once there is one for every CU (256 on MI355X); else 256 x 192 if that
-// shape gives enough CUs a tile; else the 128 x 128 kernels, which spread small products over more CUs (products of
-// whole 128 x 128 tiles that fit the machine in one round never get here, see above). "Enough" is 48
-// for products of whole tiles, which take the direct-load kernel (768 x 3072 x 3072, 48 tiles: 49 us against 56 us;
-// 3072 x 3072 x 3072, 192 tiles: 62 us against 105 us; with fewer tiles and a long K the smaller blocks win again:
-// 256 x 8192 x 28672, 43 tiles, 546 us against 496 us), and 150 for ragged ones, which take the register-staged kernel
-// (3072 x 3000 x 3072: 84 us against 102 us, but 512 x 3000 x 3072: 72 us against 55 us). Returns the tile's column
-// count, 0 for the 128 x 128 kernel.
+// Which block tile a product with K of whole tile steps takes: the family whose rounds of blocks add up to the least time.
+// A round is one set of blocks resident together (one 256-row block per CU, two two-stage 128 x 128 blocks, one four-stage
+// block), and a round costs a fixed part plus a time per K step that was measured once per kernel on an MI355X (bf16,
+// N = K = 3072 and 8192; the int8 kernels move the same bytes per step and keep the ratios): 256 x 256 1.55 us, 256 x 192
+// 1.16 us, two-stage 128 x 128 0.83 us for its two blocks, the four-stage kernels 0.42 us. What the count of rounds decides
+// is the tail: 1536 x 8192 x 8192 is 258 blocks of 256 x 192, two rounds for the sake of two blocks (262 us), and one round of
+// 192 blocks of 256 x 256. Returns 256 or 192 for the 256-row tiles, 0 for the 128-row family (launch_direct_small).
+static int whole_k_tiling(int64_t M, int64_t N, int64_t k_bytes, int cus) {
+  if (cus <= 0) cus = 256;
+  const double steps = static_cast<double>(k_bytes / kTileBytesK);
+  constexpr double kRoundFixed = 4.0;
+  auto rounds = [&](int64_t bm, int64_t bn, int64_t slots) { return static_cast<double>((((M + bm - 1) / bm) * ((N + bn - 1) / bn) + slots - 1) / slots); };
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const double small = tiles128 <= cus ? kRoundFixed + 0.42 * steps : rounds(128, 128, 2 * static_cast<int64_t>(cus)) * (kRoundFixed + 0.83 * steps);
+  const double wide = (M + 255) / 256 <= 65535 ? rounds(256, 192, cus) * (kRoundFixed + 1.16 * steps) : 1e30;
+  const double square = (M + 255) / 256 <= 65535 ? rounds(256, 256, cus) * (kRoundFixed + 1.55 * steps) : 1e30;
+  if (small <= wide && small <= square) return 0;
+  return square < wide ? 256 : 192;
+}
+
+// The same choice for products whose K is not of whole tile steps (the register-staged 256-row kernel or the single-stage
+// 128 x 128 kernel): 256 x 256 once there is one for every CU (256 on MI355X); else 256 x 192 from 150 tiles on (3072 x 3000
+// x 3072: 84 us against 102 us, but 512 x 3000 x 3072: 72 us against 55 us). Returns the tile's column count, 0 for the
+// 128 x 128 kernel.
 static int big_tile_columns(int64_t M, int64_t N, int64_t k_bytes) {
   if (M < kBigM) return 0;
   const int64_t rows = (M + kBigM - 1) / kBigM;
   if (N >= 256 && rows * ((N + 255) / 256) >= 256) return 256;
-  const bool whole = k_bytes % kTileBytesK == 0;            // the direct-load kernel takes it, overhanging tiles included
-  if (N >= 192 && rows * ((N + 191) / 192) >= (whole ? 48 : 150)) return 192;
+  (void)k_bytes;
+  if (N >= 192 && rows * ((N + 191) / 192) >= 150) return 192;
   return 0;
 }
 
@@ -1450,9 +1463,8 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
   if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldx < K || ldw < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(w_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  if (small_tiles_in_one_round<false>(M, N, K * 2))
-    return launch_direct_small<false>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, static_cast<hipStream_t>(stream));
-  if (const int columns = big_tile_columns(M, N, K * 2)) {
+  const int columns = small_whole_tiles<false>(M, N, K * 2) ? whole_k_tiling(M, N, K * 2, current_compute_units()) : big_tile_columns(M, N, K * 2);
+  if (columns != 0) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return columns == 256 ? launch_big<false, 256>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s)
                           : launch_big<false, 192>(x_dev, w_dev, nullptr, nullptr, bias_dev, y_dev, M, N, K * 2, ldx * 2, ldw * 2, ldy, out_kind, s);
@@ -1470,7 +1482,7 @@ int ep_hip_gemm_bf16(const void* x_dev, const void* w_dev, const void* bias_dev,
 
 int ep_hip_gemm_takes_small_blocks(int64_t M, int64_t N, int64_t k_bytes, int compute_units) {
   if (M <= 0 || N <= 0 || k_bytes <= 0 || compute_units <= 0) return 0;
-  return ep::small_tiles_in_one_round<false>(M, N, k_bytes) && ep::few_tiles_take_small_blocks(M, N, k_bytes, compute_units) ? 1 : 0;
+  return ep::small_whole_tiles<false>(M, N, k_bytes) && ep::few_tiles_take_small_blocks(M, N, k_bytes, compute_units) ? 1 : 0;
 }
 
 size_t ep_hip_gemm_skinny_workspace(int64_t M, int64_t N, int64_t k_bytes, int compute_units) {
@@ -1530,9 +1542,7 @@ int ep_hip_gemm_i8(const int8_t* a_dev, const int8_t* b_dev, const float* scale_
   if (K % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0 || lda < K || ldb < K || ldy < N) return EP_HIP_EINVAL;
   if (reinterpret_cast<uintptr_t>(a_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(b_dev) % 16 != 0) return EP_HIP_EINVAL;
   if (!out_kind_valid(out_kind)) return EP_HIP_EINVAL;
-  if (small_tiles_in_one_round<true>(M, N, K))
-    return launch_direct_small<true>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, static_cast<hipStream_t>(stream));
-  if (const int columns = big_tile_columns(M, N, K)) {
+  if (const int columns = small_whole_tiles<true>(M, N, K) ? whole_k_tiling(M, N, K, current_compute_units()) : big_tile_columns(M, N, K)) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return columns == 256 ? launch_big<true, 256>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s)
                           : launch_big<true, 192>(a_dev, b_dev, scale_a_dev, scale_b_dev, bias_dev, y_dev, M, N, K, lda, ldb, ldy, out_kind, s);
