@@ -70,6 +70,36 @@ def test_gemm_bf16_matches_fp32_matmul(shape, with_bias):
     assert torch.equal(as_f16, kernels.gemm_bf16(x, w, half_bias, out_dtype=torch.float32).to(torch.float16))
 
 
+def test_gemm_on_randomly_drawn_shapes_of_every_tile_family():
+    """60 bf16 and 40 int8 products from a fixed seed, drawn so that every kernel family and the boundaries between them come up
+    (few tiles, one round of 128-row blocks, several rounds, 256-row tiles, K of whole and of ragged tile steps, overhanging M
+    and N): bf16 within one ulp of the f32 product rounded once, int8 exact."""
+    rng = np.random.default_rng(77)
+    for draw in range(100):
+        int8 = draw >= 60
+        m = int(rng.choice([rng.integers(129, 700), rng.integers(700, 2600), rng.integers(2600, 5000), 128 * rng.integers(2, 33)]))
+        n = int(rng.choice([rng.integers(8, 700), rng.integers(700, 4200), 64 * rng.integers(1, 60), 96 * rng.integers(1, 40)]))
+        step = 128 if int8 else 64
+        k = int(rng.choice([step * rng.integers(1, 40), 4 * step * rng.integers(1, 12), (16 if int8 else 8) * rng.integers(1, 300)]))
+        print("draw", draw, "int8" if int8 else "bf16", (m, n, k), flush=True)
+        torch.manual_seed(draw)
+        if int8:
+            a = torch.randint(-127, 128, (m, k), device="cuda", dtype=torch.int8)
+            b = torch.randint(-127, 128, (n, k), device="cuda", dtype=torch.int8)
+            sa = torch.rand(m, device="cuda") * 0.05 + 1e-3
+            sb = torch.rand(n, device="cuda") * 0.01 + 1e-4
+            exact = a.double() @ b.double().T
+            expect = exact.float() * sa.unsqueeze(1) * sb.unsqueeze(0)
+            assert torch.equal(kernels.int8_gemm(a, b, sa, sb, None, torch.float32), expect), (m, n, k)
+        else:
+            x = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+            w = (torch.randn(n, k, device="cuda") * 0.02).to(torch.bfloat16)
+            got = kernels.gemm_bf16(x, w, None)
+            expect = x.float() @ w.float().T
+            assert within_one_ulp(got, expect.to(torch.bfloat16)), (m, n, k)
+            assert rel_l2(kernels.gemm_bf16(x, w, None, out_dtype=torch.float32), expect) <= 1e-5, (m, n, k)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_gemm_output_rows_that_are_not_16_byte_aligned(out_dtype):
     """The 256-row kernel stores whole row pieces of 16 bytes when the output allows it; an output whose rows do not
